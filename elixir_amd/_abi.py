@@ -1,0 +1,131 @@
+"""ctypes binding of ``libelx_hip.so`` (declared in ``include/elx_abi.h``).
+
+There is no CPU fallback: if the library has not been built, or a launch fails, the caller gets
+an exception.  Tables are built on the host as numpy structured arrays whose layouts mirror the
+C structs (the sizes are checked against the loaded library).
+"""
+import ctypes
+import os
+from typing import Optional
+
+import numpy as np
+
+ELX_ABI_VERSION = 1
+ELX_F32, ELX_F16, ELX_BF16, ELX_NONE = 0, 1, 2, -1
+ELX_FLAG_SCALAR_ONLY = 1
+ELX_HYPER_L2 = 1
+ELX_HYPER_LERP_FROM_G = 2
+
+CHUNK_DTYPE = np.dtype([('grad', '<u8'), ('lowp_out', '<u8'), ('master', '<u8'), ('m', '<u8'), ('v', '<u8'),
+                        ('n_alloc', '<u8'), ('n_valid', '<u8'), ('tile_begin', '<u8'), ('seg_begin', '<u4'),
+                        ('seg_end', '<u4')])
+SEG_DTYPE = np.dtype([('begin', '<u8'), ('end', '<u8'), ('hyper', '<u4'), ('reserved', '<u4')])
+HYPER_DTYPE = np.dtype([('decay_mul', '<f4'), ('l2_wd', '<f4'), ('lerp_w', '<f4'), ('beta2', '<f4'), ('omb2', '<f4'),
+                        ('bc2_sqrt', '<f4'), ('eps', '<f4'), ('neg_step', '<f4'), ('flags', '<u4'),
+                        ('reserved', '<u4', (3,))])
+STATS_DTYPE = np.dtype([('sumsq', '<f8'), ('overflow', '<u4'), ('reserved', '<u4')])
+
+LIB_NAME = 'libelx_hip.so'
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+
+EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg',
+           'elx_sizeof_hyper', 'elx_sizeof_stats', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
+           'elx_writeback_mt')
+
+
+class ElxError(RuntimeError):
+    """A call into libelx_hip.so returned a non-zero code."""
+
+    def __init__(self, func: str, code: int, text: str):
+        super().__init__(f'{func} failed with code {code}: {text}')
+        self.func = func
+        self.code = code
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raise loudly when it is missing or does not match this binding."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f'{LIB_PATH} is missing: the HIP extension has not been built. '
+                           f'Run `python -m elixir_amd.build` (needs hipcc); there is no CPU fallback.')
+    L = ctypes.CDLL(LIB_PATH)
+    u32, u64, vp, cint, flt = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    L.elx_version.restype = cint
+    L.elx_version.argtypes = []
+    L.elx_strerror.restype = ctypes.c_char_p
+    L.elx_strerror.argtypes = [cint]
+    for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats'):
+        getattr(L, name).restype = u32
+        getattr(L, name).argtypes = []
+    L.elx_check_tables.restype = cint
+    L.elx_check_tables.argtypes = [vp, u32, vp, u32, u32, cint, cint, ctypes.POINTER(u64), ctypes.POINTER(cint)]
+    L.elx_grad_stats_mt.restype = cint
+    L.elx_grad_stats_mt.argtypes = [vp, u32, cint, u32, vp, vp, cint, vp]
+    L.elx_adam_step_mt.restype = cint
+    L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, flt, cint, cint, u32, u32, vp]
+    L.elx_writeback_mt.restype = cint
+    L.elx_writeback_mt.argtypes = [vp, u32, u64, cint, u32, u32, vp]
+
+    if L.elx_version() != ELX_ABI_VERSION:
+        raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
+    for name, dt in (('chunk', CHUNK_DTYPE), ('seg', SEG_DTYPE), ('hyper', HYPER_DTYPE), ('stats', STATS_DTYPE)):
+        size = getattr(L, f'elx_sizeof_{name}')()
+        if size != dt.itemsize:
+            raise RuntimeError(f'{LIB_PATH}: sizeof {name} record is {size}, binding expects {dt.itemsize}')
+    _lib = L
+    return L
+
+
+def check(func: str, code: int) -> None:
+    if code != 0:
+        raise ElxError(func, code, load().elx_strerror(code).decode())
+
+
+def tile_elems() -> int:
+    return int(load().elx_tile_elems())
+
+
+def _np_ptr(a: Optional[np.ndarray]):
+    if a is None or a.size == 0:
+        return None
+    assert a.flags['C_CONTIGUOUS']
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, grad_dtype: int, lowp_dtype: int):
+    """Validate host tables; returns (total_tiles, all_aligned16)."""
+    assert chunks.dtype == CHUNK_DTYPE
+    n_segs = 0 if segs is None else len(segs)
+    if n_segs:
+        assert segs.dtype == SEG_DTYPE
+    tiles = ctypes.c_uint64(0)
+    aligned = ctypes.c_int(0)
+    code = load().elx_check_tables(_np_ptr(chunks), len(chunks), _np_ptr(segs), n_segs, n_hypers, grad_dtype, lowp_dtype,
+                                   ctypes.byref(tiles), ctypes.byref(aligned))
+    check('elx_check_tables', code)
+    return int(tiles.value), bool(aligned.value)
+
+
+def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_partials: int, d_stats: int,
+                  scalar_only: bool, stream: int) -> None:
+    check('elx_grad_stats_mt',
+          load().elx_grad_stats_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, d_stats,
+                                   int(scalar_only), stream))
+
+
+def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int, total_tiles: int,
+                 div_scale: float, grad_dtype: int, lowp_dtype: int, flags: int, max_blocks: int, stream: int) -> None:
+    check('elx_adam_step_mt',
+          load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, total_tiles, div_scale,
+                                  grad_dtype, lowp_dtype, flags, max_blocks, stream))
+
+
+def writeback_mt(d_chunks: int, n_chunks: int, total_tiles: int, lowp_dtype: int, flags: int, max_blocks: int,
+                 stream: int) -> None:
+    check('elx_writeback_mt', load().elx_writeback_mt(d_chunks, n_chunks, total_tiles, lowp_dtype, flags, max_blocks,
+                                                      stream))

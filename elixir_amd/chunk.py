@@ -1,0 +1,415 @@
+"""Flat chunk storage: the one-process subset of the reference's chunk runtime that the optimizer
+step reads and writes (``elixir/chunk/core/chunk.py``, ``group.py``).
+
+A chunk stores a sequence of tensors back to back in one 1-D buffer.  Parameters live in a pair of
+chunks with identical offsets: a low-precision chunk whose permanent ``shard`` doubles as the
+gradient buffer at step time, and an fp32 chunk that holds the master weights
+(``elixir/wrapper/module.py:104-133``).  On one process ``shard_size == chunk_size`` and
+``shard_begin == 0``.
+
+What is kept: the layout fields and rules (``append_tensor``, ``close_chunk``, ``valid_end``,
+``tensors_info``, ``init_pair``), the reduction flags (``overflow``, ``l2_norm``,
+``update_extra_reduce_info``) and ``optim_update``.  The flags and the low-precision refresh run on
+the HIP kernels.  What is not here: the replicated-cache blocks, gather / scatter / reduce-scatter
+and the tensor state machine of the forward/backward pass.
+"""
+import math
+from dataclasses import dataclass
+from enum import Enum
+from typing import Dict, List, Optional
+
+import numpy as np
+import torch
+
+from . import _abi
+
+
+class ChunkFullError(Exception):
+    pass
+
+
+class TensorState(Enum):
+    FREE = 0
+    COMPUTE = 1
+    HOLD = 2
+    HOLD_AFTER_BWD = 3
+    READY_FOR_REDUCE = 4
+
+
+@dataclass
+class TensorInfo:
+    state: TensorState
+    fake_data: Optional[torch.Tensor]
+    offset: int
+    end: int
+
+
+def gpu_device() -> torch.device:
+    return torch.device('cuda', torch.cuda.current_device())
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return {torch.float32: _abi.ELX_F32, torch.float16: _abi.ELX_F16, torch.bfloat16: _abi.ELX_BF16}[dtype]
+    except KeyError:
+        raise TypeError(f'chunks hold float32, float16 or bfloat16, not {dtype}') from None
+
+
+class DeviceTable:
+    """A numpy structured array and its copy in device memory."""
+
+    def __init__(self, host: np.ndarray, device: torch.device):
+        self.host = host
+        self.dev = torch.from_numpy(host.view(np.uint8).reshape(-1).copy()).to(device)
+
+    @property
+    def ptr(self) -> int:
+        return self.dev.data_ptr()
+
+    def __len__(self):
+        return len(self.host)
+
+
+def stats_launch_blocks(n_valid_max: int) -> int:
+    """Workgroups per chunk for the stats pass: enough to fill 256 compute units several times
+    over for large chunks, one per 16 Ki elements for small ones."""
+    return int(max(1, min(1024, math.ceil(n_valid_max / 16384))))
+
+
+def run_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.device, table: Optional[DeviceTable] = None,
+                   workspace: Optional[Dict] = None) -> np.ndarray:
+    """Launches the stats pass for the chunks described by ``chunk_rows`` (host table, only grad /
+    n_alloc / n_valid are read) and returns the per-chunk ElxStats records on the host.  One
+    blocking device-to-host copy of 16 bytes per chunk."""
+    n = len(chunk_rows)
+    if table is None:
+        table = DeviceTable(chunk_rows, device)
+    bpc = stats_launch_blocks(int(chunk_rows['n_valid'].max()))
+    aligned = bool(np.all(chunk_rows['grad'] % 16 == 0))
+    if workspace is None:
+        workspace = {}
+    need = (n * bpc + n) * _abi.STATS_DTYPE.itemsize
+    buf = workspace.get('stats')
+    if buf is None or buf.numel() < need or buf.device != device:
+        buf = torch.empty(need, dtype=torch.uint8, device=device)
+        workspace['stats'] = buf
+    d_partials = buf.data_ptr()
+    d_stats = d_partials + n * bpc * _abi.STATS_DTYPE.itemsize
+    stream = torch.cuda.current_stream(device).cuda_stream
+    _abi.grad_stats_mt(table.ptr, n, grad_dtype, bpc, d_partials, d_stats, not aligned, stream)
+    out = buf[n * bpc * _abi.STATS_DTYPE.itemsize:need].cpu().numpy()
+    return out.view(_abi.STATS_DTYPE).copy()
+
+
+def l2_norm_from_sumsq(sumsq: float) -> float:
+    """chunk.py:218-221 -- the reference takes the norm as an fp32 scalar and squares it in a
+    Python float: ``valid.float().norm(2).item() ** 2``."""
+    return float(np.float32(math.sqrt(sumsq)))**2
+
+
+class Chunk:
+    """A continuous memory block that stores a sequence of tensors (chunk.py:27-139).
+
+    args:
+        rcache: unused here (the replicated cache belongs to the forward/backward pass)
+        chunk_size: number of elements
+        chunk_dtype: element type
+        process_group: must be None or a group of size 1
+        temp_device: device of the temporary full chunk that exists while tensors are appended
+        shard_device: device of the permanent shard (default: the current GPU, CPU without one)
+    """
+    total_count = 0
+
+    def __init__(self,
+                 rcache=None,
+                 chunk_size: int = 0,
+                 chunk_dtype: torch.dtype = torch.float,
+                 process_group=None,
+                 temp_device: Optional[torch.device] = None,
+                 shard_device: Optional[torch.device] = None,
+                 rcache_fused: bool = False,
+                 cpu_pin_memory: bool = False) -> None:
+        self.chunk_id: int = Chunk.total_count
+        Chunk.total_count += 1
+        self.rcache = rcache
+
+        self.chunk_size: int = chunk_size
+        self.chunk_dtype: torch.dtype = chunk_dtype
+        self.utilized_size: int = 0
+
+        self.torch_pg = process_group
+        self.pg_size: int = 1
+        self.pg_rank: int = 0
+        if process_group is not None:
+            import torch.distributed as dist
+            if dist.get_world_size(process_group) != 1:
+                raise NotImplementedError('this build keeps whole chunks on one GPU (process group of size 1)')
+        assert chunk_size % self.pg_size == 0
+
+        self.shard_size: int = chunk_size // self.pg_size
+        self.shard_begin: int = self.shard_size * self.pg_rank
+        self.shard_end: int = self.shard_begin + self.shard_size
+        self.valid_end: int = self.shard_size + 1    # set to an illegal number
+
+        self.rcb = None
+        self.rcache_fused: bool = rcache_fused
+        self.is_replica: bool = True
+
+        default_device = gpu_device() if torch.cuda.is_available() else torch.device('cpu')
+        temp_device = torch.device(temp_device) if temp_device is not None else default_device
+        shard_device = torch.device(shard_device) if shard_device is not None else default_device
+        # keep all elements to zero: the padding of every shard starts as zero
+        self.chunk_temp: Optional[torch.Tensor] = None
+        self._temp_device = temp_device
+        self._meta_only = False
+        pin_flag = cpu_pin_memory and shard_device.type == 'cpu'
+        self.shard: torch.Tensor = torch.empty(self.shard_size, dtype=chunk_dtype, device=shard_device,
+                                               pin_memory=pin_flag)
+        self._is_init = True
+
+        self.tensors_info: Dict[torch.Tensor, TensorInfo] = {}
+        self.num_tensors: int = 0
+        self.tensor_state_cnter: Dict[TensorState, int] = {state: 0 for state in TensorState}
+
+        self.paired_chunk: Optional['Chunk'] = None
+        # if this chunk is synchronized with the optimizer, the flag is True
+        self.optim_sync_flag = True
+        # whether to record l2 norm for the gradient clipping calculation
+        self.l2_norm_flag = False
+        self.l2_norm: Optional[float] = None
+        # whether it overflows after the reduction
+        self.overflow = False
+        # True once overflow / l2_norm describe the gradients that sit in the shard now
+        self._stats_fresh = False
+        self._workspace: Dict = {}
+
+    # ------------------------------------------------------------------ properties
+
+    @property
+    def is_init(self) -> bool:
+        return self._is_init
+
+    @property
+    def shard_device(self) -> torch.device:
+        return self.shard.device
+
+    @property
+    def payload(self) -> torch.Tensor:
+        if self.is_init and self.chunk_temp is not None:
+            return self.chunk_temp
+        return self.shard
+
+    @property
+    def n_valid(self) -> int:
+        """Number of shard elements that hold tensor data: ``shard[:valid_end]`` (chunk.py:352)."""
+        return min(self.valid_end, self.shard_size)
+
+    @property
+    def memory_usage(self) -> Dict[str, int]:
+        memo = self.shard_size * self.shard.element_size()
+        cuda = memo if self.shard_device.type == 'cuda' else 0
+        cpu = memo if self.shard_device.type == 'cpu' else 0
+        if self.chunk_temp is not None:
+            t = self.chunk_size * self.chunk_temp.element_size()
+            if self.chunk_temp.device.type == 'cuda':
+                cuda += t
+            else:
+                cpu += t
+        return dict(cuda=cuda, cpu=cpu)
+
+    # ------------------------------------------------------------------ building
+
+    def append_tensor(self, tensor: torch.Tensor):
+        """chunk.py:223-247.  Tensors are packed back to back with no alignment padding.  A tensor
+        on the ``meta`` device only reserves its range (its values are produced in place later)."""
+        assert self.is_init
+        assert tensor.dtype == self.chunk_dtype
+
+        new_utilized_size = self.utilized_size + tensor.numel()
+        if new_utilized_size > self.chunk_size:
+            raise ChunkFullError
+
+        if tensor.device.type != 'meta':
+            if self.chunk_temp is None:
+                assert not self._meta_only, 'a chunk holds either real or meta tensors'
+                self.chunk_temp = torch.zeros(self.chunk_size, dtype=self.chunk_dtype, device=self._temp_device)
+            self.chunk_temp[self.utilized_size:new_utilized_size].copy_(tensor.data.flatten())
+            tensor.data = self.chunk_temp[self.utilized_size:new_utilized_size].view(tensor.shape)
+        else:
+            assert self.chunk_temp is None, 'a chunk holds either real or meta tensors'
+            self._meta_only = True
+
+        self.num_tensors += 1
+        tensor_state = TensorState.HOLD
+        self.tensor_state_cnter[tensor_state] += 1
+        self.tensors_info[tensor] = TensorInfo(state=tensor_state, fake_data=None, offset=self.utilized_size,
+                                               end=new_utilized_size)
+        self.utilized_size = new_utilized_size
+
+    def close_chunk(self):
+        """chunk.py:249-262: fix ``valid_end`` and move the data into the permanent shard."""
+        assert self.is_init
+
+        if self.utilized_size <= self.shard_begin:
+            self.valid_end = 0
+        elif self.utilized_size < self.shard_end:
+            self.valid_end = self.utilized_size - self.shard_begin
+
+        if self.chunk_temp is not None:
+            for tensor, info in self.tensors_info.items():
+                tensor.data = torch.empty(0, dtype=tensor.dtype, device=tensor.device)
+            self.shard.copy_(self.chunk_temp[self.shard_begin:self.shard_end])
+        else:
+            self.shard.zero_()
+        self.is_replica = False
+        self.chunk_temp = None
+        self._is_init = False
+
+    def init_pair(self, friend_chunk: 'Chunk') -> None:
+        if self.paired_chunk is None and friend_chunk.paired_chunk is None:
+            self.paired_chunk = friend_chunk
+            friend_chunk.paired_chunk = self
+        else:
+            assert self.paired_chunk is friend_chunk
+            assert friend_chunk.paired_chunk is self
+
+    def get_tensors(self) -> List[torch.Tensor]:
+        return list(self.tensors_info.keys())
+
+    # ------------------------------------------------------------------ gradient landing and flags
+
+    def _stats_row(self) -> np.ndarray:
+        row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+        row['grad'] = self.shard.data_ptr()
+        row['n_alloc'] = self.shard_size
+        row['n_valid'] = self.n_valid
+        return row
+
+    def set_overflow_flag(self, valid_tensor: Optional[torch.Tensor] = None) -> None:
+        """chunk.py:214-216; here both flags come from one pass over ``shard[:valid_end]``."""
+        assert not self.overflow
+        self._compute_stats()
+
+    def set_l2_norm(self, valid_tensor: Optional[torch.Tensor] = None) -> None:
+        assert self.l2_norm is None, 'you are calculating the l2 norm twice'
+        self._compute_stats()
+
+    def _compute_stats(self) -> None:
+        if self.shard_device.type != 'cuda':
+            raise RuntimeError('gradient flags are computed by the HIP kernels: the shard must be on the GPU')
+        stats = run_grad_stats(self._stats_row(), dtype_code(self.chunk_dtype), self.shard_device,
+                               workspace=self._workspace)
+        self._apply_stats(bool(stats['overflow'][0]), float(stats['sumsq'][0]))
+
+    def _apply_stats(self, overflow: bool, sumsq: float) -> None:
+        self.overflow = overflow
+        if self.l2_norm_flag:
+            self.l2_norm = l2_norm_from_sumsq(sumsq)
+        self._stats_fresh = True
+
+    def update_extra_reduce_info(self, block=None):
+        """chunk.py:345-356: flags over the valid head of the reduced gradients.  On one process
+        those are the first ``valid_end`` elements of the shard."""
+        assert not self.overflow
+        assert self.l2_norm is None, 'you are calculating the l2 norm twice'
+        self._compute_stats()
+
+    def reduce_chunk(self, payload: torch.Tensor, always_fp32: bool = False, sync: bool = True) -> None:
+        """The tail of chunk.py:282-315 / 358-377 for a process group of size 1: the gradients that
+        backward accumulated in ``payload`` (``chunk_size`` elements) overwrite the shard; with
+        ``sync`` the flags are computed right away, otherwise the optimizer computes them for all
+        chunks in one launch at the top of the step."""
+        assert not self.is_init
+        assert payload.numel() == self.chunk_size
+        self.shard.copy_(payload[self.shard_begin:self.shard_end])
+        self._stats_fresh = False
+        if sync:
+            self.update_extra_reduce_info()
+
+    # ------------------------------------------------------------------ low-precision refresh
+
+    def optim_update(self) -> None:
+        """Update the low-precision chunk from its fp32 chunk (chunk.py:403-421)."""
+        assert self.paired_chunk is not None
+        friend_chunk: Chunk = self.paired_chunk
+        assert not friend_chunk.is_replica
+        # gradient and optimizer should be on the same device
+        assert self.shard_device.type == friend_chunk.shard_device.type
+
+        if self.shard_device.type == 'cuda':
+            row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+            row['lowp_out'] = self.shard.data_ptr()
+            row['master'] = friend_chunk.shard.data_ptr()
+            # m and v are not touched by the refresh; the table check wants non-NULL pointers
+            row['m'] = friend_chunk.shard.data_ptr()
+            row['v'] = friend_chunk.shard.data_ptr()
+            row['n_alloc'] = self.shard_size
+            row['n_valid'] = self.n_valid
+            code = dtype_code(self.chunk_dtype)
+            tiles, aligned = _abi.check_tables(row, None, 0, code, code)
+            table = DeviceTable(row, self.shard_device)
+            stream = torch.cuda.current_stream(self.shard_device).cuda_stream
+            _abi.writeback_mt(table.ptr, 1, tiles, code, 0 if aligned else _abi.ELX_FLAG_SCALAR_ONLY, 0, stream)
+            # keep the table alive until the launch has consumed it
+            self._workspace['wb_table'] = table
+            self.optim_sync_flag = True
+        elif self.shard_device.type == 'cpu':
+            # the refresh is deferred to the next gather of this chunk
+            self.optim_sync_flag = False
+        else:
+            raise NotImplementedError
+
+    # ------------------------------------------------------------------ misc
+
+    def __hash__(self) -> int:
+        return self.chunk_id
+
+    def __lt__(self, other: object) -> bool:
+        return self.chunk_id < other.chunk_id
+
+    def __eq__(self, other: object) -> bool:
+        return isinstance(other, Chunk) and self.chunk_id == other.chunk_id
+
+    def __repr__(self):
+        state = 'initialization' if self.is_init else 'scattered'
+        return (f'Chunk {self.chunk_id}: state -> {state}, length: {self.chunk_size}, dtype: {self.chunk_dtype}, '
+                f'tensors: {self.num_tensors}, utilized size: {self.utilized_size}, valid_end: {self.valid_end}, '
+                f'shard device: {self.shard_device}')
+
+
+class ChunkGroup:
+    """Bookkeeping of a set of chunks (group.py:12-98): which chunk holds which tensor."""
+
+    def __init__(self, rcache=None) -> None:
+        self.rcache = rcache
+        self.fused_chunks: set = set()
+        self.float_chunks: set = set()
+        self.ten_to_chunk: Dict[torch.Tensor, Chunk] = dict()
+
+    def open_chunk(self, chunk_size: int, chunk_dtype: torch.dtype, process_group=None,
+                   chunk_config: Optional[Dict] = None) -> Chunk:
+        if chunk_config is None:
+            chunk_config = {}
+        return Chunk(rcache=self.rcache, chunk_size=chunk_size, chunk_dtype=chunk_dtype, process_group=process_group,
+                     **chunk_config)
+
+    def close_chunk(self, chunk: Chunk) -> bool:
+        chunk.close_chunk()
+        if chunk.rcache_fused:
+            self.fused_chunks.add(chunk)
+        else:
+            self.float_chunks.add(chunk)
+        for t in chunk.get_tensors():
+            assert t not in self.ten_to_chunk
+            self.ten_to_chunk[t] = chunk
+        return True
+
+    def inside_check(self, chunk: Chunk) -> None:
+        if chunk.rcache_fused:
+            assert chunk in self.fused_chunks
+        else:
+            assert chunk in self.float_chunks
+
+    @property
+    def all_chunks(self) -> List[Chunk]:
+        return sorted(self.fused_chunks.union(self.float_chunks))

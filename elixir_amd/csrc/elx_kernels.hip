@@ -1,0 +1,597 @@
+// Optimizer-step kernels for gfx950 (MI355X) behind the C ABI of include/elx_abi.h.
+//
+// All three passes are streaming, HBM-bound element-wise work; there is no contraction, so no
+// MFMA.  What matters is: 128-bit accesses that a wavefront issues fully coalesced, enough
+// independent loads in flight per lane, no re-reads, and one launch for the whole chunk list.
+//
+//   grad_stats_kernel   one read of the low-precision gradients -> overflow flag + sum of squares
+//                       per chunk (fp32 per-lane partials over 32-128 elements, flushed into an
+//                       fp64 accumulator; wave shuffle -> LDS -> one partial per workgroup;
+//                       a second tiny launch folds the partials in a fixed order)
+//   adam_step_kernel    unscale + Adam/AdamW on master/m/v + low-precision writeback, tile by tile
+//
+// Arithmetic contract (what the parity tests pin): fp32 throughout, IEEE division and square
+// root, the only fused multiply-adds are the three written as fmaf(); compile with
+// -ffp-contract=off.  The op order is torch.optim.Adam's single-tensor path
+// (torch/optim/adam.py:414-419, 457, 476, 528-545) with the fused forms its CPU kernels use.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "elx_abi.h"
+
+namespace {
+
+constexpr int kThreads = 256;                               // 4 wavefronts of 64
+constexpr int kVec = 4;                                     // elements per lane per access
+constexpr int kUnroll = 4;                                  // independent accesses per lane per stream
+constexpr uint32_t kSpan = kThreads * kVec;                 // elements one access of the workgroup covers
+constexpr uint32_t kTile = kSpan * kUnroll;                 // 4096 elements per tile
+constexpr uint32_t kMaxStatsBlocks = 1024;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
+
+// ---------------------------------------------------------------------------------------------
+// element codecs
+// ---------------------------------------------------------------------------------------------
+
+template <int D>
+struct Elem;
+
+template <>
+struct Elem<ELX_F32> {
+    typedef float scalar;
+    typedef f32x4 vec4;
+    static __device__ __forceinline__ float to_f32(float x) { return x; }
+    static __device__ __forceinline__ float from_f32(float x) { return x; }
+};
+
+template <>
+struct Elem<ELX_F16> {
+    typedef uint16_t scalar;
+    typedef u16x4 vec4;
+    static __device__ __forceinline__ float to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+    // v_cvt_f16_f32: round to nearest even, overflow to inf, subnormals kept
+    static __device__ __forceinline__ uint16_t from_f32(float x) {
+        return __builtin_bit_cast(uint16_t, (_Float16)x);
+    }
+};
+
+template <>
+struct Elem<ELX_BF16> {
+    typedef uint16_t scalar;
+    typedef u16x4 vec4;
+    static __device__ __forceinline__ float to_f32(uint16_t b) {
+        return __builtin_bit_cast(float, (uint32_t)b << 16);
+    }
+    // round to nearest even on the bit pattern; NaN stays a quiet NaN
+    static __device__ __forceinline__ uint16_t from_f32(float x) {
+        uint32_t u = __builtin_bit_cast(uint32_t, x);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+        u += 0x7FFFu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+};
+
+template <typename V>
+__device__ __forceinline__ V ld_stream(const V *p) {
+    return __builtin_nontemporal_load(p);
+}
+template <typename V>
+__device__ __forceinline__ void st_stream(V *p, V x) {
+    __builtin_nontemporal_store(x, p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// the update of one element
+// ---------------------------------------------------------------------------------------------
+
+struct Hyper {
+    float decay_mul, l2_wd, lerp_w, beta2, omb2, bc2_sqrt, eps, neg_step;
+    uint32_t flags;
+};
+
+__device__ __forceinline__ Hyper load_hyper(const ElxHyper *__restrict__ h) {
+    Hyper r;
+    r.decay_mul = h->decay_mul;
+    r.l2_wd = h->l2_wd;
+    r.lerp_w = h->lerp_w;
+    r.beta2 = h->beta2;
+    r.omb2 = h->omb2;
+    r.bc2_sqrt = h->bc2_sqrt;
+    r.eps = h->eps;
+    r.neg_step = h->neg_step;
+    r.flags = h->flags;
+    return r;
+}
+
+// How the gradient is unscaled: not at all, by an exact multiply with 1/div_scale (div_scale a
+// power of two: same bits as the division), or by a true IEEE division.
+enum { kDivNone = 0, kDivMulInv = 1, kDivTrue = 2 };
+
+struct Unscale {
+    float div_scale, inv_scale;
+    int mode;
+};
+
+__device__ __forceinline__ void adam_elem(float g, float &p, float &m, float &v, const Hyper &h, const Unscale &us) {
+    if (us.mode == kDivMulInv)
+        g = g * us.inv_scale;
+    else if (us.mode == kDivTrue)
+        g = g / us.div_scale;
+    p = p * h.decay_mul;                                   // AdamW: p *= 1 - lr*wd (1.0f otherwise)
+    if (h.flags & ELX_HYPER_L2) g = fmaf(h.l2_wd, p, g);  // L2: g += wd*p
+    const float diff = g - m;
+    const float base = (h.flags & ELX_HYPER_LERP_FROM_G) ? g : m;
+    m = fmaf(h.lerp_w, diff, base);                        // m.lerp_(g, 1-beta1)
+    v = fmaf(h.omb2 * g, g, v * h.beta2);                  // v.mul_(beta2).addcmul_(g, g, 1-beta2)
+    const float denom = sqrtf(v) / h.bc2_sqrt + h.eps;     // sqrt(v)/sqrt(bc2) + eps
+    p = p + (h.neg_step * m) / denom;                      // p.addcdiv_(m, denom, -lr/bc1)
+}
+
+// ---------------------------------------------------------------------------------------------
+// fused update + writeback
+// ---------------------------------------------------------------------------------------------
+
+// Whole tile inside one segment: every stream moves as 128-bit (fp32) / 64-bit (16-bit types)
+// accesses, lane l of access u touching elements [u*kSpan + 4l, u*kSpan + 4l + 4) so that each
+// wavefront instruction covers one contiguous 1 KiB (fp32) or 512 B (16-bit) span.
+template <int GD, int LD, bool NT>
+__device__ __forceinline__ void tile_update_vec(const ElxChunk &c, uint64_t base, const Hyper &h, const Unscale &us) {
+    typedef typename Elem<GD>::vec4 gvec;
+    const uint32_t lane_off = threadIdx.x * kVec;
+    const gvec *gp = c.grad ? reinterpret_cast<const gvec *>(reinterpret_cast<const typename Elem<GD>::scalar *>(c.grad) + base + lane_off) : nullptr;
+    f32x4 *pp = reinterpret_cast<f32x4 *>(c.master + base + lane_off);
+    f32x4 *mp = reinterpret_cast<f32x4 *>(c.m + base + lane_off);
+    f32x4 *vp = reinterpret_cast<f32x4 *>(c.v + base + lane_off);
+    constexpr uint32_t kStride = kSpan / kVec;    // in vec4 units
+
+    gvec G[kUnroll];
+    f32x4 P[kUnroll], M[kUnroll], V[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        if (gp) G[u] = NT ? ld_stream(gp + u * kStride) : gp[u * kStride];
+        P[u] = NT ? ld_stream(pp + u * kStride) : pp[u * kStride];
+        M[u] = NT ? ld_stream(mp + u * kStride) : mp[u * kStride];
+        V[u] = NT ? ld_stream(vp + u * kStride) : vp[u * kStride];
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+        for (int k = 0; k < kVec; ++k) {
+            float g = gp ? Elem<GD>::to_f32(G[u][k]) : 0.0f;
+            float p = P[u][k], m = M[u][k], v = V[u][k];
+            adam_elem(g, p, m, v, h, us);
+            P[u][k] = p;
+            M[u][k] = m;
+            V[u][k] = v;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        if (NT) {
+            st_stream(pp + u * kStride, P[u]);
+            st_stream(mp + u * kStride, M[u]);
+            st_stream(vp + u * kStride, V[u]);
+        } else {
+            pp[u * kStride] = P[u];
+            mp[u * kStride] = M[u];
+            vp[u * kStride] = V[u];
+        }
+    }
+    if constexpr (LD != ELX_NONE) {
+        if (c.lowp_out) {
+            typedef typename Elem<LD>::vec4 lvec;
+            lvec *lp = reinterpret_cast<lvec *>(reinterpret_cast<typename Elem<LD>::scalar *>(c.lowp_out) + base + lane_off);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                lvec L;
+#pragma unroll
+                for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
+                if (NT)
+                    st_stream(lp + u * kStride, L);
+                else
+                    lp[u * kStride] = L;
+            }
+        }
+    }
+}
+
+// Whole tile outside every segment (padding, or the writeback-only launch): refresh only.
+template <int LD, bool NT>
+__device__ __forceinline__ void tile_refresh_vec(const ElxChunk &c, uint64_t base) {
+    if constexpr (LD != ELX_NONE) {
+        if (!c.lowp_out) return;
+        typedef typename Elem<LD>::vec4 lvec;
+        const uint32_t lane_off = threadIdx.x * kVec;
+        const f32x4 *pp = reinterpret_cast<const f32x4 *>(c.master + base + lane_off);
+        lvec *lp = reinterpret_cast<lvec *>(reinterpret_cast<typename Elem<LD>::scalar *>(c.lowp_out) + base + lane_off);
+        constexpr uint32_t kStride = kSpan / kVec;
+        f32x4 P[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) P[u] = NT ? ld_stream(pp + u * kStride) : pp[u * kStride];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            lvec L;
+#pragma unroll
+            for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
+            if (NT)
+                st_stream(lp + u * kStride, L);
+            else
+                lp[u * kStride] = L;
+        }
+    }
+}
+
+// Any tile: element by element, each element looking up the segment that covers it.  Used for
+// tiles that straddle a segment boundary, the partial tile at the end of a chunk, and buffers
+// whose base pointers are not 16-byte aligned.  `s` is the first segment whose end is > base.
+template <int GD, int LD>
+__device__ __forceinline__ void tile_scalar(const ElxChunk &c, uint64_t base, uint32_t tile_n, uint32_t s,
+                                            const ElxSeg *__restrict__ segs, const ElxHyper *__restrict__ hypers,
+                                            const Unscale &us, bool refresh_only) {
+    typedef typename Elem<GD>::scalar gscalar;
+    const gscalar *grad = reinterpret_cast<const gscalar *>(c.grad);
+    for (uint32_t i = threadIdx.x; i < tile_n; i += kThreads) {
+        const uint64_t e = base + i;
+        float p = c.master[e];
+        if (!refresh_only) {
+            uint32_t cs = s;
+            while (cs < c.seg_end && segs[cs].end <= e) ++cs;
+            if (cs < c.seg_end && segs[cs].begin <= e) {
+                const Hyper h = load_hyper(hypers + segs[cs].hyper);
+                float g = grad ? Elem<GD>::to_f32(grad[e]) : 0.0f;
+                float m = c.m[e], v = c.v[e];
+                adam_elem(g, p, m, v, h, us);
+                c.master[e] = p;
+                c.m[e] = m;
+                c.v[e] = v;
+            }
+        }
+        if constexpr (LD != ELX_NONE) {
+            if (c.lowp_out) reinterpret_cast<typename Elem<LD>::scalar *>(c.lowp_out)[e] = Elem<LD>::from_f32(p);
+        }
+    }
+}
+
+template <int GD, int LD, bool NT>
+__global__ __launch_bounds__(kThreads) void adam_step_kernel(const ElxChunk *__restrict__ chunks, uint32_t n_chunks,
+                                                             const ElxSeg *__restrict__ segs,
+                                                             const ElxHyper *__restrict__ hypers, uint64_t total_tiles,
+                                                             Unscale us, uint32_t scalar_only, uint32_t refresh_only) {
+    for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+        // chunk that owns tile t: the last one whose tile_begin is <= t (uniform -> scalar loads)
+        uint32_t lo = 0, hi = n_chunks;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (chunks[mid].tile_begin <= t)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        const ElxChunk c = chunks[lo];
+        const uint64_t base = (t - c.tile_begin) * kTile;
+        if (base >= c.n_alloc) continue;    // cannot happen with checked tables
+        const uint64_t left = c.n_alloc - base;
+        const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
+        const bool whole = (tile_n == kTile) && !scalar_only;
+
+        if (refresh_only) {
+            if (whole)
+                tile_refresh_vec<LD, NT>(c, base);
+            else
+                tile_scalar<GD, LD>(c, base, tile_n, 0, segs, hypers, us, true);
+            continue;
+        }
+
+        // first segment of the chunk that ends after the start of the tile
+        uint32_t s = c.seg_begin, s_hi = c.seg_end;
+        while (s < s_hi) {
+            const uint32_t mid = (s + s_hi) >> 1;
+            if (segs[mid].end > base)
+                s_hi = mid;
+            else
+                s = mid + 1;
+        }
+        const bool has = s < c.seg_end;
+        const uint64_t sb = has ? segs[s].begin : ~0ull;
+        const uint64_t se = has ? segs[s].end : 0ull;
+
+        if (whole && has && sb <= base && se >= base + kTile) {
+            const Hyper h = load_hyper(hypers + segs[s].hyper);
+            tile_update_vec<GD, LD, NT>(c, base, h, us);
+        } else if (whole && (!has || sb >= base + kTile)) {
+            tile_refresh_vec<LD, NT>(c, base);
+        } else {
+            tile_scalar<GD, LD>(c, base, tile_n, s, segs, hypers, us, false);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// stats: overflow flag + sum of squares
+// ---------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ double wave_sum(double x) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, 64);
+    return x;
+}
+
+// Folds (sum, flag) over the workgroup; the result is valid in thread 0.  Fixed order.
+__device__ __forceinline__ void block_fold(double &sum, uint32_t &flag) {
+    __shared__ double s_sum[kThreads / 64];
+    __shared__ uint32_t s_flag[kThreads / 64];
+    sum = wave_sum(sum);
+    flag = __ballot(flag != 0) != 0ull ? 1u : 0u;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) {
+        s_sum[wave] = sum;
+        s_flag[wave] = flag;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        uint32_t f = 0;
+        for (int w = 0; w < kThreads / 64; ++w) {
+            t += s_sum[w];
+            f |= s_flag[w];
+        }
+        sum = t;
+        flag = f;
+    }
+}
+
+// x*x added in fp32; x*0 added into `poison`, which turns NaN exactly when x is inf or NaN.
+__device__ __forceinline__ void stats_elem(float x, float &acc, float &poison) {
+    acc = fmaf(x, x, acc);
+    poison = fmaf(x, 0.0f, poison);
+}
+
+template <int GD>
+__global__ __launch_bounds__(kThreads) void grad_stats_kernel(const ElxChunk *__restrict__ chunks, uint32_t bpc,
+                                                              ElxStats *__restrict__ partials, uint32_t scalar_only) {
+    typedef typename Elem<GD>::scalar gscalar;
+    constexpr uint32_t kEpl = 16 / sizeof(gscalar);    // elements per lane per 128-bit load
+    constexpr uint32_t kSSpan = kThreads * kEpl;
+    constexpr uint32_t kSTile = kSSpan * kUnroll;
+    typedef gscalar gvec __attribute__((ext_vector_type(kEpl)));
+
+    const ElxChunk c = chunks[blockIdx.y];
+    const gscalar *g = reinterpret_cast<const gscalar *>(c.grad);
+    const uint64_t n = g ? c.n_valid : 0;
+    const uint64_t n_tiles = (n + kSTile - 1) / kSTile;
+
+    double sum = 0.0;
+    float poison = 0.0f;
+    for (uint64_t t = blockIdx.x; t < n_tiles; t += bpc) {
+        const uint64_t base = t * kSTile;
+        float acc = 0.0f;
+        if (base + kSTile <= n && !scalar_only) {
+            const gvec *gp = reinterpret_cast<const gvec *>(g + base) + threadIdx.x;
+            gvec G[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) G[u] = ld_stream(gp + u * kThreads);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (uint32_t k = 0; k < kEpl; ++k) stats_elem(Elem<GD>::to_f32(G[u][k]), acc, poison);
+        } else {
+            const uint64_t left = n - base;
+            const uint32_t tile_n = left < kSTile ? (uint32_t)left : kSTile;
+            for (uint32_t i = threadIdx.x; i < tile_n; i += kThreads) stats_elem(Elem<GD>::to_f32(g[base + i]), acc, poison);
+        }
+        sum += (double)acc;
+    }
+    uint32_t flag = (poison != poison) ? 1u : 0u;
+    block_fold(sum, flag);
+    if (threadIdx.x == 0) {
+        ElxStats r;
+        r.sumsq = sum;
+        r.overflow = flag;
+        r.reserved = 0;
+        partials[(uint64_t)blockIdx.y * bpc + blockIdx.x] = r;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void stats_finish_kernel(const ElxStats *__restrict__ partials, uint32_t bpc,
+                                                                ElxStats *__restrict__ out) {
+    const ElxStats *row = partials + (uint64_t)blockIdx.x * bpc;
+    double sum = 0.0;
+    uint32_t flag = 0;
+    for (uint32_t i = threadIdx.x; i < bpc; i += kThreads) {
+        sum += row[i].sumsq;
+        flag |= row[i].overflow;
+    }
+    block_fold(sum, flag);
+    if (threadIdx.x == 0) {
+        ElxStats r;
+        r.sumsq = sum;
+        r.overflow = flag;
+        r.reserved = 0;
+        out[blockIdx.x] = r;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side of the ABI
+// ---------------------------------------------------------------------------------------------
+
+bool is_lowp_or_f32(int d) { return d == ELX_F32 || d == ELX_F16 || d == ELX_BF16; }
+
+uint32_t elem_size(int d) { return d == ELX_F32 ? 4u : 2u; }
+
+// div_scale is a power of two whose reciprocal is a normal fp32 number
+bool exact_reciprocal(float s) {
+    uint32_t u;
+    __builtin_memcpy(&u, &s, 4);
+    const uint32_t exp = (u >> 23) & 0xFFu, man = u & 0x7FFFFFu;
+    return (u >> 31) == 0 && man == 0 && exp >= 1 && exp <= 252;
+}
+
+template <int GD, int LD>
+int launch_step(bool nt, dim3 grid, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks, const ElxSeg *segs,
+                const ElxHyper *hypers, uint64_t total_tiles, Unscale us, uint32_t scalar_only, uint32_t refresh_only) {
+    if (nt)
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true>), grid, dim3(kThreads), 0, st, chunks, n_chunks, segs, hypers,
+                           total_tiles, us, scalar_only, refresh_only);
+    else
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false>), grid, dim3(kThreads), 0, st, chunks, n_chunks, segs, hypers,
+                           total_tiles, us, scalar_only, refresh_only);
+    return (int)hipGetLastError();
+}
+
+int dispatch_step(int gd, int ld, bool nt, dim3 grid, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
+                  const ElxSeg *segs, const ElxHyper *hypers, uint64_t total_tiles, Unscale us, uint32_t scalar_only,
+                  uint32_t refresh_only) {
+#define ELX_CASE(G, L)                                                                                          \
+    if (gd == G && ld == L)                                                                                     \
+        return launch_step<G, L>(nt, grid, st, chunks, n_chunks, segs, hypers, total_tiles, us, scalar_only, refresh_only);
+    ELX_CASE(ELX_F32, ELX_NONE)
+    ELX_CASE(ELX_F32, ELX_F32)
+    ELX_CASE(ELX_F16, ELX_NONE)
+    ELX_CASE(ELX_F16, ELX_F16)
+    ELX_CASE(ELX_BF16, ELX_NONE)
+    ELX_CASE(ELX_BF16, ELX_BF16)
+#undef ELX_CASE
+    return ELX_E_DTYPE;
+}
+
+dim3 step_grid(uint64_t total_tiles, uint32_t max_blocks) {
+    uint64_t blocks = total_tiles;
+    if (max_blocks && blocks > max_blocks) blocks = max_blocks;
+    if (blocks > 0x7FFFFFFFull) blocks = 0x7FFFFFFFull;
+    return dim3((uint32_t)blocks);
+}
+
+}    // namespace
+
+extern "C" {
+
+int elx_version(void) { return ELX_ABI_VERSION; }
+
+uint32_t elx_tile_elems(void) { return kTile; }
+uint32_t elx_sizeof_chunk(void) { return (uint32_t)sizeof(ElxChunk); }
+uint32_t elx_sizeof_seg(void) { return (uint32_t)sizeof(ElxSeg); }
+uint32_t elx_sizeof_hyper(void) { return (uint32_t)sizeof(ElxHyper); }
+uint32_t elx_sizeof_stats(void) { return (uint32_t)sizeof(ElxStats); }
+
+const char *elx_strerror(int code) {
+    switch (code) {
+        case 0: return "success";
+        case ELX_E_NULL: return "elx: a required pointer is NULL";
+        case ELX_E_DTYPE: return "elx: unknown or unsupported dtype combination";
+        case ELX_E_ALIGN: return "elx: a chunk base pointer is not aligned to its element size";
+        case ELX_E_RANGE: return "elx: a range is out of bounds (begin > end, end > n_alloc, n_valid > n_alloc, segment range or hyper index)";
+        case ELX_E_ORDER: return "elx: segments of a chunk are not sorted or overlap";
+        case ELX_E_TILES: return "elx: tile_begin / total_tiles disagree with the chunk sizes";
+        case ELX_E_SIZE: return "elx: a count is zero or exceeds what a launch can address";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "elx: unknown error code";
+}
+
+int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *h_segs, uint32_t n_segs,
+                     uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles, int *all_aligned16) {
+    if (!h_chunks || !total_tiles || !all_aligned16 || (n_segs && !h_segs)) return ELX_E_NULL;
+    if (n_chunks == 0 || n_chunks > 65535u) return ELX_E_SIZE;
+    if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
+    if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    const uintptr_t gmask = elem_size(grad_dtype) - 1;
+    uint64_t tiles = 0;
+    int aligned = 1;
+    for (uint32_t i = 0; i < n_chunks; ++i) {
+        const ElxChunk &c = h_chunks[i];
+        if (!c.master || !c.m || !c.v) return ELX_E_NULL;
+        if (c.lowp_out && lowp_dtype == ELX_NONE) return ELX_E_DTYPE;
+        if (c.n_alloc == 0) return ELX_E_SIZE;
+        if (c.n_valid > c.n_alloc) return ELX_E_RANGE;
+        const uintptr_t ptrs[5] = {(uintptr_t)c.grad, (uintptr_t)c.lowp_out, (uintptr_t)c.master, (uintptr_t)c.m,
+                                   (uintptr_t)c.v};
+        if ((ptrs[0] & gmask) || (ptrs[1] & gmask) || (ptrs[2] & 3u) || (ptrs[3] & 3u) || (ptrs[4] & 3u))
+            return ELX_E_ALIGN;
+        for (int k = 0; k < 5; ++k)
+            if (ptrs[k] & 15u) aligned = 0;
+        if (c.tile_begin != tiles) return ELX_E_TILES;
+        tiles += (c.n_alloc + kTile - 1) / kTile;
+        if (c.seg_begin > c.seg_end || c.seg_end > n_segs) return ELX_E_RANGE;
+        uint64_t prev_end = 0;
+        for (uint32_t s = c.seg_begin; s < c.seg_end; ++s) {
+            const ElxSeg &sg = h_segs[s];
+            if (sg.begin >= sg.end || sg.end > c.n_alloc) return ELX_E_RANGE;
+            if (sg.hyper >= n_hypers) return ELX_E_RANGE;
+            if (sg.begin < prev_end) return ELX_E_ORDER;
+            prev_end = sg.end;
+        }
+    }
+    *total_tiles = tiles;
+    *all_aligned16 = aligned;
+    return 0;
+}
+
+int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
+                      ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream) {
+    if (!d_chunks || !d_partials || !d_stats) return ELX_E_NULL;
+    if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxStatsBlocks)
+        return ELX_E_SIZE;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid(blocks_per_chunk, n_chunks);
+    const uint32_t so = scalar_only ? 1u : 0u;
+    switch (grad_dtype) {
+        case ELX_F32:
+            hipLaunchKernelGGL((grad_stats_kernel<ELX_F32>), grid, dim3(kThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
+            break;
+        case ELX_F16:
+            hipLaunchKernelGGL((grad_stats_kernel<ELX_F16>), grid, dim3(kThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
+            break;
+        case ELX_BF16:
+            hipLaunchKernelGGL((grad_stats_kernel<ELX_BF16>), grid, dim3(kThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
+            break;
+        default: return ELX_E_DTYPE;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_chunks), dim3(kThreads), 0, st, d_partials, blocks_per_chunk, d_stats);
+    return (int)hipGetLastError();
+}
+
+int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
+                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles, float div_scale, int grad_dtype,
+                     int lowp_dtype, uint32_t flags, uint32_t max_blocks, void *stream) {
+    if (!d_chunks || (n_segs && (!d_segs || !d_hypers))) return ELX_E_NULL;
+    if (n_chunks == 0 || total_tiles == 0 || (n_segs && n_hypers == 0)) return ELX_E_SIZE;
+    if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
+    if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    Unscale us;
+    us.div_scale = div_scale;
+    us.inv_scale = 1.0f;
+    us.mode = kDivNone;
+    if (div_scale > 0.0f) {
+        if (exact_reciprocal(div_scale)) {
+            us.mode = kDivMulInv;
+            us.inv_scale = 1.0f / div_scale;
+        } else {
+            us.mode = kDivTrue;
+        }
+    }
+    const bool nt = true;
+    return dispatch_step(grad_dtype, lowp_dtype, nt, step_grid(total_tiles, max_blocks), (hipStream_t)stream, d_chunks,
+                         n_chunks, d_segs, d_hypers, total_tiles, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 0u);
+}
+
+int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles, int lowp_dtype, uint32_t flags,
+                     uint32_t max_blocks, void *stream) {
+    if (!d_chunks) return ELX_E_NULL;
+    if (n_chunks == 0 || total_tiles == 0) return ELX_E_SIZE;
+    if (!is_lowp_or_f32(lowp_dtype)) return ELX_E_DTYPE;
+    Unscale us;
+    us.div_scale = -1.0f;
+    us.inv_scale = 1.0f;
+    us.mode = kDivNone;
+    return dispatch_step(lowp_dtype, lowp_dtype, true, step_grid(total_tiles, max_blocks), (hipStream_t)stream, d_chunks,
+                         n_chunks, nullptr, nullptr, total_tiles, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 1u);
+}
+
+}    // extern "C"

@@ -1,0 +1,272 @@
+"""The module side of the optimizer step: chunk plans and the pairing of low-precision parameter
+chunks with fp32 optimizer chunks (``elixir/search/result.py``, ``elixir/search/mini_waste.py:78-96``,
+``elixir/wrapper/module.py:21-25,77-138,258-344``).
+
+``ElixirModule`` here is the part of the reference's module wrapper that ``ElixirOptimizer`` reads:
+it builds the paired chunk groups and exposes ``param_chunk_group``, ``optim_chunk_group``,
+``fetcher.get_one_chunk``, ``use_amp``, ``state_dict`` / ``load_state_dict``.  The hook-driven
+forward/backward (replicated cache, gather, reduce-scatter) is not part of this path; in its place
+``land_gradients`` moves the ``.grad`` of the wrapped module's parameters into the chunk shards the
+way the reference's gradient handler and chunk reduction leave them, and ``materialize_params``
+points the parameters back at the refreshed low-precision values.
+"""
+from collections import OrderedDict
+from typing import Any, Dict, Iterable, List, Mapping, NamedTuple, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+from .chunk import Chunk, ChunkGroup, gpu_device
+
+
+class ChunkPlan(NamedTuple):
+    """Instructs the initialization of a chunk (result.py:8-20)."""
+    name_list: List[str]
+    chunk_size: int
+    chunk_dtype: torch.dtype
+    kwargs: Dict
+
+
+class SearchResult(object):
+
+    def __init__(self, chunk_group: ChunkGroup, chunk_plans: List[ChunkPlan],
+                 param_called_per_step: List[List[str]] = None) -> None:
+        super().__init__()
+        self.chunk_group = chunk_group
+        self.param_chunk_plans = chunk_plans
+        self.param_called_per_step = param_called_per_step
+
+
+def to_divide(a: int, b: int) -> int:
+    return a + (-a % b)
+
+
+def greedy_groups(sizes: Sequence[int], chunk_size: int) -> List[List[int]]:
+    """The packing rule of mini_waste.py:78-96: walk the tensors in order and open a new chunk
+    whenever the room left in the current one is smaller than the next tensor."""
+    groups: List[List[int]] = []
+    last_left = 0
+    for i, p_size in enumerate(sizes):
+        if last_left < p_size:
+            last_left = chunk_size
+            groups.append([])
+        assert last_left >= p_size, f'tensor {i} with {p_size} elements does not fit a chunk of {chunk_size}'
+        last_left -= p_size
+        groups[-1].append(i)
+    return groups
+
+
+def greedy_search(named_sizes: Sequence[Tuple[str, int]], chunk_size: int, dtype: torch.dtype,
+                  shard_device: Optional[torch.device] = None) -> SearchResult:
+    """A search result that packs every tensor into public chunks of one size with the greedy rule."""
+    names = [n for n, _ in named_sizes]
+    groups = greedy_groups([s for _, s in named_sizes], chunk_size)
+    kwargs = {} if shard_device is None else dict(shard_device=shard_device)
+    plans = [ChunkPlan([names[i] for i in g], chunk_size, dtype, dict(kwargs)) for g in groups]
+    return SearchResult(ChunkGroup(None), plans)
+
+
+def get_param_optim_data(param_data: torch.Tensor, param_dtype: torch.dtype, device: torch.device):
+    """module.py:21-25: the master copy is fp32, the parameter takes the training dtype."""
+    param_data = param_data.to(device)
+    optim_data = param_data.clone() if param_data.dtype == torch.float else param_data.float()
+    param_data = param_data.to(param_dtype)
+    return param_data, optim_data
+
+
+class _Fetcher:
+    """The one method of the chunk fetcher the optimizer wrapper calls (fetcher.py)."""
+
+    def __init__(self, group: ChunkGroup):
+        self.group = group
+
+    def get_one_chunk(self, tensor: torch.Tensor) -> Chunk:
+        return self.group.ten_to_chunk.get(tensor)
+
+
+class ElixirModule(nn.Module):
+    """Chunked storage for the parameters of ``module``.
+
+    args:
+        module: the training module, or an ordered mapping ``name -> shape`` for a synthetic
+            parameter set whose values are produced in place, directly in the chunk buffers
+        search_result: chunk plans (``greedy_search`` builds one)
+        dtype: the training dtype: float32, float16, or bfloat16
+    """
+
+    def __init__(self,
+                 module,
+                 search_result: SearchResult,
+                 process_group=None,
+                 prefetch: bool = False,
+                 dtype: torch.dtype = torch.float,
+                 reduce_always_fp32: bool = False,
+                 output_fp32: bool = False,
+                 use_fused_kernels: bool = False) -> None:
+        super().__init__()
+        assert dtype in {torch.float, torch.float16, torch.bfloat16}
+        if prefetch or use_fused_kernels:
+            raise NotImplementedError('prefetch and fused forward kernels belong to the forward/backward pass')
+
+        self.synthetic = not isinstance(module, nn.Module)
+        self.module = module if not self.synthetic else None
+        self.dtype = dtype
+        self.use_amp = (dtype == torch.float16)
+        self.process_group = process_group
+        self.reduce_always_fp32 = reduce_always_fp32
+        self.output_fp32 = output_fp32
+        self.buffer = None
+
+        self.no_grad_state_dict = dict()
+        self.grad_state_dict: Dict[str, nn.Parameter] = OrderedDict()
+        self.param_to_optim: Dict[nn.Parameter, torch.Tensor] = dict()
+        self.__init_chunk_group(search_result, module)
+        self.fetcher = _Fetcher(self.param_chunk_group)
+
+    def __init_chunk_group(self, sr: SearchResult, module):
+        device = gpu_device() if torch.cuda.is_available() else torch.device('cpu')
+        if self.synthetic:
+            for name, shape in module.items():
+                self.grad_state_dict[name] = nn.Parameter(torch.empty(tuple(shape), dtype=self.dtype, device='meta'))
+        else:
+            state_dict = module.state_dict(keep_vars=True)
+            for name, tensor in state_dict.items():
+                if isinstance(tensor, nn.Parameter):
+                    assert tensor.is_floating_point(), 'the dtypes of parameters should be float dtypes'
+                    if tensor.requires_grad:
+                        self.grad_state_dict[name] = tensor
+                    else:
+                        self.no_grad_state_dict[name] = tensor
+                        tensor.data = tensor.data.to(dtype=self.dtype, device=device)
+                else:
+                    to_dtype = self.dtype if tensor.is_floating_point() else tensor.dtype
+                    tensor.data = tensor.data.to(dtype=to_dtype, device=device)
+
+        self.param_chunk_group = sr.chunk_group
+        self.optim_chunk_group = ChunkGroup(None)
+        vis_set = set()
+
+        for plan in sr.param_chunk_plans:
+            assert plan.chunk_dtype == self.dtype
+            # optimizer chunks should not be gathered
+            optim_kwargs = dict(plan.kwargs)
+            if 'rcache_fused' in optim_kwargs:
+                optim_kwargs['rcache_fused'] = False
+
+            p_chunk = self.param_chunk_group.open_chunk(chunk_size=plan.chunk_size, chunk_dtype=plan.chunk_dtype,
+                                                        process_group=self.process_group, chunk_config=plan.kwargs)
+            o_chunk = self.optim_chunk_group.open_chunk(chunk_size=plan.chunk_size, chunk_dtype=torch.float,
+                                                        process_group=self.process_group, chunk_config=optim_kwargs)
+
+            for name in plan.name_list:
+                param = self.grad_state_dict[name]
+                if self.synthetic:
+                    optim_data = torch.empty(param.shape, dtype=torch.float, device='meta')
+                else:
+                    param_data, optim_data = get_param_optim_data(param.data, self.dtype, device)
+                    param.data = param_data
+                p_chunk.append_tensor(param)
+                o_chunk.append_tensor(optim_data)
+                self.param_to_optim[param] = optim_data
+                vis_set.add(param)
+
+            self.param_chunk_group.close_chunk(p_chunk)
+            self.optim_chunk_group.close_chunk(o_chunk)
+            p_chunk.init_pair(o_chunk)
+
+        # sanity check: every parameter needed gradient has been initialized
+        for param in self.grad_state_dict.values():
+            assert param in vis_set
+
+        if not self.synthetic:
+            self.materialize_params()
+
+    # ------------------------------------------------------------------ parameters and gradients
+
+    def parameters(self, recurse: bool = True):
+        if self.synthetic:
+            return iter(self.grad_state_dict.values())
+        return super().parameters(recurse)
+
+    def named_parameters(self, *args, **kwargs):
+        if self.synthetic:
+            return iter(self.grad_state_dict.items())
+        return super().named_parameters(*args, **kwargs)
+
+    @property
+    def param_chunks(self) -> List[Chunk]:
+        return self.param_chunk_group.all_chunks
+
+    def materialize_params(self) -> None:
+        """Give every parameter of the wrapped module a private copy of its low-precision values
+        (what a gather into the replicated cache would expose to the forward pass)."""
+        assert not self.synthetic
+        for param in self.grad_state_dict.values():
+            chunk = self.param_chunk_group.ten_to_chunk[param]
+            info = chunk.tensors_info[param]
+            param.data = chunk.shard[info.offset:info.end].clone().view(param.shape)
+
+    def forward(self, *args, **kwargs):
+        assert not self.synthetic
+        outputs = self.module(*args, **kwargs)
+        if self.output_fp32:
+            outputs = outputs.float()
+        return outputs
+
+    def backward(self, loss: torch.Tensor):
+        loss.backward()
+        self.land_gradients()
+        self.module.zero_grad(set_to_none=True)
+
+    def land_gradients(self, sync: bool = False) -> None:
+        """module.py:177-190 + chunk.py:358-393 for one process: each parameter's gradient is
+        copied into its slice of a full-size payload (zero elsewhere, as the replicated block of the
+        reference is after a gather of zero padding), and the payload overwrites the shard.  With
+        ``sync`` the flags are computed per chunk here, otherwise by the optimizer in one launch."""
+        assert not self.synthetic
+        for chunk in self.param_chunks:
+            payload = torch.zeros(chunk.chunk_size, dtype=chunk.chunk_dtype, device=chunk.shard_device)
+            for param, info in chunk.tensors_info.items():
+                assert param.grad is not None, 'every parameter of a chunk needs a gradient before the reduction'
+                payload[info.offset:info.end].copy_(param.grad.data.flatten())
+            chunk.reduce_chunk(payload, always_fp32=self.reduce_always_fp32, sync=sync)
+
+    # ------------------------------------------------------------------ checkpoint of the weights
+
+    def state_dict(self, destination=None, prefix='', keep_vars=False, only_rank_0: bool = False,
+                   from_param: bool = False):
+        """module.py:258-292: weights come from the fp32 optimizer chunks (or, with ``from_param``,
+        from the low-precision chunks), as CPU tensors."""
+        assert keep_vars is False, 'state_dict can not keep variables in ElixirModule'
+        assert not self.synthetic
+        module_state_dict = self.module.state_dict(destination=destination, prefix=prefix, keep_vars=True)
+        for name, tensor in module_state_dict.items():
+            key = name[len(prefix):]
+            if key in self.grad_state_dict:
+                param = self.grad_state_dict[key]
+                p_chunk = self.param_chunk_group.ten_to_chunk[param]
+                info = p_chunk.tensors_info[param]
+                src = p_chunk if from_param else p_chunk.paired_chunk
+                module_state_dict[name] = src.shard[info.offset:info.end].view(param.shape).cpu()
+            else:
+                module_state_dict[name] = tensor.detach()
+        return module_state_dict
+
+    def load_state_dict(self, state_dict: Mapping[str, Any], only_rank_0: bool = False):
+        """module.py:294-344: values are written into the fp32 optimizer chunks, then the paired
+        low-precision chunks are refreshed."""
+        assert not self.synthetic
+        touched = set()
+        for name, maybe_tensor in state_dict.items():
+            if name in self.no_grad_state_dict:
+                self.no_grad_state_dict[name].copy_(maybe_tensor)
+            elif name in self.grad_state_dict:
+                param = self.grad_state_dict[name]
+                p_chunk = self.param_chunk_group.ten_to_chunk[param]
+                info = p_chunk.tensors_info[param]
+                o_chunk = p_chunk.paired_chunk
+                o_chunk.shard[info.offset:info.end].copy_(maybe_tensor.data.flatten())
+                touched.add(p_chunk)
+        for p_chunk in touched:
+            p_chunk.optim_update()
+        self.materialize_params()

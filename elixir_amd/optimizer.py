@@ -1,0 +1,403 @@
+"""``ElixirOptimizer``: the optimizer wrapper of ``elixir/wrapper/optimizer.py`` with the same
+constructor, methods and control flow, driving the HIP kernels.
+
+One step is:
+
+  1. one stats launch over every parameter chunk that has no fresh flags (overflow flag and sum of
+     squares of the still-scaled gradients) and ONE device-to-host copy of 16 bytes per chunk
+     (the reference pays two ``.item()`` per chunk at gradient-landing time, plus one for the loss
+     scale, plus one for the norm);
+  2. the host decisions of optimizer.py:192-209 in Python floats: overflow -> skip and back off,
+     otherwise combined scale = loss scale (x clip coefficient);
+  3. one fused launch: unscale + Adam/AdamW on master/m/v + low-precision writeback
+     (optimizer.py:216-219), or the writeback alone on a skipped step (optimizer.py:196-203).
+
+Differences from the reference, all on purpose:
+  * clipping works: ``max_norm > 0`` switches ``l2_norm_flag`` on for every parameter chunk (the
+    reference never sets the flag and trips its own assertion, optimizer.py:152);
+  * bfloat16 parameter chunks are accepted (``use_amp`` stays tied to float16, so bf16 trains
+    with a constant scale of 1 and the overflow check still runs);
+  * exp_avg / exp_avg_sq live in flat per-chunk buffers (``state[p]['exp_avg']`` are views).
+"""
+import math
+from collections import defaultdict
+from enum import Enum
+from typing import Dict, List, Set, Tuple
+
+import numpy as np
+import torch
+from torch.nn import Parameter
+
+from . import _abi
+from .chunk import Chunk, DeviceTable, dtype_code, run_grad_stats
+from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
+from .hybrid_adam import HybridAdam
+
+_AVAIL_OPTIM_LIST = {HybridAdam}
+
+
+class OptimState(Enum):
+    SCALED = 0
+    UNSCALED = 1
+
+
+def calc_combined_scale(loss_scale: float, total_norm, max_norm: float, clipping: bool) -> float:
+    """optimizer.py:166-183 in Python floats: gradient = gradient / combined scale."""
+    combined_scale = loss_scale
+    if clipping:
+        clip = ((total_norm / loss_scale) + 1e-6) / max_norm
+        if clip > 1:
+            combined_scale = clip * loss_scale
+    if combined_scale == 1:
+        return -1
+    return combined_scale
+
+
+class ElixirOptimizer:
+    """A wrapper for optimizers; one ElixirOptimizer corresponds to one chunked module.
+
+    Args:
+        module: the chunked module (``param_chunk_group``, ``optim_chunk_group``,
+            ``fetcher.get_one_chunk``, ``use_amp``)
+        optimizer: the inner optimizer built on the module's real parameters; a ``HybridAdam``
+            takes the fused path, any other element-wise torch optimizer runs unfused and only
+            without loss scaling and clipping (optimizer.py:211-214)
+        initial_scale ... max_scale: dynamic loss scale settings (used when ``module.use_amp``)
+        max_norm: global L2 gradient-norm clip, 0 disables
+    """
+
+    def __init__(self,
+                 module,
+                 optimizer: torch.optim.Optimizer,
+                 initial_scale: float = 32768,
+                 min_scale: float = 1,
+                 growth_factor: float = 2,
+                 backoff_factor: float = 0.5,
+                 growth_interval: int = 1000,
+                 hysteresis: int = 2,
+                 max_scale: float = 2**24,
+                 max_norm: float = 0.0,
+                 norm_type: float = 2.0,
+                 init_step=False):
+        self.optim = optimizer
+        for attr in ('param_chunk_group', 'optim_chunk_group', 'fetcher', 'use_amp'):
+            assert hasattr(module, attr), f'module lacks {attr}: it is not a chunked module'
+        self.scaled_optimizer = False
+        if type(optimizer) in _AVAIL_OPTIM_LIST:
+            self.scaled_optimizer = True
+
+        self.module = module
+        self.param_chunk_group = module.param_chunk_group
+        self.optim_chunk_group = module.optim_chunk_group
+
+        self.optim_state = OptimState.UNSCALED
+        self.param_to_range: Dict[Parameter, Tuple[int, int]] = dict()
+        self.param_to_optim_chunk: Dict[Parameter, Chunk] = dict()
+        self.param_chunk_set: Set[Chunk] = self.param_chunk_group.fused_chunks.union(
+            self.param_chunk_group.float_chunks)
+        self._param_chunk_list: List[Chunk] = sorted(self.param_chunk_set)
+
+        self.clipping_flag = max_norm > 0.0
+        self.max_norm = max_norm
+        if self.clipping_flag:
+            assert norm_type == 2.0, 'ElixirOptimizer only supports L2 norm now'
+            for param_chunk in self.param_chunk_set:
+                param_chunk.l2_norm_flag = True
+
+        self.__init__optimizer()
+
+        # Grad scaler
+        self.grad_scaler: BaseGradScaler = None
+        if module.use_amp:
+            self.grad_scaler = DynamicGradScaler(initial_scale=initial_scale,
+                                                 min_scale=min_scale,
+                                                 growth_factor=growth_factor,
+                                                 backoff_factor=backoff_factor,
+                                                 growth_interval=growth_interval,
+                                                 hysteresis=hysteresis,
+                                                 max_scale=max_scale)
+        else:
+            self.grad_scaler = ConstantGradScaler(1.0, verbose=False)
+
+        self._binding = None
+        if self.scaled_optimizer:
+            ranges = {
+                fake: (self.param_to_optim_chunk[fake], ) + self.param_to_range[fake] for fake in self.param_to_range
+            }
+            if ranges:
+                self._binding = self.optim.bind_chunks(ranges)
+        self._stats_table = None
+        self._stats_workspace: Dict = {}
+        self._wb_table = None
+        self.last_step_info: Dict = {}
+
+        if init_step:
+            # allocate memory before training
+            self.__zero_step()
+
+    # ------------------------------------------------------------------ torch.optim.Optimizer facade
+
+    @property
+    def param_groups(self):
+        return self.optim.param_groups
+
+    @property
+    def defaults(self):
+        return self.optim.defaults
+
+    @property
+    def state(self):
+        return self.optim.state
+
+    def add_param_group(self, *args, **kwargs):
+        return self.optim.add_param_group(*args, **kwargs)
+
+    def state_dict(self):
+        return self.optim.state_dict()
+
+    def load_state_dict(self, *args, **kwargs):
+        return self.optim.load_state_dict(*args, **kwargs)
+
+    # ------------------------------------------------------------------ set-up
+
+    def __init__optimizer(self):
+        """optimizer.py:238-265: every real parameter becomes a zero-size fake parameter that
+        stands for its slice of this process's shard; group hyper-parameters are untouched."""
+
+        def get_range_pair(local_chunk: Chunk, local_param: Parameter):
+            param_info = local_chunk.tensors_info[local_param]
+            begin = max(0, param_info.offset - local_chunk.shard_begin)
+            end = min(local_chunk.shard_size, param_info.end - local_chunk.shard_begin)
+            return begin, end
+
+        for group in self.param_groups:
+            fake_params_list = list()
+
+            for param in group['params']:
+                if not param.requires_grad:
+                    continue
+
+                param_chunk = self.module.fetcher.get_one_chunk(param)
+                range_pair = get_range_pair(param_chunk, param)
+                if range_pair[0] >= range_pair[1]:
+                    continue
+
+                grad_device = param_chunk.shard.device
+                fake_param = torch.nn.Parameter(torch.empty([0], device=grad_device))
+                self.param_to_optim_chunk[fake_param] = param_chunk.paired_chunk
+                self.param_to_range[fake_param] = range_pair
+
+                fake_params_list.append(fake_param)
+
+            group['params'] = fake_params_list
+
+    def __zero_step(self):
+        """optimizer.py:94-113: one inner step with zero gradients, so that the optimizer state
+        exists before training.  It counts as a step (state['step'] becomes 1) and, with decoupled
+        weight decay, decays the master weights once; the low-precision copy is not refreshed."""
+        if self._binding is not None:
+            self._binding.zero_grads = True
+            try:
+                self.optim.step()
+            finally:
+                self._binding.zero_grads = False
+                self._binding.fused_writeback = False
+        else:
+            for group in self.param_groups:
+                for fake_param in group['params']:
+                    optim_chunk = self.param_to_optim_chunk[fake_param]
+                    begin, end = self.param_to_range[fake_param]
+                    fake_param.data = optim_chunk.shard[begin:end]
+                    fake_param.grad = torch.zeros_like(fake_param.data)
+            self.optim.step()
+        self.zero_grad()
+        self._update_fp16_params(update_flag=False)
+
+    # ------------------------------------------------------------------ pieces of the step
+
+    def _set_grad_ptr(self):
+        """optimizer.py:115-124.  A bound HybridAdam reads gradients and master weights straight
+        from the chunk buffers, so nothing needs to be pointed anywhere."""
+        if self._binding is not None:
+            return
+        for group in self.param_groups:
+            for fake_param in group['params']:
+                optim_chunk = self.param_to_optim_chunk[fake_param]
+                begin, end = self.param_to_range[fake_param]
+                param_chunk = optim_chunk.paired_chunk
+
+                fake_param.data = param_chunk.shard[begin:end]
+                fake_param.grad = fake_param.data
+                fake_param.data = optim_chunk.shard[begin:end]
+
+    def _update_fp16_params(self, update_flag: bool = True):
+        """optimizer.py:126-135: detach the fake parameters and refresh the low-precision shards
+        from the fp32 shards -- unless the fused launch has just done so."""
+        if self._binding is None:
+            none_tensor = torch.empty([0])
+            for group in self.param_groups:
+                for fake_param in group['params']:
+                    assert fake_param.grad is None
+                    fake_param.data = none_tensor.to(fake_param.device)
+
+        if not update_flag:
+            return
+        if self._binding is not None and self._binding.fused_writeback:
+            self._binding.fused_writeback = False
+            for param_chunk in self.param_chunk_set:
+                param_chunk.optim_sync_flag = True
+            return
+        self._writeback_all()
+
+    def _writeback_all(self) -> None:
+        """``optim_update`` for every parameter chunk in one launch."""
+        gpu_chunks = [c for c in self._param_chunk_list if c.shard_device.type == 'cuda']
+        for c in self._param_chunk_list:
+            if c.shard_device.type != 'cuda':
+                c.optim_update()
+        if not gpu_chunks:
+            return
+        if self._wb_table is None:
+            tile = _abi.tile_elems()
+            rows = np.zeros(len(gpu_chunks), dtype=_abi.CHUNK_DTYPE)
+            tiles = 0
+            for i, c in enumerate(gpu_chunks):
+                friend = c.paired_chunk
+                assert friend is not None and not friend.is_replica
+                assert friend.shard_device == c.shard_device
+                rows[i]['lowp_out'] = c.shard.data_ptr()
+                rows[i]['master'] = friend.shard.data_ptr()
+                rows[i]['m'] = friend.shard.data_ptr()
+                rows[i]['v'] = friend.shard.data_ptr()
+                rows[i]['n_alloc'] = c.shard_size
+                rows[i]['n_valid'] = c.n_valid
+                rows[i]['tile_begin'] = tiles
+                tiles += (c.shard_size + tile - 1) // tile
+            code = dtype_code(gpu_chunks[0].chunk_dtype)
+            total_tiles, aligned = _abi.check_tables(rows, None, 0, code, code)
+            self._wb_table = (DeviceTable(rows, gpu_chunks[0].shard_device), total_tiles, aligned, code)
+        table, total_tiles, aligned, code = self._wb_table
+        stream = torch.cuda.current_stream(table.dev.device).cuda_stream
+        _abi.writeback_mt(table.ptr, len(table), total_tiles, code, 0 if aligned else _abi.ELX_FLAG_SCALAR_ONLY, 0,
+                          stream)
+        for c in gpu_chunks:
+            c.optim_sync_flag = True
+
+    def _refresh_chunk_stats(self) -> None:
+        """Flags for every parameter chunk whose gradients landed without them: one launch over
+        the chunk list and one device-to-host copy."""
+        pending = [c for c in self._param_chunk_list if not c._stats_fresh]
+        if not pending:
+            return
+        device = pending[0].shard_device
+        if device.type != 'cuda':
+            raise RuntimeError('gradient flags are computed by the HIP kernels: shards must be on the GPU')
+        ids = tuple(c.chunk_id for c in pending)
+        if self._stats_table is None or self._stats_table[0] != ids:
+            rows = np.zeros(len(pending), dtype=_abi.CHUNK_DTYPE)
+            for i, c in enumerate(pending):
+                rows[i]['grad'] = c.shard.data_ptr()
+                rows[i]['n_alloc'] = c.shard_size
+                rows[i]['n_valid'] = c.n_valid
+            self._stats_table = (ids, rows, DeviceTable(rows, device))
+        _, rows, table = self._stats_table
+        stats = run_grad_stats(rows, dtype_code(pending[0].chunk_dtype), device, table=table,
+                               workspace=self._stats_workspace)
+        for c, rec in zip(pending, stats):
+            c._apply_stats(bool(rec['overflow']), float(rec['sumsq']))
+
+    def _check_overflow(self) -> bool:
+        # calculate the overflow counter
+        overflow_counter = 0
+        for param_chunk in self.param_chunk_set:
+            overflow_counter += int(param_chunk.overflow)
+        return overflow_counter > 0
+
+    def _clear_optim_states(self) -> None:
+        for param_chunk in self.param_chunk_set:
+            param_chunk.overflow = False
+            param_chunk.l2_norm = None
+            param_chunk._stats_fresh = False
+
+    def _calc_global_norm(self) -> float:
+        """optimizer.py:149-164 on one process: the per-group sum passes through a one-element fp32
+        buffer before the square root."""
+        group_to_norm = defaultdict(float)
+        for param_chunk in self.param_chunk_set:
+            assert param_chunk.l2_norm is not None
+            assert not param_chunk.is_replica
+            group_to_norm[param_chunk.torch_pg] += param_chunk.l2_norm
+
+        norm_sqr = 0.0
+        for group, part_norm in group_to_norm.items():
+            norm_sqr += float(np.float32(part_norm))
+
+        global_norm = math.sqrt(norm_sqr)
+        return global_norm
+
+    def _get_combined_scale(self):
+        assert self.optim_state == OptimState.SCALED
+        loss_scale = self.loss_scale
+        self.optim_state = OptimState.UNSCALED
+
+        total_norm = self._calc_global_norm() if self.clipping_flag else None
+        self.last_step_info['total_norm'] = total_norm
+        return calc_combined_scale(loss_scale, total_norm, self.max_norm, self.clipping_flag)
+
+    @property
+    def loss_scale(self):
+        return self.grad_scaler.scale_value
+
+    def zero_grad(self, *args, **kwargs):
+        return self.optim.zero_grad(set_to_none=True)
+
+    # ------------------------------------------------------------------ the step
+
+    def step(self, *args, **kwargs):
+        self._refresh_chunk_stats()
+        self._set_grad_ptr()
+        found_inf = self._check_overflow()
+        self.last_step_info = dict(found_inf=found_inf, combined_scale=None, total_norm=None)
+
+        if found_inf:
+            self.optim_state = OptimState.UNSCALED    # no need to unscale grad
+            self.grad_scaler.update(found_inf)    # update gradient scaler
+            self._clear_optim_states()    # clear chunk states used for optimizer update
+            self.zero_grad()    # reset all gradients
+            self._update_fp16_params()
+            return
+
+        # get combined scale. combined scale = loss scale * clipping norm
+        # so that gradient = gradient / combined scale
+        combined_scale = self._get_combined_scale()
+        self.last_step_info['combined_scale'] = combined_scale
+        self.grad_scaler.update(found_inf)
+        self._clear_optim_states()
+
+        if not self.scaled_optimizer:
+            assert combined_scale == -1, 'You should use an optimizer in the available list:\n' \
+            f'{_AVAIL_OPTIM_LIST}'
+            ret = self.optim.step(*args, **kwargs)
+        else:
+            ret = self.optim.step(div_scale=combined_scale, *args, **kwargs)
+
+        self.zero_grad()
+        self._update_fp16_params()
+        return ret
+
+    def clip_grad_norm(self, model: torch.nn.Module, max_norm: float, norm_type: float = 2.0):
+        raise NotImplementedError
+
+    def backward(self, loss: torch.Tensor):
+        loss = self.loss_scale * loss
+        self.optim_state = OptimState.SCALED
+        self.module.backward(loss)
+
+    def backward_by_grad(self, tensor: torch.Tensor, grad: torch.Tensor):
+        self.optim_state = OptimState.SCALED
+        self.module.backward_by_grad(tensor, grad)
+
+    def mark_gradients_scaled(self) -> None:
+        """For callers that land gradients in the chunk shards themselves (no ``backward`` through
+        this wrapper): declares that the shards now hold gradients scaled by ``loss_scale``."""
+        self.optim_state = OptimState.SCALED

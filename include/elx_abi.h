@@ -1,0 +1,181 @@
+/*
+ * C ABI of libelx_hip.so -- the optimizer-step kernels for gfx950 (MI355X).
+ *
+ * The library implements, over chunk-packed parameters, the device work of the reference's
+ * ElixirOptimizer.step (elixir/wrapper/optimizer.py:192-220):
+ *
+ *   stats     overflow flag and sum of squares of the (still loss-scaled) gradients that sit in
+ *             each low-precision chunk shard;
+ *   update    unscale + Adam/AdamW on the fp32 master, exp_avg and exp_avg_sq held in flat
+ *             per-chunk storage + low-precision writeback, in one pass;
+ *   writeback the low-precision refresh alone (the skip-step branch and state loading).
+ *
+ * Conventions
+ *   - plain C, no C++ or torch types; every pointer in a table is a DEVICE pointer;
+ *   - the caller owns all memory (chunk buffers, tables, workspaces); the library allocates
+ *     nothing and keeps no mutable global state; all entry points are reentrant;
+ *   - all device work is enqueued on the hipStream_t passed as `stream` (NULL = default
+ *     stream) and is asynchronous with respect to the host; borrowed pointers must stay valid
+ *     until that work has completed;
+ *   - every function returns an int: 0 = success, > 0 = a hipError_t raised by a launch,
+ *     < 0 = an ELX_E_* argument error.  An overflow in the gradients is data
+ *     (ElxStats.overflow), never an error.
+ */
+#ifndef ELX_ABI_H
+#define ELX_ABI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ELX_ABI_VERSION 1
+
+/* element types of gradient / low-precision buffers */
+enum { ELX_F32 = 0, ELX_F16 = 1, ELX_BF16 = 2, ELX_NONE = -1 };
+
+/* argument errors */
+enum {
+    ELX_E_NULL = -1,     /* a required pointer is NULL */
+    ELX_E_DTYPE = -2,    /* unknown or unsupported dtype combination */
+    ELX_E_ALIGN = -3,    /* a chunk base pointer is not aligned to its element size */
+    ELX_E_RANGE = -4,    /* begin > end, end > n_alloc, n_valid > n_alloc, bad segment range or hyper index */
+    ELX_E_ORDER = -5,    /* segments of a chunk are not sorted by begin or overlap */
+    ELX_E_TILES = -6,    /* tile_begin / total_tiles disagree with the chunk sizes */
+    ELX_E_SIZE = -7      /* a count is zero or exceeds what a launch can address */
+};
+
+/* flags of elx_adam_step_mt */
+enum {
+    ELX_FLAG_SCALAR_ONLY = 1u    /* take the element-by-element path for every tile (set by the host when
+                                    elx_check_tables reports base pointers that are not 16-byte aligned) */
+};
+
+/*
+ * One flat chunk: the paired low-precision / fp32 shards of the reference's Chunk
+ * (elixir/chunk/core/chunk.py:59-139) plus the flat exp_avg / exp_avg_sq this build keeps beside
+ * the master shard.  `grad` and `lowp_out` may be the same buffer: in the reference the
+ * low-precision parameter shard holds the reduced gradients at step time (chunk.py:313) and is
+ * overwritten with the refreshed parameters afterwards (chunk.py:414).
+ */
+typedef struct ElxChunk {
+    const void *grad;    /* n_alloc elements of the gradient dtype; NULL = gradient is zero */
+    void *lowp_out;      /* n_alloc elements of the low-precision dtype; NULL = no writeback */
+    float *master;       /* n_alloc fp32 master weights */
+    float *m;            /* n_alloc fp32 exp_avg */
+    float *v;            /* n_alloc fp32 exp_avg_sq */
+    uint64_t n_alloc;    /* shard_size: elements allocated, padding included */
+    uint64_t n_valid;    /* elements of the head of the shard that hold tensors (valid_end clipped to n_alloc) */
+    uint64_t tile_begin; /* launch-wide index of this chunk's first tile: sum over earlier chunks of
+                            ceil(n_alloc / elx_tile_elems()) */
+    uint32_t seg_begin;  /* this chunk's segments are segs[seg_begin, seg_end) */
+    uint32_t seg_end;
+} ElxChunk;
+
+/*
+ * One tensor's slice [begin, end) of a chunk -- the (begin, end) pair of
+ * elixir/wrapper/optimizer.py:240-244 -- and the index of the hyper-parameter record it uses.
+ * Elements of a chunk that no segment covers (padding, tensors the optimizer does not own) are
+ * not updated; they still take part in the writeback, as in chunk.py:414.
+ */
+typedef struct ElxSeg {
+    uint64_t begin;
+    uint64_t end;
+    uint32_t hyper;
+    uint32_t reserved;
+} ElxSeg;
+
+/* flags of ElxHyper */
+enum {
+    ELX_HYPER_L2 = 1u,          /* L2 mode: g += l2_wd * p before the moments */
+    ELX_HYPER_LERP_FROM_G = 2u  /* 1-beta1 >= 0.5: m = g + lerp_w*(g-m) with lerp_w = (1-beta1)-1 */
+};
+
+/*
+ * Hyper-parameters of one (param group, step count) pair, narrowed to fp32 on the host from the
+ * float64 values a torch optimizer holds (torch/optim/adam.py:528-545):
+ *   bc1 = 1 - beta1^step, bc2 = 1 - beta2^step (both 1 when bias correction is off)
+ */
+typedef struct ElxHyper {
+    float decay_mul; /* AdamW: (float)(1 - lr*wd); 1.0f when there is no decoupled decay */
+    float l2_wd;     /* L2 mode: (float)wd */
+    float lerp_w;    /* (float)(1-beta1), or that minus 1 when ELX_HYPER_LERP_FROM_G */
+    float beta2;     /* (float)beta2 */
+    float omb2;      /* (float)(1-beta2) */
+    float bc2_sqrt;  /* (float)sqrt(bc2) */
+    float eps;       /* (float)eps */
+    float neg_step;  /* (float)(-(lr/bc1)) */
+    uint32_t flags;
+    uint32_t reserved[3];
+} ElxHyper;
+
+/* Result of the stats pass for one chunk; also the element type of its partials workspace. */
+typedef struct ElxStats {
+    double sumsq;      /* sum over the valid elements of (double)(float)g * (float)g */
+    uint32_t overflow; /* 1 if any valid element is +inf, -inf or NaN */
+    uint32_t reserved;
+} ElxStats;
+
+/* ABI version of the loaded library (ELX_ABI_VERSION). */
+int elx_version(void);
+
+/* Text for a return code of this library (argument errors and hipError_t values). */
+const char *elx_strerror(int code);
+
+/* Elements per tile of the update / writeback launch; ElxChunk.tile_begin is counted in these. */
+uint32_t elx_tile_elems(void);
+
+/* sizeof() of the table records as compiled, for bindings to verify their mirrors. */
+uint32_t elx_sizeof_chunk(void);
+uint32_t elx_sizeof_seg(void);
+uint32_t elx_sizeof_hyper(void);
+uint32_t elx_sizeof_stats(void);
+
+/*
+ * Host-side validation of HOST copies of the tables, to be called once before they are uploaded:
+ * NULL / dtype / range / ordering / tile checks as listed under the ELX_E_* codes.  On success
+ * writes the launch-wide tile count to *total_tiles and to *all_aligned16 whether every non-NULL
+ * base pointer is 16-byte aligned (if not, pass ELX_FLAG_SCALAR_ONLY to the launches).
+ * lowp_dtype may be ELX_NONE when no chunk has a lowp_out buffer.
+ * Replaces the per-tensor asserts and range bookkeeping of optimizer.py:238-265 at the boundary.
+ */
+int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *h_segs, uint32_t n_segs,
+                     uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles,
+                     int *all_aligned16);
+
+/*
+ * Stats pass over grad[0, n_valid) of every chunk: replaces Chunk.set_overflow_flag and
+ * Chunk.set_l2_norm (elixir/chunk/core/chunk.py:214-221) for a whole chunk list in two launches.
+ *   d_partials  workspace of n_chunks * blocks_per_chunk ElxStats records (contents ignored)
+ *   d_stats     n_chunks results; the reduction order is fixed, so results are reproducible
+ *   blocks_per_chunk  1..1024
+ */
+int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
+                      ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream);
+
+/*
+ * Fused update over every chunk: for each element inside a segment
+ *   g = (float)grad; if (div_scale > 0) g /= div_scale;            -- the div_scale of optimizer.py:216
+ *   Adam / AdamW on master, m, v with the segment's ElxHyper;
+ * and for every element of the shard (padding included), when lowp_out is set,
+ *   lowp_out = round-to-nearest-even(master)                       -- chunk.py:414
+ * Replaces the inner optimizer's step over the fake parameters plus Chunk.optim_update.
+ *   max_blocks  0 = one workgroup per tile, otherwise the grid is capped and strides over tiles
+ */
+int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
+                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles, float div_scale,
+                     int grad_dtype, int lowp_dtype, uint32_t flags, uint32_t max_blocks, void *stream);
+
+/*
+ * Low-precision refresh alone: lowp_out[0, n_alloc) = round-to-nearest-even(master) for every
+ * chunk.  The skip-step branch (optimizer.py:196-203 -> chunk.py:403-414) and state loading
+ * (elixir/wrapper/module.py:343) use it.
+ */
+int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles, int lowp_dtype,
+                     uint32_t flags, uint32_t max_blocks, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ELX_ABI_H */

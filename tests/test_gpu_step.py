@@ -1,0 +1,479 @@
+"""Parity of the HIP optimizer-step path with the CPU oracle, through the C ABI, on a real GPU.
+
+Bars (from the task's parity statement):
+  * overflow flag, skip decision, loss-scale trajectory: bit-exact;
+  * fp32 master / exp_avg / exp_avg_sq: within 1e-6 relative;
+  * fp16 / bf16 writeback: within 1 ulp.
+The kernels follow the oracle's op order, so most comparisons are also checked for identical bits.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import elixir_amd as ea
+from elixir_amd import _abi
+from elixir_amd import shapes as S
+from elixir_amd.chunk import run_grad_stats
+from oracle import oracle as O
+
+from helpers import (CODE, assert_close_f32, build_workload, compare_state, from_bits, refresh_oracle_grads, to_np,
+                     ulp_distance)
+
+pytestmark = pytest.mark.gpu
+
+DEV = 'cuda'
+
+
+def tiny_gpt2(n_layer=2, hidden=64, vocab=1000, n_pos=32):
+    return S.gpt2_shapes(n_layer=n_layer, hidden=hidden, vocab=vocab, n_pos=n_pos)
+
+
+def odd_shapes():
+    """Tensor sizes that put segment boundaries at every alignment, including inside 4-element
+    vectors and across tile boundaries."""
+    return [('a', (4097, )), ('b', (3, )), ('c', (5000, 3)), ('d', (1, )), ('e', (8191, )), ('f', (12289, )),
+            ('g', (7, 11)), ('h', (4096, )), ('i', (2, ))]
+
+
+# ------------------------------------------------------------------------------------------------
+# stats pass
+# ------------------------------------------------------------------------------------------------
+
+
+def _stats(t: torch.Tensor, n_valid: int):
+    row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+    row['grad'] = t.data_ptr()
+    row['n_alloc'] = t.numel()
+    row['n_valid'] = n_valid
+    rec = run_grad_stats(row, CODE[t.dtype], t.device)
+    return bool(rec['overflow'][0]), float(rec['sumsq'][0])
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('n', [1, 7, 4095, 8192, 8192 * 4 + 5, 1 << 20, (1 << 22) + 12345])
+def test_stats_matches_oracle(oracle, dtype, n):
+    g = torch.Generator(device=DEV)
+    g.manual_seed(n)
+    x = (torch.randn(n, generator=g, device=DEV) * 3.0).to(dtype)
+    flag, sumsq = _stats(x, n)
+    xn = to_np(x)
+    assert flag == oracle.overflow(xn, CODE[dtype]) == False
+    want = oracle.sumsq(xn, CODE[dtype])
+    assert abs(sumsq - want) <= 1e-6 * want, (sumsq, want)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('bad', [float('inf'), float('-inf'), float('nan')])
+@pytest.mark.parametrize('where', ['first', 'last', 'middle'])
+def test_stats_flags_nonfinite(oracle, dtype, bad, where):
+    n = 70001
+    x = torch.ones(n, device=DEV, dtype=dtype)
+    idx = dict(first=0, last=n - 1, middle=n // 2 + 1)[where]
+    x[idx] = bad
+    flag, _ = _stats(x, n)
+    assert flag is True
+    assert oracle.overflow(to_np(x), CODE[dtype]) is True
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_stats_ignores_padding_and_large_finite(oracle, dtype):
+    """Garbage beyond valid_end must not raise the flag; the largest finite values must not either."""
+    n, valid = 50000, 41234
+    x = torch.zeros(n, device=DEV, dtype=dtype)
+    x[:valid] = torch.finfo(dtype).max if dtype == torch.float16 else 1e18
+    x[valid:] = float('inf')
+    x[valid + 5] = float('nan')
+    flag, sumsq = _stats(x, valid)
+    assert flag is False
+    want = oracle.sumsq(to_np(x)[:valid], CODE[dtype])
+    assert abs(sumsq - want) <= 1e-6 * want
+    flag, _ = _stats(x, valid + 1)
+    assert flag is True
+
+
+def test_stats_quiet_and_signalling_nan_payloads(oracle):
+    bits = np.zeros(9000, dtype=np.uint16)
+    for payload in (0x7C01, 0x7DFF, 0x7E00, 0xFE00, 0xFFFF):
+        b = bits.copy()
+        b[8999] = payload
+        x = from_bits(b, torch.float16, DEV)
+        assert _stats(x, 9000)[0] is True
+    x = from_bits(bits, torch.float16, DEV)
+    assert _stats(x, 9000) == (False, 0.0)
+
+
+def test_stats_zero_valid_elements():
+    x = torch.full((4096, ), float('inf'), device=DEV, dtype=torch.float16)
+    assert _stats(x, 0) == (False, 0.0)
+
+
+def test_stats_unaligned_base(oracle):
+    buf = (torch.randn(100003, device=DEV) * 2).to(torch.float16)
+    x = buf[1:]    # 2-byte aligned only
+    flag, sumsq = _stats(x, x.numel())
+    want = oracle.sumsq(to_np(x), O.F16)
+    assert flag is False and abs(sumsq - want) <= 1e-6 * want
+
+
+def test_stats_multi_chunk_flag_in_later_chunk(oracle):
+    xs = [(torch.randn(30000 + 977 * i, device=DEV)).to(torch.float16) for i in range(5)]
+    xs[3][12345] = float('-inf')
+    rows = np.zeros(len(xs), dtype=_abi.CHUNK_DTYPE)
+    for i, x in enumerate(xs):
+        rows[i]['grad'] = x.data_ptr()
+        rows[i]['n_alloc'] = x.numel()
+        rows[i]['n_valid'] = x.numel() - i
+    rec = run_grad_stats(rows, O.F16, torch.device(DEV, torch.cuda.current_device()))
+    assert list(rec['overflow']) == [0, 0, 0, 1, 0]
+    for i, x in enumerate(xs):
+        if i == 3:
+            continue
+        want = oracle.sumsq(to_np(x)[:x.numel() - i], O.F16)
+        assert abs(rec['sumsq'][i] - want) <= 1e-6 * want
+
+
+def test_stats_is_reproducible():
+    x = (torch.randn((1 << 22) + 3, device=DEV)).to(torch.bfloat16)
+    a = _stats(x, x.numel())
+    for _ in range(3):
+        assert _stats(x, x.numel()) == a
+
+
+# ------------------------------------------------------------------------------------------------
+# plain fp32 Adam on flat parameters (HybridAdam used directly)
+# ------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize('adamw,wd', [(True, 0.0), (True, 0.01), (False, 0.01)])
+@pytest.mark.parametrize('n', [1, 4099, (1 << 20) + 3])
+def test_flat_fp32_adam_matches_oracle_and_torch(oracle, adamw, wd, n):
+    torch.manual_seed(n)
+    p0 = torch.randn(n) * 0.02
+    p = torch.nn.Parameter(p0.clone().to(DEV))
+    opt = ea.HybridAdam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=wd, adamw_mode=adamw)
+    tp = torch.nn.Parameter(p0.clone())
+    topt = (torch.optim.AdamW if adamw else torch.optim.Adam)([tp], lr=1e-3, betas=(0.9, 0.999), eps=1e-8,
+                                                              weight_decay=wd)
+    pn, mn, vn = p0.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for step in range(1, 4):
+        g = torch.randn(n) * 1e-2
+        p.grad = g.to(DEV)
+        opt.step()
+        tp.grad = g.clone()
+        topt.step()
+        oracle.adam(g.numpy().copy(), O.F32, pn, mn, vn, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=wd,
+                    step=step, adamw_mode=adamw)
+        st = opt.state[p]
+        assert st['step'] == step
+        got = dict(p=to_np(p.data), m=to_np(st['exp_avg']), v=to_np(st['exp_avg_sq']))
+        # against the oracle: identical bits
+        for name, want in (('p', pn), ('m', mn), ('v', vn)):
+            assert np.array_equal(got[name].view(np.uint32), want.view(np.uint32)), f'step {step} {name} vs oracle'
+        # against torch's CPU Adam: 1e-6 relative; p needs an absolute floor of one part in 1e6 of
+        # the update size, because p - update cancels for elements near zero
+        tst = topt.state[tp]
+        assert_close_f32(got['p'], tp.data.numpy(), f'step {step} p vs torch', rtol=1e-6, atol=1e-9)
+        assert_close_f32(got['m'], tst['exp_avg'].numpy(), f'step {step} m vs torch', rtol=1e-6, atol=1e-12)
+        assert_close_f32(got['v'], tst['exp_avg_sq'].numpy(), f'step {step} v vs torch', rtol=1e-6, atol=1e-16)
+
+
+def test_flat_fp16_grads_fp32_params(oracle):
+    n = 33333
+    torch.manual_seed(5)
+    p0 = torch.randn(n) * 0.02
+    p = torch.nn.Parameter(p0.clone().to(DEV))
+    opt = ea.HybridAdam([p], lr=2e-3, weight_decay=0.05)
+    g = (torch.randn(n) * 1e-2 * 128).to(torch.float16)
+    p.grad = g.to(DEV)
+    opt.step(div_scale=128.0)
+    pn, mn, vn = p0.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    oracle.adam(to_np(g), O.F16, pn, mn, vn, lr=2e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.05, step=1,
+                adamw_mode=True, div_scale=128.0)
+    assert np.array_equal(to_np(p.data).view(np.uint32), pn.view(np.uint32))
+
+
+def test_first_step_is_sign_descent():
+    """Closed form: with m = v = 0 and step 1, p moves by -lr * g / (|g| + eps) ~ -lr * sign(g)."""
+    n = 10000
+    p = torch.nn.Parameter(torch.zeros(n, device=DEV))
+    opt = ea.HybridAdam([p], lr=1e-3, weight_decay=0.0)
+    g = torch.randn(n, device=DEV)
+    g[::7] = 0.0
+    p.grad = g.clone()
+    opt.step()
+    want = -1e-3 * torch.sign(g)
+    assert torch.allclose(p.data, want, rtol=1e-4, atol=0)
+    assert torch.all(p.data[::7] == 0)
+
+
+# ------------------------------------------------------------------------------------------------
+# the chunked mixed-precision step through ElixirOptimizer
+# ------------------------------------------------------------------------------------------------
+
+
+def _run_and_compare(module, opt, ochunks, dtype, oracle_scaler, *, max_norm=0.0, adamw_mode=True, tag=''):
+    opt.mark_gradients_scaled()
+    opt.step()
+    info = O.reference_step(ochunks, CODE[dtype], oracle_scaler, max_norm=max_norm, adamw_mode=adamw_mode)
+    assert opt.last_step_info['found_inf'] == info['found_inf'], tag
+    assert opt.loss_scale == info['loss_scale'], tag
+    if not info['found_inf']:
+        assert opt.last_step_info['combined_scale'] == info['combined_scale'], tag
+    return info
+
+
+@pytest.mark.parametrize('dtype,loss_scale', [(torch.float16, 64.0), (torch.float16, 65536.0), (torch.bfloat16, 1.0),
+                                              (torch.float32, 1.0)])
+def test_mixed_step_matches_oracle(oracle, dtype, loss_scale):
+    """Config-2 shape in miniature: unscale + overflow check + Adam + writeback, several steps."""
+    kw = dict(initial_scale=loss_scale, hysteresis=1) if dtype == torch.float16 else {}
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=11, loss_scale=loss_scale, **kw)
+    scaler = (O.DynamicGradScalerOracle(initial_scale=loss_scale, min_scale=1, max_scale=2**24, hysteresis=1)
+              if dtype == torch.float16 else O.ConstantGradScalerOracle(1.0))
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(3)
+    for step in range(3):
+        if step:
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (1e-3 * loss_scale)
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+            refresh_oracle_grads(module, ochunks)
+        info = _run_and_compare(module, opt, ochunks, dtype, scaler, tag=f'step {step}')
+        assert info['found_inf'] is False
+        ulp = compare_state(module, opt, ochunks, dtype, tag=f'step {step}')
+        compare_state(module, opt, ochunks, dtype, exact=True, tag=f'step {step} exact')
+        assert ulp == 0
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_odd_boundaries_and_decay_groups(oracle, dtype):
+    """Segments that start and end inside vectors and tiles; two groups with different decay."""
+    module, opt, ochunks = build_workload(odd_shapes(), 20000, dtype, seed=2, loss_scale=8.0 if dtype == torch.float16 else 1.0,
+                                          weight_decay=0.1, **(dict(initial_scale=8.0) if dtype == torch.float16 else {}))
+    scaler = (O.DynamicGradScalerOracle(initial_scale=8.0, min_scale=1, max_scale=2**24)
+              if dtype == torch.float16 else O.ConstantGradScalerOracle())
+    _run_and_compare(module, opt, ochunks, dtype, scaler)
+    compare_state(module, opt, ochunks, dtype, exact=True)
+
+
+@pytest.mark.parametrize('dtype,loss_scale', [(torch.bfloat16, 1.0), (torch.float16, 65536.0)])
+def test_clipped_adamw_step(oracle, dtype, loss_scale):
+    """Config-4/5 shape in miniature: global L2 clip at 1.0 (active: the gradient norm is well above
+    it), AdamW with exempt 1-D tensors.  The combined scale is not a power of two, so the unscale is
+    a true division."""
+    kw = dict(initial_scale=loss_scale) if dtype == torch.float16 else {}
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=4, grad_std=5e-2, loss_scale=loss_scale,
+                                          weight_decay=0.1, max_norm=1.0, **kw)
+    scaler = (O.DynamicGradScalerOracle(initial_scale=loss_scale, min_scale=1, max_scale=2**24)
+              if dtype == torch.float16 else O.ConstantGradScalerOracle())
+    info = _run_and_compare(module, opt, ochunks, dtype, scaler, max_norm=1.0)
+    assert info['total_norm'] / loss_scale > 1.0    # clipping is active
+    # the norm feeds every element through the combined scale: the two sides sum the squares in a
+    # different order, so allow the 1e-6 bar here rather than identical bits
+    assert math.isclose(opt.last_step_info['total_norm'], info['total_norm'], rel_tol=1e-6)
+    compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-11, atol_v=1e-14)
+
+
+def test_clip_inactive_below_threshold(oracle):
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, torch.bfloat16, seed=6, grad_std=1e-6, max_norm=1.0)
+    info = _run_and_compare(module, opt, ochunks, torch.bfloat16, O.ConstantGradScalerOracle(), max_norm=1.0)
+    assert info['combined_scale'] == -1
+    compare_state(module, opt, ochunks, torch.bfloat16, exact=True)
+
+
+@pytest.mark.parametrize('adamw_mode,betas,bias_correction', [(False, (0.9, 0.999), True), (True, (0.4, 0.95), True),
+                                                              (True, (0.9, 0.999), False)])
+def test_l2_mode_low_beta1_and_no_bias_correction(oracle, adamw_mode, betas, bias_correction):
+    module, opt, ochunks = build_workload(tiny_gpt2(n_layer=1), 1 << 16, torch.float16, seed=9, loss_scale=32.0,
+                                          weight_decay=0.01, adamw_mode=adamw_mode, betas=betas, initial_scale=32.0)
+    for group in opt.param_groups:
+        group['bias_correction'] = bias_correction
+    for oc in ochunks:
+        for s in oc.segments:
+            s.bias_correction = bias_correction
+    scaler = O.DynamicGradScalerOracle(initial_scale=32.0, min_scale=1, max_scale=2**24)
+    _run_and_compare(module, opt, ochunks, torch.float16, scaler, adamw_mode=adamw_mode)
+    compare_state(module, opt, ochunks, torch.float16, exact=True)
+
+
+# ------------------------------------------------------------------------------------------------
+# overflow: skip, restore, back off, recover (config 3 in miniature)
+# ------------------------------------------------------------------------------------------------
+
+
+def _poison(module, seed):
+    """About one gradient element per 1e4 becomes +inf / -inf / NaN at seeded positions."""
+    gen = torch.Generator(device='cpu')
+    gen.manual_seed(seed)
+    vals = [float('inf'), float('-inf'), float('nan')]
+    k = 0
+    for pc in module.param_chunks:
+        n = pc.n_valid
+        count = max(1, n // 10000)
+        pos = torch.randperm(n, generator=gen)[:count]
+        for j in pos.tolist():
+            pc.shard[j] = vals[k % 3]
+            k += 1
+
+
+@pytest.mark.parametrize('hysteresis', [1, 2])
+def test_overflow_skips_restores_and_backs_off(oracle, hysteresis):
+    dtype = torch.float16
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=21, loss_scale=64.0, initial_scale=64.0,
+                                          hysteresis=hysteresis)
+    scaler = O.DynamicGradScalerOracle(initial_scale=64.0, min_scale=1, max_scale=2**24, hysteresis=hysteresis)
+    _poison(module, 1)
+    refresh_oracle_grads(module, ochunks)
+    before = [(to_np(pc.paired_chunk.shard), *(to_np(t) for t in opt._binding.moments(pc.paired_chunk)))
+              for pc in module.param_chunks]
+
+    info = _run_and_compare(module, opt, ochunks, dtype, scaler)
+    assert info['found_inf'] is True
+    assert opt.loss_scale == (32.0 if hysteresis == 1 else 64.0)
+    for pc, (p0, m0, v0) in zip(module.param_chunks, before):
+        m, v = opt._binding.moments(pc.paired_chunk)
+        assert np.array_equal(to_np(pc.paired_chunk.shard).view(np.uint32), p0.view(np.uint32))
+        assert np.array_equal(to_np(m).view(np.uint32), m0.view(np.uint32))
+        assert np.array_equal(to_np(v).view(np.uint32), v0.view(np.uint32))
+        # the shard that held the gradients is the cast of the master again
+        assert np.array_equal(to_np(pc.shard), oracle.writeback(p0, O.F16))
+    # no state was created or advanced by the skipped step
+    assert all(st.get('step', 0) == 0 for st in opt.state.values())
+    compare_state(module, opt, ochunks, dtype, exact=True)
+
+    if hysteresis == 2:    # a second overflow in a row does back off
+        _poison(module, 2)
+        refresh_oracle_grads(module, ochunks)
+        info = _run_and_compare(module, opt, ochunks, dtype, scaler)
+        assert info['found_inf'] is True and opt.loss_scale == 32.0
+
+    # clean follow-up step at the reduced scale
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(77)
+    for pc in module.param_chunks:
+        g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (1e-3 * opt.loss_scale)
+        g[pc.utilized_size:] = 0
+        pc.shard.copy_(g.to(dtype))
+    refresh_oracle_grads(module, ochunks)
+    info = _run_and_compare(module, opt, ochunks, dtype, scaler)
+    assert info['found_inf'] is False and info['combined_scale'] == 32.0
+    assert all(st['step'] == 1 for st in opt.state.values())
+    compare_state(module, opt, ochunks, dtype, exact=True)
+
+
+def test_loss_scale_grows_after_interval(oracle):
+    dtype = torch.float16
+    module, opt, ochunks = build_workload(tiny_gpt2(n_layer=1, hidden=16, vocab=64, n_pos=8), 4096, dtype, seed=1,
+                                          loss_scale=4.0, initial_scale=4.0, growth_interval=3, max_scale=16.0)
+    scaler = O.DynamicGradScalerOracle(initial_scale=4.0, min_scale=1, max_scale=16.0, growth_interval=3)
+    seen = []
+    for step in range(10):
+        for pc in module.param_chunks:
+            pc.shard.copy_((torch.randn(pc.shard_size, device=DEV) * 1e-3 * opt.loss_scale).to(dtype))
+        refresh_oracle_grads(module, ochunks)
+        _run_and_compare(module, opt, ochunks, dtype, scaler)
+        seen.append(opt.loss_scale)
+    assert seen == [4.0, 4.0, 8.0, 8.0, 8.0, 16.0, 16.0, 16.0, 16.0, 16.0]
+    compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-11, atol_v=1e-14)
+
+
+def test_padding_garbage_is_ignored_then_overwritten(oracle):
+    dtype = torch.float16
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=8, loss_scale=16.0, initial_scale=16.0)
+    some = False
+    for pc in module.param_chunks:
+        if pc.utilized_size < pc.shard_size:
+            pc.shard[pc.utilized_size:] = float('inf')
+            some = True
+    assert some
+    refresh_oracle_grads(module, ochunks)
+    scaler = O.DynamicGradScalerOracle(initial_scale=16.0, min_scale=1, max_scale=2**24)
+    info = _run_and_compare(module, opt, ochunks, dtype, scaler)
+    assert info['found_inf'] is False
+    compare_state(module, opt, ochunks, dtype, exact=True)
+    for pc in module.param_chunks:
+        assert torch.all(pc.shard[pc.utilized_size:] == 0)
+
+
+def test_init_step_allocates_state_and_counts(oracle):
+    """optimizer.py:94-113: the allocation step runs Adam on zero gradients: step becomes 1,
+    moments stay zero, decoupled decay shrinks the master once, the low-precision copy is untouched."""
+    dtype = torch.float16
+    named = tiny_gpt2(n_layer=1)
+    sr = ea.greedy_search([(n, S.numel(s)) for n, s in named], 1 << 16, dtype)
+    module = ea.ElixirModule(dict(named), sr, dtype=dtype)
+    for pc in module.param_chunks:
+        pc.paired_chunk.shard.normal_(0, 0.02)
+        pc.optim_update()
+    lowp_before = [to_np(pc.shard) for pc in module.param_chunks]
+    master_before = [to_np(pc.paired_chunk.shard) for pc in module.param_chunks]
+    inner = ea.HybridAdam(module.parameters(), lr=1e-2, weight_decay=0.5)
+    opt = ea.ElixirOptimizer(module, inner, init_step=True)
+    assert all(st['step'] == 1 for st in opt.state.values())
+    for pc, lp, mp in zip(module.param_chunks, lowp_before, master_before):
+        m, v = opt._binding.moments(pc.paired_chunk)
+        assert torch.count_nonzero(m) == 0 and torch.count_nonzero(v) == 0
+        assert np.array_equal(to_np(pc.shard), lp)
+        want = mp.copy()
+        used = pc.utilized_size
+        want[:used] = (want[:used] * np.float32(1.0 - 1e-2 * 0.5))
+        assert np.array_equal(to_np(pc.paired_chunk.shard).view(np.uint32), want.view(np.uint32))
+
+
+def test_writeback_matches_oracle_on_special_values(oracle):
+    """Rounding of the low-precision refresh: ties, subnormals, overflow to inf, signed zeros."""
+    for dtype in (torch.float16, torch.bfloat16):
+        rng = np.random.default_rng(3)
+        bits = rng.integers(0, 2**32, size=(1 << 18) + 77, dtype=np.uint32)
+        special = np.array([0x00000000, 0x80000000, 0x33000000, 0x33000001, 0x387FC000, 0x387FE000, 0x477FE000,
+                            0x477FF000, 0x7F7FFFFF, 0x7F800000, 0xFF800000, 0x3F801000, 0x3F803000, 0x3F808000,
+                            0x3F818000, 0x00000001, 0x007FFFFF], dtype=np.uint32)
+        bits[:special.size] = special
+        vals = bits.view(np.float32)
+        nan = np.isnan(vals)
+        sr = ea.greedy_search([('w', vals.size)], vals.size, dtype)
+        module = ea.ElixirModule({'w': (vals.size, )}, sr, dtype=dtype)
+        pc = module.param_chunks[0]
+        pc.paired_chunk.shard.copy_(torch.from_numpy(vals.copy()))
+        pc.optim_update()
+        got = to_np(pc.shard)
+        want = oracle.writeback(vals, CODE[dtype])
+        assert np.array_equal(got[~nan], want[~nan])
+        assert np.all(np.isnan(oracle.lowp_to_f32(got[nan], CODE[dtype])))
+
+
+# ------------------------------------------------------------------------------------------------
+# C ABI argument checking (no kernel is launched by a rejected call)
+# ------------------------------------------------------------------------------------------------
+
+
+def test_abi_rejects_bad_tables():
+    x = torch.zeros(8192, device=DEV)
+    row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+    for f in ('master', 'm', 'v'):
+        row[f] = x.data_ptr()
+    row['n_alloc'] = 8192
+    row['n_valid'] = 8192
+    seg = np.zeros(1, dtype=_abi.SEG_DTYPE)
+    seg[0] = (0, 8192, 0, 0)
+    row['seg_end'] = 1
+    assert _abi.check_tables(row, seg, 1, _abi.ELX_F32, _abi.ELX_NONE) == (2, True)
+
+    def expect(code, chunk=row, segs=seg, n_hypers=1, gd=_abi.ELX_F32, ld=_abi.ELX_NONE):
+        with pytest.raises(_abi.ElxError) as e:
+            _abi.check_tables(chunk, segs, n_hypers, gd, ld)
+        assert e.value.code == code
+
+    bad = row.copy(); bad['master'] = 0; expect(-1, chunk=bad)
+    expect(-2, gd=7)
+    bad = row.copy(); bad['m'] = x.data_ptr() + 2; expect(-3, chunk=bad)
+    bad = row.copy(); bad['n_valid'] = 9000; expect(-4, chunk=bad)
+    s2 = seg.copy(); s2[0] = (0, 9000, 0, 0); expect(-4, segs=s2)
+    s2 = seg.copy(); s2[0] = (0, 8192, 3, 0); expect(-4, segs=s2)
+    two = np.zeros(2, dtype=_abi.SEG_DTYPE); two[0] = (100, 200, 0, 0); two[1] = (150, 300, 0, 0)
+    bad = row.copy(); bad['seg_end'] = 2; expect(-5, chunk=bad, segs=two)
+    bad = row.copy(); bad['tile_begin'] = 1; expect(-6, chunk=bad)
+    bad = row.copy(); bad['n_alloc'] = 0; bad['n_valid'] = 0; expect(-7, chunk=bad, segs=None)
