@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the optimizer step (ElixirOptimizer.step over chunk-packed parameters) on one GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c2]
+
+A step is one full pass of the hot path over one set of synthetic gradients that already sit in
+the low-precision chunk shards: stats launch (overflow flag + sum of squares) -> 16 B/chunk
+device-to-host copy -> host scalars -> fused unscale + AdamW + low-precision writeback launch.
+Step time is host wall-clock between two device synchronisations, so host overhead counts.
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
+BYTES_UPDATE = 28               # per valid element: read g(2)+p,m,v(12); write p,m,v(12)+lowp(2)
+BYTES_STATS = 2                 # per valid element: the compulsory second read of g
+
+
+def cpu_baseline(built, sample_elems: int, steps: int = 3):
+    """The same step as torch CPU ops (the oracle's torch harness) on a bounded sample: the first
+    `sample_elems` elements of chunk 0.  Returns the cpu_baseline object of the JSON line."""
+    from oracle import oracle as O
+    from oracle.torch_ref import TorchCpuStep
+    spec = built.spec
+    pc = built.module.param_chunks[0]
+    oc = pc.paired_chunk
+    n = min(sample_elems, pc.utilized_size)
+    m, v = built.optimizer._binding.moments(oc)
+    master = oc.shard[:n].cpu()
+    g = built.grads[0][:n].cpu()
+    ref = TorchCpuStep(master, spec.dtype, lr=spec.lr, betas=spec.betas, eps=spec.eps, weight_decay=spec.weight_decay,
+                       adamw_mode=spec.adamw_mode, exp_avg=m[:n].cpu(), exp_avg_sq=v[:n].cpu())
+    times = []
+    for i in range(steps + 1):
+        t0 = time.perf_counter()
+        ref.step(g, loss_scale=spec.loss_scale, max_norm=spec.max_norm)
+        times.append(time.perf_counter() - t0)
+    t = float(np.median(times[1:]))
+
+    # the C restatement (OpenMP) on the same sample, for reference
+    code = {torch.float16: O.F16, torch.bfloat16: O.BF16, torch.float32: O.F32}[spec.dtype]
+    gb = g.view(torch.int16).numpy().view(np.uint16).copy() if code != O.F32 else g.numpy().copy()
+    pn, mn, vn = master.numpy().copy(), m[:n].cpu().numpy().copy(), v[:n].cpu().numpy().copy()
+    ctimes = []
+    for i in range(steps + 1):
+        t0 = time.perf_counter()
+        O.overflow(gb, code)
+        O.l2norm_sq_ref(gb, code)
+        O.adam(gb, code, pn, mn, vn, lr=spec.lr, beta1=spec.betas[0], beta2=spec.betas[1], eps=spec.eps,
+               weight_decay=spec.weight_decay, step=i + 1, adamw_mode=spec.adamw_mode, div_scale=spec.loss_scale * 1.5)
+        O.writeback(pn, code)
+        ctimes.append(time.perf_counter() - t0)
+    tc = float(np.median(ctimes[1:]))
+    return {
+        'value': n / t,
+        'unit': 'elements/s',
+        'cores': torch.get_num_threads(),
+        'kind': 'port',
+        'sample': f'first {n} elements of chunk 0 of {spec.name}; torch CPU ops (isinf/isnan, float().norm, '
+                  f'float().div_, torch.optim.AdamW, .to(lowp)); median of {steps} steps after 1 warm-up',
+        'ms_per_step_sample': t * 1e3,
+        'gbps_30B': 30 * n / t / 1e9,
+        'oracle_c_openmp': {'value': n / tc, 'unit': 'elements/s', 'cores': O.num_threads()},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--workload', default='c5', choices=['c2', 'c4', 'c5'])
+    ap.add_argument('--cpu-sample', type=int, default=32 << 20, help='elements of the CPU baseline sample; 0 skips it')
+    ap.add_argument('--max-blocks', type=int, default=0, help='cap on the update grid (0 = one workgroup per tile)')
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print('bench.py measures the optimizer step on ONE GPU (each rank owns whole shards; there is no '
+              'multi-GPU path in this build): run with --gpus 1', file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print('bench.py needs a GPU: the optimizer step has no CPU path', file=sys.stderr)
+        sys.exit(2)
+
+    from elixir_amd import _abi, workloads
+    _abi.load()
+    device = torch.device('cuda', 0)
+    torch.cuda.set_device(device)
+
+    t_build = time.perf_counter()
+    built = workloads.build(args.workload, device)
+    t_build = time.perf_counter() - t_build
+    opt = built.optimizer
+    opt.optim.max_blocks = args.max_blocks
+    n_valid = built.n_valid
+
+    step_s, upd_ms, stats_ms = [], [], []
+    for i in range(args.warmup + args.steps):
+        built.land_gradients()
+        opt.kernel_events = {}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert opt.last_step_info['found_inf'] is False
+        if i >= args.warmup:
+            step_s.append(dt)
+            ev = opt.kernel_events
+            upd_ms.append(ev['update'][0].elapsed_time(ev['update'][1]))
+            stats_ms.append(ev['stats'][0].elapsed_time(ev['stats'][1]))
+    opt.kernel_events = None
+
+    t_step = float(np.mean(step_s))
+    t_upd = float(np.mean(upd_ms)) * 1e-3
+    t_stats = float(np.mean(stats_ms)) * 1e-3
+    upd_gbps = BYTES_UPDATE * n_valid / t_upd / 1e9
+    out = {
+        'metric': 'adam_elements_per_sec',
+        'value': n_valid / t_step,
+        'unit': 'elements/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': t_step * 1e3,
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'f32',
+        'data': 'synthetic',
+        'config': {
+            'workload': built.spec.name + ': ' + built.spec.description,
+            'valid_elements': n_valid,
+            'allocated_elements': built.n_alloc,
+            'chunks': len(built.module.param_chunks),
+            'tensors': len(opt.param_to_range),
+            'loss_scale': built.spec.loss_scale,
+            'combined_scale': opt.last_step_info['combined_scale'],
+            'max_blocks': args.max_blocks,
+        },
+        'step': {
+            'ms_min': float(np.min(step_s)) * 1e3,
+            'ms_median': float(np.median(step_s)) * 1e3,
+            'gbps_30B': (BYTES_UPDATE + BYTES_STATS) * n_valid / t_step / 1e9,
+            'frac_30B': (BYTES_UPDATE + BYTES_STATS) * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
+            'gbps_touch_once_28B': BYTES_UPDATE * n_valid / t_step / 1e9,
+            'frac_touch_once_28B': BYTES_UPDATE * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
+        },
+        'roofline': {
+            'kernel': 'adam_step_kernel',
+            'bound': 'hbm',
+            'achieved': upd_gbps,
+            'peak': HBM_PEAK_GBPS,
+            'unit': 'GB/s',
+            'frac': upd_gbps / HBM_PEAK_GBPS,
+            'traffic': None,
+            'bytes_per_launch': BYTES_UPDATE * n_valid,
+            'ms_per_launch': t_upd * 1e3,
+        },
+        'stats_kernel': {
+            'kernel': 'grad_stats_kernel+stats_finish_kernel',
+            'achieved': BYTES_STATS * n_valid / t_stats / 1e9,
+            'unit': 'GB/s',
+            'frac': BYTES_STATS * n_valid / t_stats / 1e9 / HBM_PEAK_GBPS,
+            'ms_per_launch': t_stats * 1e3,
+        },
+        'build_s': t_build,
+    }
+    if args.cpu_sample > 0:
+        out['cpu_baseline'] = cpu_baseline(built, args.cpu_sample)
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

@@ -76,11 +76,11 @@ def stats_launch_blocks(n_valid_max: int) -> int:
     return int(max(1, min(1024, math.ceil(n_valid_max / 16384))))
 
 
-def run_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.device, table: Optional[DeviceTable] = None,
-                   workspace: Optional[Dict] = None) -> np.ndarray:
-    """Launches the stats pass for the chunks described by ``chunk_rows`` (host table, only grad /
-    n_alloc / n_valid are read) and returns the per-chunk ElxStats records on the host.  One
-    blocking device-to-host copy of 16 bytes per chunk."""
+def launch_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.device,
+                      table: Optional[DeviceTable] = None, workspace: Optional[Dict] = None) -> torch.Tensor:
+    """Enqueues the stats pass for the chunks described by ``chunk_rows`` (host table, only grad /
+    n_alloc / n_valid are read) on the current stream and returns the device bytes that will hold
+    the per-chunk ElxStats records."""
     n = len(chunk_rows)
     if table is None:
         table = DeviceTable(chunk_rows, device)
@@ -93,12 +93,23 @@ def run_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.device
     if buf is None or buf.numel() < need or buf.device != device:
         buf = torch.empty(need, dtype=torch.uint8, device=device)
         workspace['stats'] = buf
+    workspace['stats_table'] = table    # keep the table alive until the launch has run
     d_partials = buf.data_ptr()
     d_stats = d_partials + n * bpc * _abi.STATS_DTYPE.itemsize
     stream = torch.cuda.current_stream(device).cuda_stream
     _abi.grad_stats_mt(table.ptr, n, grad_dtype, bpc, d_partials, d_stats, not aligned, stream)
-    out = buf[n * bpc * _abi.STATS_DTYPE.itemsize:need].cpu().numpy()
-    return out.view(_abi.STATS_DTYPE).copy()
+    return buf[n * bpc * _abi.STATS_DTYPE.itemsize:need]
+
+
+def read_grad_stats(dev_records: torch.Tensor) -> np.ndarray:
+    """One blocking device-to-host copy of 16 bytes per chunk."""
+    return dev_records.cpu().numpy().view(_abi.STATS_DTYPE).copy()
+
+
+def run_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.device, table: Optional[DeviceTable] = None,
+                   workspace: Optional[Dict] = None) -> np.ndarray:
+    """Stats pass + readback: the per-chunk ElxStats records on the host."""
+    return read_grad_stats(launch_grad_stats(chunk_rows, grad_dtype, device, table, workspace))
 
 
 def l2_norm_from_sumsq(sumsq: float) -> float:

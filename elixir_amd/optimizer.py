@@ -29,7 +29,7 @@ import torch
 from torch.nn import Parameter
 
 from . import _abi
-from .chunk import Chunk, DeviceTable, dtype_code, run_grad_stats
+from .chunk import Chunk, DeviceTable, dtype_code, launch_grad_stats, read_grad_stats
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
 from .hybrid_adam import HybridAdam
 
@@ -51,6 +51,26 @@ def calc_combined_scale(loss_scale: float, total_norm, max_norm: float, clipping
     if combined_scale == 1:
         return -1
     return combined_scale
+
+
+class _EventPair:
+    """Context manager that brackets launches with events on the current stream."""
+
+    def __init__(self, sink, key):
+        self.sink, self.key = sink, key
+
+    def __enter__(self):
+        if self.sink is not None:
+            self.begin = torch.cuda.Event(enable_timing=True)
+            self.end = torch.cuda.Event(enable_timing=True)
+            self.begin.record()
+        return self
+
+    def __exit__(self, *exc):
+        if self.sink is not None:
+            self.end.record()
+            self.sink[self.key] = (self.begin, self.end)
+        return False
 
 
 class ElixirOptimizer:
@@ -130,6 +150,9 @@ class ElixirOptimizer:
         self._stats_workspace: Dict = {}
         self._wb_table = None
         self.last_step_info: Dict = {}
+        # when set to a dict, step() records (begin, end) torch.cuda.Event pairs on the launch
+        # stream under the keys 'stats' and 'update' (for per-kernel timing by a benchmark)
+        self.kernel_events = None
 
         if init_step:
             # allocate memory before training
@@ -301,10 +324,15 @@ class ElixirOptimizer:
                 rows[i]['n_valid'] = c.n_valid
             self._stats_table = (ids, rows, DeviceTable(rows, device))
         _, rows, table = self._stats_table
-        stats = run_grad_stats(rows, dtype_code(pending[0].chunk_dtype), device, table=table,
-                               workspace=self._stats_workspace)
+        with self._timed('stats'):
+            records = launch_grad_stats(rows, dtype_code(pending[0].chunk_dtype), device, table=table,
+                                        workspace=self._stats_workspace)
+        stats = read_grad_stats(records)
         for c, rec in zip(pending, stats):
             c._apply_stats(bool(rec['overflow']), float(rec['sumsq']))
+
+    def _timed(self, key: str):
+        return _EventPair(self.kernel_events, key)
 
     def _check_overflow(self) -> bool:
         # calculate the overflow counter
@@ -379,7 +407,8 @@ class ElixirOptimizer:
             f'{_AVAIL_OPTIM_LIST}'
             ret = self.optim.step(*args, **kwargs)
         else:
-            ret = self.optim.step(div_scale=combined_scale, *args, **kwargs)
+            with self._timed('update'):
+                ret = self.optim.step(div_scale=combined_scale, *args, **kwargs)
 
         self.zero_grad()
         self._update_fp16_params()

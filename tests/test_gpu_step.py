@@ -171,12 +171,16 @@ def test_flat_fp32_adam_matches_oracle_and_torch(oracle, adamw, wd, n):
         # against the oracle: identical bits
         for name, want in (('p', pn), ('m', mn), ('v', vn)):
             assert np.array_equal(got[name].view(np.uint32), want.view(np.uint32)), f'step {step} {name} vs oracle'
-        # against torch's CPU Adam: 1e-6 relative; p needs an absolute floor of one part in 1e6 of
-        # the update size, because p - update cancels for elements near zero
+        # against torch's CPU Adam: 1e-6 relative.  Each result is a sum that can cancel (p - update,
+        # m + w*(g - m)), so the bound is relative to the size of the operands: 1e-6 of the step
+        # size lr for p, of the largest gradient for m, of its square for v.  (torch's CPU sqrt is
+        # not correctly rounded for ~0.6% of inputs, which moves p by one ulp now and then.)
         tst = topt.state[tp]
-        assert_close_f32(got['p'], tp.data.numpy(), f'step {step} p vs torch', rtol=1e-6, atol=1e-9)
-        assert_close_f32(got['m'], tst['exp_avg'].numpy(), f'step {step} m vs torch', rtol=1e-6, atol=1e-12)
-        assert_close_f32(got['v'], tst['exp_avg_sq'].numpy(), f'step {step} v vs torch', rtol=1e-6, atol=1e-16)
+        gmax = float(g.abs().max())
+        assert_close_f32(got['p'], tp.data.numpy(), f'step {step} p vs torch', rtol=1e-6, atol=1e-6 * 1e-3)
+        assert_close_f32(got['m'], tst['exp_avg'].numpy(), f'step {step} m vs torch', rtol=1e-6, atol=1e-6 * gmax)
+        assert_close_f32(got['v'], tst['exp_avg_sq'].numpy(), f'step {step} v vs torch', rtol=1e-6,
+                         atol=1e-6 * gmax * gmax)
 
 
 def test_flat_fp16_grads_fp32_params(oracle):
@@ -186,6 +190,7 @@ def test_flat_fp16_grads_fp32_params(oracle):
     p = torch.nn.Parameter(p0.clone().to(DEV))
     opt = ea.HybridAdam([p], lr=2e-3, weight_decay=0.05)
     g = (torch.randn(n) * 1e-2 * 128).to(torch.float16)
+    p.grad_dtype = None    # let an fp32 parameter carry a low-precision gradient
     p.grad = g.to(DEV)
     opt.step(div_scale=128.0)
     pn, mn, vn = p0.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
@@ -220,7 +225,12 @@ def _run_and_compare(module, opt, ochunks, dtype, oracle_scaler, *, max_norm=0.0
     assert opt.last_step_info['found_inf'] == info['found_inf'], tag
     assert opt.loss_scale == info['loss_scale'], tag
     if not info['found_inf']:
-        assert opt.last_step_info['combined_scale'] == info['combined_scale'], tag
+        if info['total_norm'] is None:
+            assert opt.last_step_info['combined_scale'] == info['combined_scale'], tag
+        else:
+            # with clipping the scale carries the gradient norm, which the two sides sum in a
+            # different order (and round to fp32 once, chunk.py:220): 1e-6 relative
+            assert math.isclose(opt.last_step_info['combined_scale'], info['combined_scale'], rel_tol=1e-6), tag
     return info
 
 
