@@ -82,7 +82,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--workload', default='c5', choices=['c2', 'c4', 'c5'])
     ap.add_argument('--cpu-sample', type=int, default=32 << 20, help='elements of the CPU baseline sample; 0 skips it')
-    ap.add_argument('--max-blocks', type=int, default=0, help='cap on the update grid (0 = one workgroup per tile)')
+    ap.add_argument('--blocks-per-cu', type=int, default=0,
+                    help='cap on resident update workgroups per compute unit (0 = library default)')
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -102,7 +103,8 @@ def main():
     built = workloads.build(args.workload, device)
     t_build = time.perf_counter() - t_build
     opt = built.optimizer
-    opt.optim.max_blocks = args.max_blocks
+    opt.optim.blocks_per_cu = args.blocks_per_cu
+    opt.blocks_per_cu = args.blocks_per_cu
     n_valid = built.n_valid
 
     step_s, upd_ms, stats_ms = [], [], []
@@ -147,7 +149,7 @@ def main():
             'tensors': len(opt.param_to_range),
             'loss_scale': built.spec.loss_scale,
             'combined_scale': opt.last_step_info['combined_scale'],
-            'max_blocks': args.max_blocks,
+            'blocks_per_cu': args.blocks_per_cu,
         },
         'step': {
             'ms_min': float(np.min(step_s)) * 1e3,

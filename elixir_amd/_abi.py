@@ -63,13 +63,14 @@ def load() -> ctypes.CDLL:
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
-    L.elx_check_tables.argtypes = [vp, u32, vp, u32, u32, cint, cint, ctypes.POINTER(u64), ctypes.POINTER(cint)]
+    L.elx_check_tables.argtypes = [vp, u32, vp, u32, u32, cint, cint, ctypes.POINTER(u64), ctypes.POINTER(u32),
+                                   ctypes.POINTER(cint)]
     L.elx_grad_stats_mt.restype = cint
     L.elx_grad_stats_mt.argtypes = [vp, u32, cint, u32, vp, vp, cint, vp]
     L.elx_adam_step_mt.restype = cint
-    L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, flt, cint, cint, u32, u32, vp]
+    L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_writeback_mt.restype = cint
-    L.elx_writeback_mt.argtypes = [vp, u32, u64, cint, u32, u32, vp]
+    L.elx_writeback_mt.argtypes = [vp, u32, u64, u32, cint, u32, u32, vp]
 
     if L.elx_version() != ELX_ABI_VERSION:
         raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
@@ -97,18 +98,41 @@ def _np_ptr(a: Optional[np.ndarray]):
     return a.ctypes.data_as(ctypes.c_void_p)
 
 
-def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, grad_dtype: int, lowp_dtype: int):
-    """Validate host tables; returns (total_tiles, all_aligned16)."""
+class TableInfo(tuple):
+    """(total_tiles, uniform_tiles_per_chunk, all_aligned16) as reported by elx_check_tables."""
+    __slots__ = ()
+
+    @property
+    def total_tiles(self) -> int:
+        return self[0]
+
+    @property
+    def uniform_tiles(self) -> int:
+        return self[1]
+
+    @property
+    def aligned(self) -> bool:
+        return self[2]
+
+    @property
+    def flags(self) -> int:
+        return 0 if self[2] else ELX_FLAG_SCALAR_ONLY
+
+
+def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, grad_dtype: int,
+                 lowp_dtype: int) -> TableInfo:
+    """Validate host tables; returns (total_tiles, uniform_tiles_per_chunk, all_aligned16)."""
     assert chunks.dtype == CHUNK_DTYPE
     n_segs = 0 if segs is None else len(segs)
     if n_segs:
         assert segs.dtype == SEG_DTYPE
     tiles = ctypes.c_uint64(0)
+    uniform = ctypes.c_uint32(0)
     aligned = ctypes.c_int(0)
     code = load().elx_check_tables(_np_ptr(chunks), len(chunks), _np_ptr(segs), n_segs, n_hypers, grad_dtype, lowp_dtype,
-                                   ctypes.byref(tiles), ctypes.byref(aligned))
+                                   ctypes.byref(tiles), ctypes.byref(uniform), ctypes.byref(aligned))
     check('elx_check_tables', code)
-    return int(tiles.value), bool(aligned.value)
+    return TableInfo((int(tiles.value), int(uniform.value), bool(aligned.value)))
 
 
 def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_partials: int, d_stats: int,
@@ -118,14 +142,16 @@ def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chun
                                    int(scalar_only), stream))
 
 
-def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int, total_tiles: int,
-                 div_scale: float, grad_dtype: int, lowp_dtype: int, flags: int, max_blocks: int, stream: int) -> None:
+def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int, info: TableInfo,
+                 div_scale: float, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int, stream: int) -> None:
     check('elx_adam_step_mt',
-          load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, total_tiles, div_scale,
-                                  grad_dtype, lowp_dtype, flags, max_blocks, stream))
+          load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles,
+                                  info.uniform_tiles, div_scale, grad_dtype, lowp_dtype, info.flags, blocks_per_cu,
+                                  stream))
 
 
-def writeback_mt(d_chunks: int, n_chunks: int, total_tiles: int, lowp_dtype: int, flags: int, max_blocks: int,
+def writeback_mt(d_chunks: int, n_chunks: int, info: TableInfo, lowp_dtype: int, blocks_per_cu: int,
                  stream: int) -> None:
-    check('elx_writeback_mt', load().elx_writeback_mt(d_chunks, n_chunks, total_tiles, lowp_dtype, flags, max_blocks,
-                                                      stream))
+    check('elx_writeback_mt',
+          load().elx_writeback_mt(d_chunks, n_chunks, info.total_tiles, info.uniform_tiles, lowp_dtype, info.flags,
+                                  blocks_per_cu, stream))

@@ -357,10 +357,10 @@ class Chunk:
             row['n_alloc'] = self.shard_size
             row['n_valid'] = self.n_valid
             code = dtype_code(self.chunk_dtype)
-            tiles, aligned = _abi.check_tables(row, None, 0, code, code)
+            info = _abi.check_tables(row, None, 0, code, code)
             table = DeviceTable(row, self.shard_device)
             stream = torch.cuda.current_stream(self.shard_device).cuda_stream
-            _abi.writeback_mt(table.ptr, 1, tiles, code, 0 if aligned else _abi.ELX_FLAG_SCALAR_ONLY, 0, stream)
+            _abi.writeback_mt(table.ptr, 1, info, code, 0, stream)
             # keep the table alive until the launch has consumed it
             self._workspace['wb_table'] = table
             self.optim_sync_flag = True

@@ -1,14 +1,27 @@
 // Optimizer-step kernels for gfx950 (MI355X) behind the C ABI of include/elx_abi.h.
 //
-// All three passes are streaming, HBM-bound element-wise work; there is no contraction, so no
-// MFMA.  What matters is: 128-bit accesses that a wavefront issues fully coalesced, enough
-// independent loads in flight per lane, no re-reads, and one launch for the whole chunk list.
+// All passes are streaming, HBM-bound element-wise work; there is no contraction, so no MFMA.
 //
 //   grad_stats_kernel   one read of the low-precision gradients -> overflow flag + sum of squares
 //                       per chunk (fp32 per-lane partials over 32-128 elements, flushed into an
 //                       fp64 accumulator; wave shuffle -> LDS -> one partial per workgroup;
 //                       a second tiny launch folds the partials in a fixed order)
 //   adam_step_kernel    unscale + Adam/AdamW on master/m/v + low-precision writeback, tile by tile
+//
+// Shape of the update launch, as measured on MI355X.  The update moves 14 B in and 14 B out per
+// element over four in-place regions.  HBM serves such a read/write mix best when the set of
+// addresses in flight is a tight, orderly moving window that is only just deep enough to cover
+// the memory latency; deeper queues cost bandwidth (full occupancy: ~5.5 TB/s; 40-60 KB in flight
+// per compute unit: 6.2-6.5 TB/s; a plain copy peaks at ~6.65 TB/s the same way, write-only traffic
+// falls from 7.2 to 6.2 TB/s between a shallow and a full queue).  Hence:
+//   * one wavefront per workgroup, one 512-element tile per workgroup, tiles handed out in
+//     address order by the dispatcher (a persistent grid-stride loop is much slower here);
+//   * every access is a fully coalesced 128-bit (fp32) / 64-bit (16-bit types) per-lane access,
+//     so one wavefront instruction covers one contiguous 1 KiB / 512 B span;
+//   * the number of resident workgroups per compute unit is capped through a dynamic LDS
+//     reservation (default 10: each wavefront spends part of its short life fetching its chunk
+//     record, so about 8 of them have memory requests in flight), not by the register file;
+//   * loads carry the non-temporal hint, stores go out non-temporal at agent scope.
 //
 // Arithmetic contract (what the parity tests pin): fp32 throughout, IEEE division and square
 // root, the only fused multiply-adds are the three written as fmaf(); compile with
@@ -21,16 +34,22 @@
 
 namespace {
 
-constexpr int kThreads = 256;                               // 4 wavefronts of 64
-constexpr int kVec = 4;                                     // elements per lane per access
-constexpr int kUnroll = 4;                                  // independent accesses per lane per stream
-constexpr uint32_t kSpan = kThreads * kVec;                 // elements one access of the workgroup covers
-constexpr uint32_t kTile = kSpan * kUnroll;                 // 4096 elements per tile
+constexpr int kWave = 64;                              // one wavefront per update workgroup
+constexpr int kVec = 4;                                // elements per lane per access
+constexpr int kUnroll = 2;                             // independent accesses per lane per stream
+constexpr uint32_t kSpan = kWave * kVec;               // elements one wavefront access covers
+constexpr uint32_t kTile = kSpan * kUnroll;            // 512 elements per tile
+constexpr uint32_t kLdsPerCu = 160u * 1024u;           // gfx950
+constexpr uint32_t kDefaultBlocksPerCu = 10;
+constexpr uint32_t kMinBlocksPerCu = 3;                // keeps the reservation below 64 KiB
+constexpr uint32_t kMaxBlocksPerCu = 32;
+
+constexpr int kStatsThreads = 256;
+constexpr int kStatsUnroll = 4;
 constexpr uint32_t kMaxStatsBlocks = 1024;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
-typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
 
 // ---------------------------------------------------------------------------------------------
 // element codecs
@@ -78,10 +97,43 @@ template <typename V>
 __device__ __forceinline__ V ld_stream(const V *p) {
     return __builtin_nontemporal_load(p);
 }
-template <typename V>
-__device__ __forceinline__ void st_stream(V *p, V x) {
-    __builtin_nontemporal_store(x, p);
+
+// Tile-local buffer addressing for the update launch: each stream of a tile is described by a
+// raw buffer resource (uniform base = start of the tile, extent = the tile), and a lane addresses
+// it with a 32-bit byte offset.  Loads carry the non-temporal hint; stores go out non-temporal at
+// agent scope.  Being compiler intrinsics (not inline assembly) they keep the compiler's own
+// hazard and wait-count handling.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+constexpr int kAuxLoad = 2;          // nt
+constexpr int kAuxStore = 2 | 16;    // nt | sc1
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
+
+template <typename V>
+struct TileIo;
+
+template <>
+struct TileIo<f32x4> {
+    static __device__ __forceinline__ f32x4 load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxLoad));
+    }
+    static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, f32x4 x) {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, (int)off, 0, kAuxStore);
+    }
+};
+
+template <>
+struct TileIo<u16x4> {
+    static __device__ __forceinline__ u16x4 load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_bit_cast(u16x4, __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kAuxLoad));
+    }
+    static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, u16x4 x) {
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, x), r, (int)off, 0, kAuxStore);
+    }
+};
 
 // ---------------------------------------------------------------------------------------------
 // the update of one element
@@ -134,93 +186,33 @@ __device__ __forceinline__ void adam_elem(float g, float &p, float &m, float &v,
 // fused update + writeback
 // ---------------------------------------------------------------------------------------------
 
-// Whole tile inside one segment: every stream moves as 128-bit (fp32) / 64-bit (16-bit types)
-// accesses, lane l of access u touching elements [u*kSpan + 4l, u*kSpan + 4l + 4) so that each
-// wavefront instruction covers one contiguous 1 KiB (fp32) or 512 B (16-bit) span.
-template <int GD, int LD, bool NT>
-__device__ __forceinline__ void tile_update_vec(const ElxChunk &c, uint64_t base, const Hyper &h, const Unscale &us) {
-    typedef typename Elem<GD>::vec4 gvec;
-    const uint32_t lane_off = threadIdx.x * kVec;
-    const gvec *gp = c.grad ? reinterpret_cast<const gvec *>(reinterpret_cast<const typename Elem<GD>::scalar *>(c.grad) + base + lane_off) : nullptr;
-    f32x4 *pp = reinterpret_cast<f32x4 *>(c.master + base + lane_off);
-    f32x4 *mp = reinterpret_cast<f32x4 *>(c.m + base + lane_off);
-    f32x4 *vp = reinterpret_cast<f32x4 *>(c.v + base + lane_off);
-    constexpr uint32_t kStride = kSpan / kVec;    // in vec4 units
-
-    gvec G[kUnroll];
-    f32x4 P[kUnroll], M[kUnroll], V[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        if (gp) G[u] = NT ? ld_stream(gp + u * kStride) : gp[u * kStride];
-        P[u] = NT ? ld_stream(pp + u * kStride) : pp[u * kStride];
-        M[u] = NT ? ld_stream(mp + u * kStride) : mp[u * kStride];
-        V[u] = NT ? ld_stream(vp + u * kStride) : vp[u * kStride];
-    }
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-        for (int k = 0; k < kVec; ++k) {
-            float g = gp ? Elem<GD>::to_f32(G[u][k]) : 0.0f;
-            float p = P[u][k], m = M[u][k], v = V[u][k];
-            adam_elem(g, p, m, v, h, us);
-            P[u][k] = p;
-            M[u][k] = m;
-            V[u][k] = v;
-        }
-    }
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        if (NT) {
-            st_stream(pp + u * kStride, P[u]);
-            st_stream(mp + u * kStride, M[u]);
-            st_stream(vp + u * kStride, V[u]);
-        } else {
-            pp[u * kStride] = P[u];
-            mp[u * kStride] = M[u];
-            vp[u * kStride] = V[u];
-        }
-    }
-    if constexpr (LD != ELX_NONE) {
-        if (c.lowp_out) {
-            typedef typename Elem<LD>::vec4 lvec;
-            lvec *lp = reinterpret_cast<lvec *>(reinterpret_cast<typename Elem<LD>::scalar *>(c.lowp_out) + base + lane_off);
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                lvec L;
-#pragma unroll
-                for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
-                if (NT)
-                    st_stream(lp + u * kStride, L);
-                else
-                    lp[u * kStride] = L;
-            }
-        }
-    }
-}
-
-// Whole tile outside every segment (padding, or the writeback-only launch): refresh only.
-template <int LD, bool NT>
-__device__ __forceinline__ void tile_refresh_vec(const ElxChunk &c, uint64_t base) {
+template <int LD>
+__device__ __forceinline__ void store_lowp_vec(const ElxChunk &c, uint64_t base, const f32x4 (&P)[kUnroll]) {
     if constexpr (LD != ELX_NONE) {
         if (!c.lowp_out) return;
         typedef typename Elem<LD>::vec4 lvec;
-        const uint32_t lane_off = threadIdx.x * kVec;
-        const f32x4 *pp = reinterpret_cast<const f32x4 *>(c.master + base + lane_off);
-        lvec *lp = reinterpret_cast<lvec *>(reinterpret_cast<typename Elem<LD>::scalar *>(c.lowp_out) + base + lane_off);
-        constexpr uint32_t kStride = kSpan / kVec;
-        f32x4 P[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) P[u] = NT ? ld_stream(pp + u * kStride) : pp[u * kStride];
+        typedef typename Elem<LD>::scalar lscalar;
+        const __amdgpu_buffer_rsrc_t lr = tile_rsrc(reinterpret_cast<lscalar *>(c.lowp_out) + base, kTile * sizeof(lscalar));
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             lvec L;
 #pragma unroll
             for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
-            if (NT)
-                st_stream(lp + u * kStride, L);
-            else
-                lp[u * kStride] = L;
+            TileIo<lvec>::store(lr, (threadIdx.x + u * kWave) * sizeof(lvec), L);
         }
+    }
+}
+
+// Whole tile outside the valid head of the shard (padding), or the writeback-only launch.
+template <int LD>
+__device__ __forceinline__ void tile_refresh_vec(const ElxChunk &c, uint64_t base) {
+    if constexpr (LD != ELX_NONE) {
+        if (!c.lowp_out) return;
+        const __amdgpu_buffer_rsrc_t pr = tile_rsrc(c.master + base, kTile * sizeof(float));
+        f32x4 P[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) P[u] = TileIo<f32x4>::load(pr, (threadIdx.x + u * kWave) * sizeof(f32x4));
+        store_lowp_vec<LD>(c, base, P);
     }
 }
 
@@ -233,7 +225,7 @@ __device__ __forceinline__ void tile_scalar(const ElxChunk &c, uint64_t base, ui
                                             const Unscale &us, bool refresh_only) {
     typedef typename Elem<GD>::scalar gscalar;
     const gscalar *grad = reinterpret_cast<const gscalar *>(c.grad);
-    for (uint32_t i = threadIdx.x; i < tile_n; i += kThreads) {
+    for (uint32_t i = threadIdx.x; i < tile_n; i += kWave) {
         const uint64_t e = base + i;
         float p = c.master[e];
         if (!refresh_only) {
@@ -255,13 +247,45 @@ __device__ __forceinline__ void tile_scalar(const ElxChunk &c, uint64_t base, ui
     }
 }
 
-template <int GD, int LD, bool NT>
-__global__ __launch_bounds__(kThreads) void adam_step_kernel(const ElxChunk *__restrict__ chunks, uint32_t n_chunks,
-                                                             const ElxSeg *__restrict__ segs,
-                                                             const ElxHyper *__restrict__ hypers, uint64_t total_tiles,
-                                                             Unscale us, uint32_t scalar_only, uint32_t refresh_only) {
-    for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-        // chunk that owns tile t: the last one whose tile_begin is <= t (uniform -> scalar loads)
+// Fetches a whole chunk record with one round trip of scalar loads.  Left to itself the compiler
+// loads the fields in the order the branches below first need them, which costs three dependent
+// trips to the scalar cache before the first vector load of the tile can be issued.
+__device__ __forceinline__ ElxChunk load_chunk_row(const ElxChunk *__restrict__ row) {
+    const uint64_t *w = reinterpret_cast<const uint64_t *>(row);
+    uint64_t w0 = w[0], w1 = w[1], w2 = w[2], w3 = w[3], w4 = w[4], w5 = w[5], w6 = w[6], w7 = w[7], w8 = w[8];
+    asm volatile("" : "+s"(w0), "+s"(w1), "+s"(w2), "+s"(w3), "+s"(w4), "+s"(w5), "+s"(w6), "+s"(w7), "+s"(w8));
+    ElxChunk c;
+    c.grad = reinterpret_cast<const void *>(w0);
+    c.lowp_out = reinterpret_cast<void *>(w1);
+    c.master = reinterpret_cast<float *>(w2);
+    c.m = reinterpret_cast<float *>(w3);
+    c.v = reinterpret_cast<float *>(w4);
+    c.n_alloc = w5;
+    c.n_valid = w6;
+    c.tile_begin = w7;
+    c.seg_begin = (uint32_t)w8;
+    c.seg_end = (uint32_t)(w8 >> 32);
+    return c;
+}
+static_assert(sizeof(ElxChunk) == 72, "load_chunk_row reads nine 64-bit words");
+
+extern __shared__ char elx_occupancy_reservation[];    // never touched: it only caps residency
+
+template <int GD, int LD>
+__global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks, uint32_t n_chunks,
+                                                          const ElxSeg *__restrict__ segs,
+                                                          const ElxHyper *__restrict__ hypers,
+                                                          uint32_t uniform_tiles_per_chunk, Unscale us,
+                                                          uint32_t scalar_only, uint32_t refresh_only) {
+    // chunk that owns this tile: with a uniform tile count per chunk the grid is (tiles, chunks)
+    // and nothing has to be looked up; otherwise the grid is flat and the owner is the last chunk
+    // whose tile_begin is <= the tile index (all uniform -> scalar loads)
+    uint32_t ci, local_tile;
+    if (uniform_tiles_per_chunk) {
+        ci = blockIdx.y;
+        local_tile = blockIdx.x;
+    } else {
+        const uint32_t t = blockIdx.x;
         uint32_t lo = 0, hi = n_chunks;
         while (hi - lo > 1) {
             const uint32_t mid = (lo + hi) >> 1;
@@ -270,42 +294,87 @@ __global__ __launch_bounds__(kThreads) void adam_step_kernel(const ElxChunk *__r
             else
                 hi = mid;
         }
-        const ElxChunk c = chunks[lo];
-        const uint64_t base = (t - c.tile_begin) * kTile;
-        if (base >= c.n_alloc) continue;    // cannot happen with checked tables
-        const uint64_t left = c.n_alloc - base;
-        const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
-        const bool whole = (tile_n == kTile) && !scalar_only;
+        ci = lo;
+        local_tile = t - (uint32_t)chunks[lo].tile_begin;
+    }
+    const ElxChunk c = load_chunk_row(chunks + ci);
+    const uint64_t base = (uint64_t)local_tile * kTile;
+    if (base >= c.n_alloc) return;    // cannot happen with checked tables
+    const uint64_t left = c.n_alloc - base;
+    const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
+    const bool whole = (tile_n == kTile) && !scalar_only;
 
-        if (refresh_only) {
-            if (whole)
-                tile_refresh_vec<LD, NT>(c, base);
-            else
-                tile_scalar<GD, LD>(c, base, tile_n, 0, segs, hypers, us, true);
-            continue;
-        }
+    if (refresh_only || base >= c.n_valid) {    // nothing to update in this tile
+        if (whole)
+            tile_refresh_vec<LD>(c, base);
+        else
+            tile_scalar<GD, LD>(c, base, tile_n, 0, segs, hypers, us, true);
+        return;
+    }
 
-        // first segment of the chunk that ends after the start of the tile
-        uint32_t s = c.seg_begin, s_hi = c.seg_end;
-        while (s < s_hi) {
-            const uint32_t mid = (s + s_hi) >> 1;
-            if (segs[mid].end > base)
-                s_hi = mid;
-            else
-                s = mid + 1;
+    typedef typename Elem<GD>::vec4 gvec;
+    typedef typename Elem<GD>::scalar gscalar;
+    gvec G[kUnroll];
+    f32x4 P[kUnroll], M[kUnroll], V[kUnroll];
+    const __amdgpu_buffer_rsrc_t pr = tile_rsrc(c.master + base, kTile * sizeof(float));
+    const __amdgpu_buffer_rsrc_t mr = tile_rsrc(c.m + base, kTile * sizeof(float));
+    const __amdgpu_buffer_rsrc_t vr = tile_rsrc(c.v + base, kTile * sizeof(float));
+    if (whole) {
+        // issue every load of the tile before looking at the segment table: the table lookups
+        // below then overlap the memory latency
+        if (c.grad) {
+            const __amdgpu_buffer_rsrc_t gr = tile_rsrc(reinterpret_cast<const gscalar *>(c.grad) + base, kTile * sizeof(gscalar));
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) G[u] = TileIo<gvec>::load(gr, (threadIdx.x + u * kWave) * sizeof(gvec));
         }
-        const bool has = s < c.seg_end;
-        const uint64_t sb = has ? segs[s].begin : ~0ull;
-        const uint64_t se = has ? segs[s].end : 0ull;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t off = (threadIdx.x + u * kWave) * sizeof(f32x4);
+            P[u] = TileIo<f32x4>::load(pr, off);
+            M[u] = TileIo<f32x4>::load(mr, off);
+            V[u] = TileIo<f32x4>::load(vr, off);
+        }
+    }
 
-        if (whole && has && sb <= base && se >= base + kTile) {
-            const Hyper h = load_hyper(hypers + segs[s].hyper);
-            tile_update_vec<GD, LD, NT>(c, base, h, us);
-        } else if (whole && (!has || sb >= base + kTile)) {
-            tile_refresh_vec<LD, NT>(c, base);
-        } else {
-            tile_scalar<GD, LD>(c, base, tile_n, s, segs, hypers, us, false);
+    // first segment of the chunk that ends after the start of the tile
+    uint32_t s = c.seg_begin, s_hi = c.seg_end;
+    while (s < s_hi) {
+        const uint32_t mid = (s + s_hi) >> 1;
+        if (segs[mid].end > base)
+            s_hi = mid;
+        else
+            s = mid + 1;
+    }
+    const bool has = s < c.seg_end;
+    const uint64_t sb = has ? segs[s].begin : ~0ull;
+    const uint64_t se = has ? segs[s].end : 0ull;
+
+    if (whole && has && sb <= base && se >= base + kTile) {
+        const Hyper h = load_hyper(hypers + segs[s].hyper);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+            for (int k = 0; k < kVec; ++k) {
+                float g = c.grad ? Elem<GD>::to_f32(G[u][k]) : 0.0f;
+                float p = P[u][k], m = M[u][k], v = V[u][k];
+                adam_elem(g, p, m, v, h, us);
+                P[u][k] = p;
+                M[u][k] = m;
+                V[u][k] = v;
+            }
         }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t off = (threadIdx.x + u * kWave) * sizeof(f32x4);
+            TileIo<f32x4>::store(pr, off, P[u]);
+            TileIo<f32x4>::store(mr, off, M[u]);
+            TileIo<f32x4>::store(vr, off, V[u]);
+        }
+        store_lowp_vec<LD>(c, base, P);
+    } else if (whole && (!has || sb >= base + kTile)) {
+        store_lowp_vec<LD>(c, base, P);    // inside the valid head but owned by no segment
+    } else {
+        tile_scalar<GD, LD>(c, base, tile_n, s, segs, hypers, us, false);
     }
 }
 
@@ -321,8 +390,8 @@ __device__ __forceinline__ double wave_sum(double x) {
 
 // Folds (sum, flag) over the workgroup; the result is valid in thread 0.  Fixed order.
 __device__ __forceinline__ void block_fold(double &sum, uint32_t &flag) {
-    __shared__ double s_sum[kThreads / 64];
-    __shared__ uint32_t s_flag[kThreads / 64];
+    __shared__ double s_sum[kStatsThreads / 64];
+    __shared__ uint32_t s_flag[kStatsThreads / 64];
     sum = wave_sum(sum);
     flag = __ballot(flag != 0) != 0ull ? 1u : 0u;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -334,7 +403,7 @@ __device__ __forceinline__ void block_fold(double &sum, uint32_t &flag) {
     if (threadIdx.x == 0) {
         double t = 0.0;
         uint32_t f = 0;
-        for (int w = 0; w < kThreads / 64; ++w) {
+        for (int w = 0; w < kStatsThreads / 64; ++w) {
             t += s_sum[w];
             f |= s_flag[w];
         }
@@ -350,12 +419,13 @@ __device__ __forceinline__ void stats_elem(float x, float &acc, float &poison) {
 }
 
 template <int GD>
-__global__ __launch_bounds__(kThreads) void grad_stats_kernel(const ElxChunk *__restrict__ chunks, uint32_t bpc,
-                                                              ElxStats *__restrict__ partials, uint32_t scalar_only) {
+__global__ __launch_bounds__(kStatsThreads) void grad_stats_kernel(const ElxChunk *__restrict__ chunks, uint32_t bpc,
+                                                                   ElxStats *__restrict__ partials,
+                                                                   uint32_t scalar_only) {
     typedef typename Elem<GD>::scalar gscalar;
     constexpr uint32_t kEpl = 16 / sizeof(gscalar);    // elements per lane per 128-bit load
-    constexpr uint32_t kSSpan = kThreads * kEpl;
-    constexpr uint32_t kSTile = kSSpan * kUnroll;
+    constexpr uint32_t kSSpan = kStatsThreads * kEpl;
+    constexpr uint32_t kSTile = kSSpan * kStatsUnroll;
     typedef gscalar gvec __attribute__((ext_vector_type(kEpl)));
 
     const ElxChunk c = chunks[blockIdx.y];
@@ -370,17 +440,18 @@ __global__ __launch_bounds__(kThreads) void grad_stats_kernel(const ElxChunk *__
         float acc = 0.0f;
         if (base + kSTile <= n && !scalar_only) {
             const gvec *gp = reinterpret_cast<const gvec *>(g + base) + threadIdx.x;
-            gvec G[kUnroll];
+            gvec G[kStatsUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) G[u] = ld_stream(gp + u * kThreads);
+            for (int u = 0; u < kStatsUnroll; ++u) G[u] = ld_stream(gp + u * kStatsThreads);
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kStatsUnroll; ++u)
 #pragma unroll
                 for (uint32_t k = 0; k < kEpl; ++k) stats_elem(Elem<GD>::to_f32(G[u][k]), acc, poison);
         } else {
             const uint64_t left = n - base;
             const uint32_t tile_n = left < kSTile ? (uint32_t)left : kSTile;
-            for (uint32_t i = threadIdx.x; i < tile_n; i += kThreads) stats_elem(Elem<GD>::to_f32(g[base + i]), acc, poison);
+            for (uint32_t i = threadIdx.x; i < tile_n; i += kStatsThreads)
+                stats_elem(Elem<GD>::to_f32(g[base + i]), acc, poison);
         }
         sum += (double)acc;
     }
@@ -395,12 +466,12 @@ __global__ __launch_bounds__(kThreads) void grad_stats_kernel(const ElxChunk *__
     }
 }
 
-__global__ __launch_bounds__(kThreads) void stats_finish_kernel(const ElxStats *__restrict__ partials, uint32_t bpc,
-                                                                ElxStats *__restrict__ out) {
+__global__ __launch_bounds__(kStatsThreads) void stats_finish_kernel(const ElxStats *__restrict__ partials,
+                                                                     uint32_t bpc, ElxStats *__restrict__ out) {
     const ElxStats *row = partials + (uint64_t)blockIdx.x * bpc;
     double sum = 0.0;
     uint32_t flag = 0;
-    for (uint32_t i = threadIdx.x; i < bpc; i += kThreads) {
+    for (uint32_t i = threadIdx.x; i < bpc; i += kStatsThreads) {
         sum += row[i].sumsq;
         flag |= row[i].overflow;
     }
@@ -430,24 +501,31 @@ bool exact_reciprocal(float s) {
     return (u >> 31) == 0 && man == 0 && exp >= 1 && exp <= 252;
 }
 
+// dynamic LDS bytes that let exactly `blocks_per_cu` update workgroups share a compute unit
+int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes) {
+    if (blocks_per_cu == 0) blocks_per_cu = kDefaultBlocksPerCu;
+    if (blocks_per_cu < kMinBlocksPerCu || blocks_per_cu > kMaxBlocksPerCu) return ELX_E_SIZE;
+    *lds_bytes = (kLdsPerCu / blocks_per_cu) & ~255u;
+    return 0;
+}
+
 template <int GD, int LD>
-int launch_step(bool nt, dim3 grid, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks, const ElxSeg *segs,
-                const ElxHyper *hypers, uint64_t total_tiles, Unscale us, uint32_t scalar_only, uint32_t refresh_only) {
-    if (nt)
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true>), grid, dim3(kThreads), 0, st, chunks, n_chunks, segs, hypers,
-                           total_tiles, us, scalar_only, refresh_only);
-    else
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false>), grid, dim3(kThreads), 0, st, chunks, n_chunks, segs, hypers,
-                           total_tiles, us, scalar_only, refresh_only);
+int launch_step(uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
+                const ElxSeg *segs, const ElxHyper *hypers, uint32_t uniform_tiles, Unscale us, uint32_t scalar_only,
+                uint32_t refresh_only) {
+    const dim3 grid = uniform_tiles ? dim3(uniform_tiles, n_chunks) : dim3(tiles);
+    hipLaunchKernelGGL((adam_step_kernel<GD, LD>), grid, dim3(kWave), lds, st, chunks, n_chunks, segs, hypers,
+                       uniform_tiles, us, scalar_only, refresh_only);
     return (int)hipGetLastError();
 }
 
-int dispatch_step(int gd, int ld, bool nt, dim3 grid, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
-                  const ElxSeg *segs, const ElxHyper *hypers, uint64_t total_tiles, Unscale us, uint32_t scalar_only,
-                  uint32_t refresh_only) {
-#define ELX_CASE(G, L)                                                                                          \
-    if (gd == G && ld == L)                                                                                     \
-        return launch_step<G, L>(nt, grid, st, chunks, n_chunks, segs, hypers, total_tiles, us, scalar_only, refresh_only);
+int dispatch_step(int gd, int ld, uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks,
+                  uint32_t n_chunks, const ElxSeg *segs, const ElxHyper *hypers, uint32_t uniform_tiles, Unscale us,
+                  uint32_t scalar_only, uint32_t refresh_only) {
+#define ELX_CASE(G, L)                                                                                         \
+    if (gd == G && ld == L)                                                                                    \
+        return launch_step<G, L>(tiles, lds, st, chunks, n_chunks, segs, hypers, uniform_tiles, us, scalar_only, \
+                                 refresh_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -456,13 +534,6 @@ int dispatch_step(int gd, int ld, bool nt, dim3 grid, hipStream_t st, const ElxC
     ELX_CASE(ELX_BF16, ELX_BF16)
 #undef ELX_CASE
     return ELX_E_DTYPE;
-}
-
-dim3 step_grid(uint64_t total_tiles, uint32_t max_blocks) {
-    uint64_t blocks = total_tiles;
-    if (max_blocks && blocks > max_blocks) blocks = max_blocks;
-    if (blocks > 0x7FFFFFFFull) blocks = 0x7FFFFFFFull;
-    return dim3((uint32_t)blocks);
 }
 
 }    // namespace
@@ -483,10 +554,10 @@ const char *elx_strerror(int code) {
         case ELX_E_NULL: return "elx: a required pointer is NULL";
         case ELX_E_DTYPE: return "elx: unknown or unsupported dtype combination";
         case ELX_E_ALIGN: return "elx: a chunk base pointer is not aligned to its element size";
-        case ELX_E_RANGE: return "elx: a range is out of bounds (begin > end, end > n_alloc, n_valid > n_alloc, segment range or hyper index)";
+        case ELX_E_RANGE: return "elx: a range is out of bounds (begin >= end, end > n_valid, n_valid > n_alloc, segment range or hyper index)";
         case ELX_E_ORDER: return "elx: segments of a chunk are not sorted or overlap";
         case ELX_E_TILES: return "elx: tile_begin / total_tiles disagree with the chunk sizes";
-        case ELX_E_SIZE: return "elx: a count is zero or exceeds what a launch can address";
+        case ELX_E_SIZE: return "elx: a count is zero, out of its allowed range, or exceeds what a launch can address";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -494,16 +565,19 @@ const char *elx_strerror(int code) {
 }
 
 int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *h_segs, uint32_t n_segs,
-                     uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles, int *all_aligned16) {
-    if (!h_chunks || !total_tiles || !all_aligned16 || (n_segs && !h_segs)) return ELX_E_NULL;
+                     uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles,
+                     uint32_t *uniform_tiles_per_chunk, int *all_aligned16) {
+    if (!h_chunks || !total_tiles || !uniform_tiles_per_chunk || !all_aligned16 || (n_segs && !h_segs)) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u) return ELX_E_SIZE;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
     const uintptr_t gmask = elem_size(grad_dtype) - 1;
     uint64_t tiles = 0;
     int aligned = 1;
+    uint64_t uniform = (h_chunks[0].n_alloc + kTile - 1) / kTile;
     for (uint32_t i = 0; i < n_chunks; ++i) {
         const ElxChunk &c = h_chunks[i];
+        if ((c.n_alloc + kTile - 1) / kTile != uniform) uniform = 0;
         if (!c.master || !c.m || !c.v) return ELX_E_NULL;
         if (c.lowp_out && lowp_dtype == ELX_NONE) return ELX_E_DTYPE;
         if (c.n_alloc == 0) return ELX_E_SIZE;
@@ -520,13 +594,15 @@ int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *
         uint64_t prev_end = 0;
         for (uint32_t s = c.seg_begin; s < c.seg_end; ++s) {
             const ElxSeg &sg = h_segs[s];
-            if (sg.begin >= sg.end || sg.end > c.n_alloc) return ELX_E_RANGE;
+            if (sg.begin >= sg.end || sg.end > c.n_valid) return ELX_E_RANGE;
             if (sg.hyper >= n_hypers) return ELX_E_RANGE;
             if (sg.begin < prev_end) return ELX_E_ORDER;
             prev_end = sg.end;
         }
     }
+    if (tiles > 0x7FFFFFFFull) return ELX_E_SIZE;    // one workgroup per tile
     *total_tiles = tiles;
+    *uniform_tiles_per_chunk = (uint32_t)uniform;
     *all_aligned16 = aligned;
     return 0;
 }
@@ -541,29 +617,33 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
     const uint32_t so = scalar_only ? 1u : 0u;
     switch (grad_dtype) {
         case ELX_F32:
-            hipLaunchKernelGGL((grad_stats_kernel<ELX_F32>), grid, dim3(kThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
+            hipLaunchKernelGGL((grad_stats_kernel<ELX_F32>), grid, dim3(kStatsThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
             break;
         case ELX_F16:
-            hipLaunchKernelGGL((grad_stats_kernel<ELX_F16>), grid, dim3(kThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
+            hipLaunchKernelGGL((grad_stats_kernel<ELX_F16>), grid, dim3(kStatsThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
             break;
         case ELX_BF16:
-            hipLaunchKernelGGL((grad_stats_kernel<ELX_BF16>), grid, dim3(kThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
+            hipLaunchKernelGGL((grad_stats_kernel<ELX_BF16>), grid, dim3(kStatsThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
             break;
         default: return ELX_E_DTYPE;
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_chunks), dim3(kThreads), 0, st, d_partials, blocks_per_chunk, d_stats);
+    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, st, d_partials, blocks_per_chunk, d_stats);
     return (int)hipGetLastError();
 }
 
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
-                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles, float div_scale, int grad_dtype,
-                     int lowp_dtype, uint32_t flags, uint32_t max_blocks, void *stream) {
+                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles, uint32_t uniform_tiles_per_chunk,
+                     float div_scale, int grad_dtype, int lowp_dtype, uint32_t flags, uint32_t blocks_per_cu,
+                     void *stream) {
     if (!d_chunks || (n_segs && (!d_segs || !d_hypers))) return ELX_E_NULL;
-    if (n_chunks == 0 || total_tiles == 0 || (n_segs && n_hypers == 0)) return ELX_E_SIZE;
+    if (n_chunks == 0 || total_tiles == 0 || total_tiles > 0x7FFFFFFFull || (n_segs && n_hypers == 0)) return ELX_E_SIZE;
+    if (uniform_tiles_per_chunk && (uint64_t)uniform_tiles_per_chunk * n_chunks != total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    uint32_t lds = 0;
+    if (int rc = occupancy_reservation(blocks_per_cu, &lds)) return rc;
     Unscale us;
     us.div_scale = div_scale;
     us.inv_scale = 1.0f;
@@ -576,22 +656,24 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
             us.mode = kDivTrue;
         }
     }
-    const bool nt = true;
-    return dispatch_step(grad_dtype, lowp_dtype, nt, step_grid(total_tiles, max_blocks), (hipStream_t)stream, d_chunks,
-                         n_chunks, d_segs, d_hypers, total_tiles, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 0u);
+    return dispatch_step(grad_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
+                         d_segs, d_hypers, uniform_tiles_per_chunk, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 0u);
 }
 
-int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles, int lowp_dtype, uint32_t flags,
-                     uint32_t max_blocks, void *stream) {
+int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles, uint32_t uniform_tiles_per_chunk,
+                     int lowp_dtype, uint32_t flags, uint32_t blocks_per_cu, void *stream) {
     if (!d_chunks) return ELX_E_NULL;
-    if (n_chunks == 0 || total_tiles == 0) return ELX_E_SIZE;
+    if (n_chunks == 0 || total_tiles == 0 || total_tiles > 0x7FFFFFFFull) return ELX_E_SIZE;
+    if (uniform_tiles_per_chunk && (uint64_t)uniform_tiles_per_chunk * n_chunks != total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(lowp_dtype)) return ELX_E_DTYPE;
+    uint32_t lds = 0;
+    if (int rc = occupancy_reservation(blocks_per_cu, &lds)) return rc;
     Unscale us;
     us.div_scale = -1.0f;
     us.inv_scale = 1.0f;
     us.mode = kDivNone;
-    return dispatch_step(lowp_dtype, lowp_dtype, true, step_grid(total_tiles, max_blocks), (hipStream_t)stream, d_chunks,
-                         n_chunks, nullptr, nullptr, total_tiles, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 1u);
+    return dispatch_step(lowp_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
+                         nullptr, nullptr, uniform_tiles_per_chunk, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 1u);
 }
 
 }    // extern "C"

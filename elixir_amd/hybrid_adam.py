@@ -129,7 +129,7 @@ class HybridAdam(torch.optim.Optimizer):
         default_args = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, bias_correction=bias_correction)
         super().__init__(model_params, default_args)
         self.adamw_mode = adamw_mode
-        self.max_blocks = 0    # 0: one workgroup per tile
+        self.blocks_per_cu = 0    # cap on resident update workgroups per compute unit; 0: library default
         self._binding: Optional[ChunkBinding] = None
         self._chunk_table = _CachedTable()
         self._seg_table = _CachedTable()
@@ -184,15 +184,14 @@ class HybridAdam(torch.optim.Optimizer):
         if key != self._checked_key:
             self._checked = _abi.check_tables(chunks, segs, len(hyper_host), grad_code, lowp_code)
             self._checked_key = key
-        total_tiles, aligned = self._checked
+        info = self._checked
 
         d_chunks = self._chunk_table.get(chunks, device)
         d_segs = self._seg_table.get(segs, device)
         d_hypers = self._hyper_table.get(hyper_host, device)
         stream = torch.cuda.current_stream(device).cuda_stream
-        _abi.adam_step_mt(d_chunks.ptr, len(chunks), d_segs.ptr, len(segs), d_hypers.ptr, len(hyper_host), total_tiles,
-                          float(div_scale), grad_code, lowp_code, 0 if aligned else _abi.ELX_FLAG_SCALAR_ONLY,
-                          self.max_blocks, stream)
+        _abi.adam_step_mt(d_chunks.ptr, len(chunks), d_segs.ptr, len(segs), d_hypers.ptr, len(hyper_host), info,
+                          float(div_scale), grad_code, lowp_code, self.blocks_per_cu, stream)
         if self._binding is not None and lowp_code != _abi.ELX_NONE:
             self._binding.fused_writeback = True
         return loss

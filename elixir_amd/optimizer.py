@@ -153,6 +153,8 @@ class ElixirOptimizer:
         # when set to a dict, step() records (begin, end) torch.cuda.Event pairs on the launch
         # stream under the keys 'stats' and 'update' (for per-kernel timing by a benchmark)
         self.kernel_events = None
+        # cap on resident update workgroups per compute unit (0 = the library default)
+        self.blocks_per_cu = 0
 
         if init_step:
             # allocate memory before training
@@ -297,12 +299,11 @@ class ElixirOptimizer:
                 rows[i]['tile_begin'] = tiles
                 tiles += (c.shard_size + tile - 1) // tile
             code = dtype_code(gpu_chunks[0].chunk_dtype)
-            total_tiles, aligned = _abi.check_tables(rows, None, 0, code, code)
-            self._wb_table = (DeviceTable(rows, gpu_chunks[0].shard_device), total_tiles, aligned, code)
-        table, total_tiles, aligned, code = self._wb_table
+            info = _abi.check_tables(rows, None, 0, code, code)
+            self._wb_table = (DeviceTable(rows, gpu_chunks[0].shard_device), info, code)
+        table, info, code = self._wb_table
         stream = torch.cuda.current_stream(table.dev.device).cuda_stream
-        _abi.writeback_mt(table.ptr, len(table), total_tiles, code, 0 if aligned else _abi.ELX_FLAG_SCALAR_ONLY, 0,
-                          stream)
+        _abi.writeback_mt(table.ptr, len(table), info, code, self.blocks_per_cu, stream)
         for c in gpu_chunks:
             c.optim_sync_flag = True
 

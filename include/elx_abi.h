@@ -40,10 +40,10 @@ enum {
     ELX_E_NULL = -1,     /* a required pointer is NULL */
     ELX_E_DTYPE = -2,    /* unknown or unsupported dtype combination */
     ELX_E_ALIGN = -3,    /* a chunk base pointer is not aligned to its element size */
-    ELX_E_RANGE = -4,    /* begin > end, end > n_alloc, n_valid > n_alloc, bad segment range or hyper index */
+    ELX_E_RANGE = -4,    /* begin >= end, end > n_valid, n_valid > n_alloc, bad segment range or hyper index */
     ELX_E_ORDER = -5,    /* segments of a chunk are not sorted by begin or overlap */
     ELX_E_TILES = -6,    /* tile_begin / total_tiles disagree with the chunk sizes */
-    ELX_E_SIZE = -7      /* a count is zero or exceeds what a launch can address */
+    ELX_E_SIZE = -7      /* a count is zero, out of its allowed range, or exceeds what a launch can address */
 };
 
 /* flags of elx_adam_step_mt */
@@ -135,14 +135,18 @@ uint32_t elx_sizeof_stats(void);
 /*
  * Host-side validation of HOST copies of the tables, to be called once before they are uploaded:
  * NULL / dtype / range / ordering / tile checks as listed under the ELX_E_* codes.  On success
- * writes the launch-wide tile count to *total_tiles and to *all_aligned16 whether every non-NULL
- * base pointer is 16-byte aligned (if not, pass ELX_FLAG_SCALAR_ONLY to the launches).
+ * writes
+ *   *total_tiles              the launch-wide tile count (one workgroup per tile, < 2^31),
+ *   *uniform_tiles_per_chunk  the tile count of every chunk when they all agree, else 0
+ *                             (lets the kernels find a tile's chunk with one division),
+ *   *all_aligned16            whether every non-NULL base pointer is 16-byte aligned (if not, pass
+ *                             ELX_FLAG_SCALAR_ONLY to the launches).
  * lowp_dtype may be ELX_NONE when no chunk has a lowp_out buffer.
  * Replaces the per-tensor asserts and range bookkeeping of optimizer.py:238-265 at the boundary.
  */
 int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *h_segs, uint32_t n_segs,
                      uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles,
-                     int *all_aligned16);
+                     uint32_t *uniform_tiles_per_chunk, int *all_aligned16);
 
 /*
  * Stats pass over grad[0, n_valid) of every chunk: replaces Chunk.set_overflow_flag and
@@ -161,19 +165,23 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
  * and for every element of the shard (padding included), when lowp_out is set,
  *   lowp_out = round-to-nearest-even(master)                       -- chunk.py:414
  * Replaces the inner optimizer's step over the fake parameters plus Chunk.optim_update.
- *   max_blocks  0 = one workgroup per tile, otherwise the grid is capped and strides over tiles
+ *   total_tiles, uniform_tiles_per_chunk   as returned by elx_check_tables for these tables
+ *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (10).
+ *                  The update streams best with a shallow, orderly queue of memory requests.
  */
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
-                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles, float div_scale,
-                     int grad_dtype, int lowp_dtype, uint32_t flags, uint32_t max_blocks, void *stream);
+                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,
+                     uint32_t uniform_tiles_per_chunk, float div_scale, int grad_dtype, int lowp_dtype,
+                     uint32_t flags, uint32_t blocks_per_cu, void *stream);
 
 /*
  * Low-precision refresh alone: lowp_out[0, n_alloc) = round-to-nearest-even(master) for every
  * chunk.  The skip-step branch (optimizer.py:196-203 -> chunk.py:403-414) and state loading
  * (elixir/wrapper/module.py:343) use it.
  */
-int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles, int lowp_dtype,
-                     uint32_t flags, uint32_t max_blocks, void *stream);
+int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles,
+                     uint32_t uniform_tiles_per_chunk, int lowp_dtype, uint32_t flags, uint32_t blocks_per_cu,
+                     void *stream);
 
 #ifdef __cplusplus
 }

@@ -470,7 +470,7 @@ def test_abi_rejects_bad_tables():
     seg = np.zeros(1, dtype=_abi.SEG_DTYPE)
     seg[0] = (0, 8192, 0, 0)
     row['seg_end'] = 1
-    assert _abi.check_tables(row, seg, 1, _abi.ELX_F32, _abi.ELX_NONE) == (2, True)
+    assert _abi.check_tables(row, seg, 1, _abi.ELX_F32, _abi.ELX_NONE) == (8192 // _abi.tile_elems(), 8192 // _abi.tile_elems(), True)
 
     def expect(code, chunk=row, segs=seg, n_hypers=1, gd=_abi.ELX_F32, ld=_abi.ELX_NONE):
         with pytest.raises(_abi.ElxError) as e:
