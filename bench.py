@@ -25,6 +25,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
 BYTES_UPDATE = 28               # per valid element: read g(2)+p,m,v(12); write p,m,v(12)+lowp(2)
 BYTES_STATS = 2                 # per valid element: the compulsory second read of g
+# HBM bytes per update launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
+# scaled by what the same counters read for a plain copy of known size (--calibrate-copy):
+# 96.375e9 read + 95.356e9 written for c5, i.e. the algorithmic bytes plus the refresh of the
+# chunk padding.  Counter runs cannot ride along with a timed run, hence a recorded figure.
+MEASURED_TRAFFIC_BYTES = {'c5': 191.73e9}
 
 
 def cpu_baseline(built, sample_elems: int, steps: int = 3):
@@ -84,6 +89,9 @@ def main():
     ap.add_argument('--cpu-sample', type=int, default=32 << 20, help='elements of the CPU baseline sample; 0 skips it')
     ap.add_argument('--blocks-per-cu', type=int, default=0,
                     help='cap on resident update workgroups per compute unit (0 = library default)')
+    ap.add_argument('--calibrate-copy', type=float, default=0.0,
+                    help='instead of the benchmark, run three plain device copies of this many GiB (a kernel of '
+                    'known traffic, to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit')
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -93,6 +101,16 @@ def main():
     if not torch.cuda.is_available():
         print('bench.py needs a GPU: the optimizer step has no CPU path', file=sys.stderr)
         sys.exit(2)
+
+    if args.calibrate_copy > 0:
+        n = int(args.calibrate_copy * (1 << 30)) // 4
+        src = torch.rand(n, device='cuda')
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({'calibrate_copy_bytes_read': n * 4, 'calibrate_copy_bytes_written': n * 4, 'copies': 3}))
+        return
 
     from elixir_amd import _abi, workloads
     _abi.load()
@@ -166,7 +184,7 @@ def main():
             'peak': HBM_PEAK_GBPS,
             'unit': 'GB/s',
             'frac': upd_gbps / HBM_PEAK_GBPS,
-            'traffic': None,
+            'traffic': MEASURED_TRAFFIC_BYTES.get(built.spec.name),
             'bytes_per_launch': BYTES_UPDATE * n_valid,
             'ms_per_launch': t_upd * 1e3,
         },

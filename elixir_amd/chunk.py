@@ -253,7 +253,9 @@ class Chunk:
         self.num_tensors += 1
         tensor_state = TensorState.HOLD
         self.tensor_state_cnter[tensor_state] += 1
-        self.tensors_info[tensor] = TensorInfo(state=tensor_state, fake_data=None, offset=self.utilized_size,
+        # a data-less stand-in that remembers the tensor's shape while its storage lives in the chunk
+        fake_data = torch.empty(tensor.shape, dtype=tensor.dtype, device='meta')
+        self.tensors_info[tensor] = TensorInfo(state=tensor_state, fake_data=fake_data, offset=self.utilized_size,
                                                end=new_utilized_size)
         self.utilized_size = new_utilized_size
 

@@ -204,7 +204,7 @@ class ElixirModule(nn.Module):
         for param in self.grad_state_dict.values():
             chunk = self.param_chunk_group.ten_to_chunk[param]
             info = chunk.tensors_info[param]
-            param.data = chunk.shard[info.offset:info.end].clone().view(param.shape)
+            param.data = chunk.shard[info.offset:info.end].clone().view(info.fake_data.shape)
 
     def forward(self, *args, **kwargs):
         assert not self.synthetic
@@ -247,7 +247,7 @@ class ElixirModule(nn.Module):
                 p_chunk = self.param_chunk_group.ten_to_chunk[param]
                 info = p_chunk.tensors_info[param]
                 src = p_chunk if from_param else p_chunk.paired_chunk
-                module_state_dict[name] = src.shard[info.offset:info.end].view(param.shape).cpu()
+                module_state_dict[name] = src.shard[info.offset:info.end].view(info.fake_data.shape).cpu()
             else:
                 module_state_dict[name] = tensor.detach()
         return module_state_dict

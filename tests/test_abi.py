@@ -1,0 +1,127 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol include/elx_abi.h declares, its
+record layouts match the Python mirrors, and its host-side table validation returns the documented
+codes.  No kernel is launched here."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+from elixir_amd import _abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, 'include', 'elx_abi.h')
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(elx_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = _abi.load()
+    names = declared_functions()
+    assert names, 'no declarations found in the header'
+    for name in names:
+        assert hasattr(lib, name), f'{name} is declared in elx_abi.h but not exported'
+    assert sorted(_abi.EXPORTS) == names, 'the binding and the header disagree on the entry points'
+    assert lib.elx_version() == _abi.ELX_ABI_VERSION
+
+
+def test_record_layouts_match_the_header():
+    lib = _abi.load()
+    assert lib.elx_sizeof_chunk() == _abi.CHUNK_DTYPE.itemsize == 72
+    assert lib.elx_sizeof_seg() == _abi.SEG_DTYPE.itemsize == 24
+    assert lib.elx_sizeof_hyper() == _abi.HYPER_DTYPE.itemsize == 48
+    assert lib.elx_sizeof_stats() == _abi.STATS_DTYPE.itemsize == 16
+    # field offsets as the C struct lays them out
+    assert [_abi.CHUNK_DTYPE.fields[f][1] for f in ('grad', 'lowp_out', 'master', 'm', 'v', 'n_alloc', 'n_valid',
+                                                    'tile_begin', 'seg_begin', 'seg_end')] == [0, 8, 16, 24, 32, 40, 48,
+                                                                                              56, 64, 68]
+    assert [_abi.HYPER_DTYPE.fields[f][1] for f in ('decay_mul', 'l2_wd', 'lerp_w', 'beta2', 'omb2', 'bc2_sqrt', 'eps',
+                                                    'neg_step', 'flags')] == [0, 4, 8, 12, 16, 20, 24, 28, 32]
+    assert _abi.tile_elems() == 512
+
+
+def test_strerror_covers_every_code():
+    lib = _abi.load()
+    seen = set()
+    for code in range(0, -8, -1):
+        text = lib.elx_strerror(code).decode()
+        assert text and text not in seen
+        seen.add(text)
+    assert 'unknown' in lib.elx_strerror(-99).decode()
+
+
+def _row(n=8192, base=0x10000000):
+    row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+    row['grad'] = base
+    row['master'] = base + (1 << 20)
+    row['m'] = base + (2 << 20)
+    row['v'] = base + (3 << 20)
+    row['n_alloc'] = n
+    row['n_valid'] = n
+    row['seg_end'] = 1
+    return row
+
+
+def test_check_tables_accepts_and_rejects():
+    tile = _abi.tile_elems()
+    row = _row()
+    seg = np.zeros(1, dtype=_abi.SEG_DTYPE)
+    seg[0] = (0, 8192, 0, 0)
+    info = _abi.check_tables(row, seg, 1, _abi.ELX_F32, _abi.ELX_NONE)
+    assert info == (8192 // tile, 8192 // tile, True)
+
+    def expect(code, chunk=row, segs=seg, n_hypers=1, gd=_abi.ELX_F32, ld=_abi.ELX_NONE):
+        with pytest.raises(_abi.ElxError) as e:
+            _abi.check_tables(chunk, segs, n_hypers, gd, ld)
+        assert e.value.code == code, e.value
+
+    bad = row.copy(); bad['master'] = 0; expect(-1, chunk=bad)                        # NULL
+    expect(-2, gd=7)                                                                  # dtype
+    expect(-2, gd=_abi.ELX_F16, ld=_abi.ELX_BF16)
+    bad = row.copy(); bad['lowp_out'] = 0x20000000; expect(-2, chunk=bad)             # lowp_out without a dtype
+    bad = row.copy(); bad['m'] = int(row['m'][0]) + 2; expect(-3, chunk=bad)          # fp32 pointer at +2
+    bad = row.copy(); bad['grad'] = int(row['grad'][0]) + 1; expect(-3, chunk=bad, gd=_abi.ELX_F16)
+    bad = row.copy(); bad['n_valid'] = 9000; expect(-4, chunk=bad)                    # n_valid > n_alloc
+    s2 = seg.copy(); s2[0] = (0, 9000, 0, 0); expect(-4, segs=s2)                     # end > n_valid
+    s2 = seg.copy(); s2[0] = (10, 10, 0, 0); expect(-4, segs=s2)                      # empty segment
+    s2 = seg.copy(); s2[0] = (0, 8192, 3, 0); expect(-4, segs=s2)                     # hyper index
+    bad = row.copy(); bad['n_valid'] = 4096; expect(-4, chunk=bad)                    # segment beyond valid head
+    two = np.zeros(2, dtype=_abi.SEG_DTYPE); two[0] = (100, 200, 0, 0); two[1] = (150, 300, 0, 0)
+    bad = row.copy(); bad['seg_end'] = 2; expect(-5, chunk=bad, segs=two)             # overlap
+    two[0] = (300, 400, 0, 0); two[1] = (100, 200, 0, 0); expect(-5, chunk=bad, segs=two)    # unsorted
+    bad = row.copy(); bad['tile_begin'] = 1; expect(-6, chunk=bad)                    # tile bookkeeping
+    bad = row.copy(); bad['n_alloc'] = 0; bad['n_valid'] = 0; expect(-7, chunk=bad, segs=None)
+
+
+def test_check_tables_reports_alignment_and_uniformity():
+    tile = _abi.tile_elems()
+    rows = np.concatenate([_row(8192, 0x10000000), _row(8192, 0x20000000), _row(5000, 0x30000000)])
+    rows['seg_begin'] = 0
+    rows['seg_end'] = 0
+    rows['tile_begin'] = [0, 16, 32]
+    info = _abi.check_tables(rows, None, 0, _abi.ELX_F16, _abi.ELX_NONE)
+    assert info.total_tiles == 32 + (5000 + tile - 1) // tile and info.uniform_tiles == 0 and info.aligned
+    info = _abi.check_tables(rows[:2], None, 0, _abi.ELX_F16, _abi.ELX_NONE)
+    assert info.total_tiles == 32 and info.uniform_tiles == 16
+    rows[1]['grad'] += 2    # 2-byte aligned only: legal for fp16, but not vectorisable
+    info = _abi.check_tables(rows[:2], None, 0, _abi.ELX_F16, _abi.ELX_NONE)
+    assert not info.aligned and info.flags == _abi.ELX_FLAG_SCALAR_ONLY
+
+
+def test_launch_entry_points_reject_bad_arguments_before_launching():
+    """Argument errors are returned before any kernel is enqueued, so this runs without a GPU."""
+    lib = _abi.load()
+    assert lib.elx_grad_stats_mt(None, 1, _abi.ELX_F16, 1, None, None, 0, None) == -1
+    assert lib.elx_grad_stats_mt(1, 1, _abi.ELX_F16, 0, 1, 1, 0, None) == -7
+    assert lib.elx_grad_stats_mt(1, 1, _abi.ELX_F16, 2000, 1, 1, 0, None) == -7
+    assert lib.elx_adam_step_mt(None, 1, None, 0, None, 0, 1, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -1
+    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 0, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -7
+    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, 9, _abi.ELX_NONE, 0, 0, None) == -2
+    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 2, None) == -7
+    assert lib.elx_adam_step_mt(1, 2, None, 0, None, 0, 5, 2, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -6
+    assert lib.elx_writeback_mt(None, 1, 4, 0, _abi.ELX_F16, 0, 0, None) == -1
+    assert lib.elx_writeback_mt(1, 1, 4, 0, _abi.ELX_NONE, 0, 0, None) == -2

@@ -1,0 +1,171 @@
+"""The step at the full sizes of the benchmark workloads (GPT-2 small, OPT-1.3B, LLaMA-7B chunk
+sets).  The oracle cannot chew through billions of elements in seconds, so the checks here are the
+ones that do not depend on size:
+
+  * the update is element-wise, so ANY slice of a chunk is a complete small problem: seeded slices
+    (segment heads and tails, chunk tails with padding, random interiors) are replayed by the CPU
+    oracle from the pre-step state and must match the GPU's post-step state;
+  * the gradient norm is additive: the global norm the step used equals the float64 sum over
+    torch-computed slice norms;
+  * writeback is idempotent and total: after the step every low-precision shard equals the cast of
+    its master shard, padding included;
+  * a skipped step (overflow) leaves master / exp_avg / exp_avg_sq bit-identical, restores the
+    low-precision shards, and moves the loss scale as the state machine says;
+  * the step is deterministic: replaying it from the same state gives the same bits.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from elixir_amd import workloads
+from oracle import oracle as O
+
+from helpers import CODE, to_np, ulp_distance
+
+pytestmark = pytest.mark.gpu
+
+
+def _slices(pc, opt, rng, width=4096, n_random=6):
+    """(begin, end) windows of one chunk: around every few segment boundaries, the chunk tail
+    (valid end and padding), and random interiors."""
+    oc = pc.paired_chunk
+    n = pc.shard_size
+    bounds = sorted({b for f, c in opt.param_to_optim_chunk.items() if c is oc for b in opt.param_to_range[f]})
+    picks = set()
+    for b in bounds[::max(1, len(bounds) // 6)]:
+        picks.add(max(0, min(n - width, b - width // 2)))
+    picks.add(max(0, n - width))
+    picks.add(max(0, min(n - width, pc.utilized_size - width // 2)))
+    for _ in range(n_random):
+        picks.add(int(rng.integers(0, max(1, n - width))))
+    return [(b, min(n, b + width)) for b in sorted(picks)]
+
+
+def _oracle_on_slice(pc, opt, b, e, pre, comb, dtype):
+    """Replays the update on [b, e) of one chunk with the CPU oracle; returns (p, m, v, lowp)."""
+    oc = pc.paired_chunk
+    g, p, m, v = (a.copy() for a in pre)
+    inner = opt.optim
+    for group in inner.param_groups:
+        for fake in group['params']:
+            if opt.param_to_optim_chunk[fake] is not oc:
+                continue
+            sb, se = opt.param_to_range[fake]
+            lo, hi = max(sb, b), min(se, e)
+            if lo >= hi:
+                continue
+            sl = slice(lo - b, hi - b)
+            O.adam(g[sl], CODE[dtype], p[sl], m[sl], v[sl], lr=group['lr'], beta1=group['betas'][0],
+                   beta2=group['betas'][1], eps=group['eps'], weight_decay=group['weight_decay'],
+                   step=inner.state[fake]['step'], adamw_mode=inner.adamw_mode,
+                   bias_correction=group['bias_correction'], div_scale=float(comb))
+    return p, m, v, O.writeback(p, CODE[dtype])
+
+
+@pytest.mark.parametrize('name', ['c2', 'c4', 'c5'])
+def test_full_size_step(oracle, name):
+    built = workloads.build(name, seed=4321)
+    opt, module, dtype = built.optimizer, built.module, built.spec.dtype
+    rng = np.random.default_rng(11)
+    binding = opt._binding
+
+    # ---- a clean step, checked on slices ------------------------------------------------------
+    built.land_gradients()
+    windows, pre = {}, {}
+    norm_sq = 0.0
+    for ci, pc in enumerate(module.param_chunks):
+        oc = pc.paired_chunk
+        m, v = binding.moments(oc)
+        windows[ci] = _slices(pc, opt, rng)
+        for (b, e) in windows[ci]:
+            pre[(ci, b)] = (to_np(pc.shard[b:e]), to_np(oc.shard[b:e]), to_np(m[b:e]), to_np(v[b:e]))
+        if built.spec.max_norm > 0:
+            # per-chunk squared norm the way the reference takes it (chunk.py:218-221), with torch
+            norm_sq += float(pc.shard[:pc.n_valid].float().norm(2).item())**2
+    opt.step()
+    info = opt.last_step_info
+    assert info['found_inf'] is False
+    if built.spec.max_norm > 0:
+        assert math.isclose(info['total_norm'], math.sqrt(norm_sq), rel_tol=1e-6)
+        want_comb = O.combined_scale(built.spec.loss_scale, info['total_norm'], built.spec.max_norm)
+        assert info['combined_scale'] == want_comb
+    else:
+        assert info['combined_scale'] == O.combined_scale(built.spec.loss_scale, None, 0.0)
+    comb = info['combined_scale']
+    assert all(st['step'] == 1 for st in opt.state.values())
+
+    for ci, pc in enumerate(module.param_chunks):
+        oc = pc.paired_chunk
+        m, v = binding.moments(oc)
+        for (b, e) in windows[ci]:
+            wp, wm, wv, wl = _oracle_on_slice(pc, opt, b, e, pre[(ci, b)], comb, dtype)
+            tag = f'{name} chunk {ci} [{b},{e})'
+            assert np.array_equal(to_np(oc.shard[b:e]).view(np.uint32), wp.view(np.uint32)), tag + ' master'
+            assert np.array_equal(to_np(m[b:e]).view(np.uint32), wm.view(np.uint32)), tag + ' exp_avg'
+            assert np.array_equal(to_np(v[b:e]).view(np.uint32), wv.view(np.uint32)), tag + ' exp_avg_sq'
+            assert ulp_distance(to_np(pc.shard[b:e]), wl) == 0, tag + ' writeback'
+        # writeback is total: the whole low-precision shard is the cast of the master shard
+        assert torch.equal(pc.shard, oc.shard.to(dtype)), f'{name} chunk {ci}: shard != cast(master)'
+        assert pc.optim_sync_flag is True
+
+    # ---- determinism: replay the same step from a restored slice of state ---------------------
+    ci = 0
+    pc = module.param_chunks[ci]
+    oc = pc.paired_chunk
+    m, v = binding.moments(oc)
+    after = (oc.shard[:65536].clone(), m[:65536].clone(), v[:65536].clone())
+
+    # ---- an overflow: skip, restore, back off --------------------------------------------------
+    built.land_gradients()
+    last = module.param_chunks[-1]
+    last.shard[last.n_valid - 1] = float('nan')
+    if last.n_valid < last.shard_size:
+        last.shard[last.n_valid] = float('inf')           # padding: must not matter
+    keep = [(pc.paired_chunk.shard[:65536].clone(), *(t[:65536].clone() for t in binding.moments(pc.paired_chunk)))
+            for pc in module.param_chunks]
+    scale_before = opt.loss_scale
+    opt.step()
+    assert opt.last_step_info['found_inf'] is True
+    assert opt.loss_scale == (scale_before * 0.5 if module.use_amp else scale_before)
+    assert all(st['step'] == 1 for st in opt.state.values())
+    for pc, (p0, m0, v0) in zip(module.param_chunks, keep):
+        oc = pc.paired_chunk
+        m, v = binding.moments(oc)
+        assert torch.equal(oc.shard[:65536], p0) and torch.equal(m[:65536], m0) and torch.equal(v[:65536], v0)
+        assert torch.equal(pc.shard, oc.shard.to(dtype))
+    assert torch.equal(after[0], oc.shard[:65536] if False else module.param_chunks[0].paired_chunk.shard[:65536])
+
+    # ---- a clean follow-up step at the new scale passes the same slice check ------------------
+    if module.use_amp:
+        for pc, g in zip(module.param_chunks, built.grads):
+            g.mul_(0.5)                                    # the same gradients at the halved loss scale
+    built.land_gradients()
+    pc = module.param_chunks[1 % len(module.param_chunks)]
+    oc = pc.paired_chunk
+    m, v = binding.moments(oc)
+    b, e = windows[1 % len(module.param_chunks)][0]
+    pre1 = (to_np(pc.shard[b:e]), to_np(oc.shard[b:e]), to_np(m[b:e]), to_np(v[b:e]))
+    opt.step()
+    assert opt.last_step_info['found_inf'] is False
+    assert all(st['step'] == 2 for st in opt.state.values())
+    wp, wm, wv, wl = _oracle_on_slice(pc, opt, b, e, pre1, opt.last_step_info['combined_scale'], dtype)
+    assert np.array_equal(to_np(oc.shard[b:e]).view(np.uint32), wp.view(np.uint32))
+    assert np.array_equal(to_np(m[b:e]).view(np.uint32), wm.view(np.uint32))
+    assert ulp_distance(to_np(pc.shard[b:e]), wl) == 0
+
+
+def test_full_size_step_is_deterministic():
+    a = workloads.build('c2', seed=99)
+    a.land_gradients()
+    a.optimizer.step()
+    first = [(pc.paired_chunk.shard.clone(), pc.shard.clone()) for pc in a.module.param_chunks]
+    norm = a.optimizer.last_step_info
+    del a
+    b = workloads.build('c2', seed=99)
+    b.land_gradients()
+    b.optimizer.step()
+    assert b.optimizer.last_step_info == norm
+    for (p0, l0), pc in zip(first, b.module.param_chunks):
+        assert torch.equal(p0, pc.paired_chunk.shard) and torch.equal(l0, pc.shard)

@@ -1,0 +1,127 @@
+"""End-to-end: a small network trained through ElixirModule + ElixirOptimizer(HybridAdam) against
+plain PyTorch training of an identical copy -- the shape of the reference's own tests
+(test/wrapper/test_optimizer.py: fp32, rtol 2e-6 / atol 2e-5 on the weights after the step;
+test/wrapper/test_amp.py: fp16 against master-weight AMP, assert_close defaults)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import elixir_amd as ea
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+class Net(nn.Module):
+    """Dense layers only: no scatter-add in backward, so two runs of the same step produce the
+    same gradients bit for bit and the comparison sees the optimizers, not atomics."""
+
+    def __init__(self, width=24, hidden=32):
+        super().__init__()
+        self.inp = nn.Linear(width, hidden)
+        self.norm1 = nn.LayerNorm(hidden)
+        self.fc1 = nn.Linear(hidden, 4 * hidden)
+        self.fc2 = nn.Linear(4 * hidden, hidden)
+        self.norm2 = nn.LayerNorm(hidden)
+        self.head = nn.Linear(hidden, 50, bias=False)
+
+    def forward(self, x):
+        h = self.inp(x.to(self.inp.weight.dtype))
+        h = h + self.fc2(torch.nn.functional.gelu(self.fc1(self.norm1(h))))
+        return self.head(self.norm2(h)).float().logsumexp(-1).mean()
+
+
+def batch(gen):
+    return torch.randn(8, 16, 24, device=DEV, generator=gen)
+
+
+def groups_of(model, wd):
+    decay = [p for p in model.parameters() if p.dim() > 1]
+    exempt = [p for p in model.parameters() if p.dim() == 1]
+    return [dict(params=decay, weight_decay=wd), dict(params=exempt, weight_decay=0.0)]
+
+
+def wrap(model, dtype, chunk_size=4096, **kw):
+    named = [(n, p.numel()) for n, p in model.named_parameters()]
+    module = ea.ElixirModule(model, ea.greedy_search(named, chunk_size, dtype), dtype=dtype)
+    inner = ea.HybridAdam(groups_of(model, 0.1), lr=1e-2, weight_decay=0.1)
+    return module, ea.ElixirOptimizer(module, inner, **kw)
+
+
+def test_fp32_training_matches_torch_adamw():
+    torch.manual_seed(0)
+    ref = Net().to(DEV)
+    model = copy.deepcopy(ref)
+    ropt = torch.optim.AdamW(groups_of(ref, 0.1), lr=1e-2, weight_decay=0.1)
+    module, opt = wrap(model, torch.float32)
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    for step in range(4):
+        x = batch(gen)
+        ropt.zero_grad()
+        ref(x).backward()
+        ropt.step()
+        opt.zero_grad()
+        opt.backward(module(x))
+        opt.step()
+        module.materialize_params()
+        sd = module.state_dict()
+        for name, want in ref.state_dict().items():
+            torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
+
+
+def test_fp16_training_matches_master_weight_amp_and_recovers_from_overflow():
+    torch.manual_seed(0)
+    master = Net().to(DEV)                         # fp32 master copy trained by plain torch
+    model = copy.deepcopy(master)
+    ropt = torch.optim.AdamW(groups_of(master, 0.1), lr=1e-2, weight_decay=0.1)
+    module, opt = wrap(model, torch.float16, initial_scale=1024.0, hysteresis=1, growth_interval=1000)
+    gen = torch.Generator(device=DEV).manual_seed(2)
+    scale = 1024.0
+    for step in range(5):
+        x = batch(gen)
+        poison = step == 2
+        # reference side: fp16 working copy of the fp32 master, scaled loss, unscale in fp32
+        work = copy.deepcopy(master).half()
+        (work(x) * scale).backward()
+        grads = [p.grad for p in work.parameters()]
+        if poison:
+            grads[3].view(-1)[5] = float('inf')
+        if any((~torch.isfinite(g)).any() for g in grads):
+            scale *= 0.5
+        else:
+            for p, g in zip(master.parameters(), grads):
+                p.grad = g.float() / scale
+            ropt.step()
+        # this build
+        assert opt.loss_scale == (1024.0 if step <= 2 else 512.0)
+        opt.zero_grad()
+        opt.backward(module(x))
+        if poison:
+            pc = module.param_chunks[0]
+            pc.shard[7] = float('inf')
+        opt.step()
+        assert opt.last_step_info['found_inf'] == poison
+        module.materialize_params()
+        sd = module.state_dict()
+        for name, want in master.state_dict().items():
+            torch.testing.assert_close(sd[name], want.cpu(), msg=f'step {step} {name}')
+        # the parameters the forward pass sees are the rounded masters
+        for name, p in model.named_parameters():
+            assert torch.equal(p.data.cpu(), sd[name].half())
+    assert opt.loss_scale == scale == 512.0
+
+
+def test_state_dict_round_trip_and_load():
+    torch.manual_seed(3)
+    model = Net().to(DEV)
+    module, opt = wrap(model, torch.bfloat16)
+    sd = module.state_dict()
+    new = {k: torch.randn_like(v) for k, v in sd.items()}
+    module.load_state_dict(new)
+    back = module.state_dict()
+    for k in new:
+        assert torch.equal(back[k], new[k])
+        assert torch.equal(module.state_dict(from_param=True)[k], new[k].bfloat16())

@@ -1,0 +1,273 @@
+"""Host side of the optimizer step without a GPU: loss scaler, combined scale, hyper-parameter
+records, chunk layout, chunk pairing, fake-parameter ranges, and the refusal to run without the
+HIP path."""
+import math
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import elixir_amd as ea
+from elixir_amd import _abi
+from elixir_amd import shapes as S
+from elixir_amd.chunk import l2_norm_from_sumsq, stats_launch_blocks
+from elixir_amd.hybrid_adam import make_hyper_record
+from oracle import oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ------------------------------------------------------------------------------------------------
+# scalers and host scalars
+# ------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize('hysteresis', [1, 2, 3])
+@pytest.mark.parametrize('factors', [(2, 0.5), (1.7, 0.3)])
+def test_dynamic_scaler_follows_the_oracle(hysteresis, factors):
+    growth, backoff = factors
+    rng = np.random.default_rng(hysteresis)
+    kw = dict(initial_scale=2**10, growth_factor=growth, backoff_factor=backoff, growth_interval=4, min_scale=1,
+              max_scale=2**14, hysteresis=hysteresis)
+    a, b = ea.DynamicGradScaler(**kw), O.DynamicGradScalerOracle(**kw)
+    for _ in range(400):
+        found = bool(rng.random() < 0.2)
+        a.update(found)
+        b.update(found)
+        assert a.scale_value == float(b.scale)
+        assert a.scale.dtype == torch.float32 and a.scale.item() == float(b.scale)
+
+
+def test_default_scaler_settings_skip_without_backoff_on_first_overflow():
+    """With the wrapper's default hysteresis of 2 the first overflow only arms the back-off."""
+    sc = ea.DynamicGradScaler(initial_scale=32768, min_scale=1, growth_factor=2, backoff_factor=0.5,
+                              growth_interval=1000, hysteresis=2, max_scale=2**24)
+    sc.update(True)
+    assert sc.scale_value == 32768.0
+    sc.update(True)
+    assert sc.scale_value == 16384.0
+    for _ in range(1000):
+        sc.update(False)
+    assert sc.scale_value == 32768.0
+    sd = sc.state_dict()
+    sc2 = ea.DynamicGradScaler(initial_scale=1.0)
+    sc2.load_state_dict(sd)
+    assert sc2.scale_value == 32768.0 and float(sc.inv_scale) == 1 / 32768.0
+    const = ea.ConstantGradScaler(1.0)
+    const.update(True)
+    assert const.scale_value == 1.0
+
+
+def test_combined_scale_matches_the_oracle():
+    rng = np.random.default_rng(0)
+    for _ in range(2000):
+        loss_scale = float(2.0**rng.integers(0, 20))
+        norm = float(10.0**rng.uniform(-6, 6)) * loss_scale
+        max_norm = float(rng.choice([0.0, 0.5, 1.0, 2.0]))
+        got = ea.calc_combined_scale(loss_scale, norm, max_norm, max_norm > 0)
+        assert got == O.combined_scale(loss_scale, norm if max_norm > 0 else None, max_norm)
+    assert ea.calc_combined_scale(1.0, None, 0.0, False) == -1
+
+
+def test_l2_norm_takes_the_fp32_detour():
+    for sumsq in (0.0, 1.0, 3.0, 123456.789, 1e-12, 6.5e9):
+        assert l2_norm_from_sumsq(sumsq) == float(np.float32(math.sqrt(sumsq)))**2
+    x = (np.random.default_rng(1).standard_normal(5000) * 30).astype(np.float32)
+    assert l2_norm_from_sumsq(O.sumsq(x, O.F32)) == O.l2norm_sq_ref(x, O.F32)
+
+
+def test_hyper_record_scalars():
+    """float64 host scalars narrowed to fp32, as torch narrows Python scalars in tensor ops."""
+    lr, b1, b2, eps, wd, step = 3e-4, 0.9, 0.95, 1e-8, 0.1, 7
+    r = make_hyper_record(lr, b1, b2, eps, wd, step, True, True)[0]
+    bc1, bc2 = 1 - b1**step, 1 - b2**step
+    assert r['decay_mul'] == np.float32(1 - lr * wd) and r['l2_wd'] == 0 and r['flags'] == 0
+    assert r['lerp_w'] == np.float32(1 - b1) and r['beta2'] == np.float32(b2) and r['omb2'] == np.float32(1 - b2)
+    assert r['bc2_sqrt'] == np.float32(math.sqrt(bc2)) and r['neg_step'] == np.float32(-(lr / bc1))
+    assert r['eps'] == np.float32(eps)
+    r = make_hyper_record(lr, b1, b2, eps, wd, step, True, False)[0]                # L2 mode
+    assert r['decay_mul'] == 1.0 and r['l2_wd'] == np.float32(wd) and r['flags'] == _abi.ELX_HYPER_L2
+    r = make_hyper_record(lr, b1, b2, eps, 0.0, step, False, True)[0]               # no decay, no bias correction
+    assert r['decay_mul'] == 1.0 and r['bc2_sqrt'] == 1.0 and r['neg_step'] == np.float32(-lr) and r['flags'] == 0
+    r = make_hyper_record(lr, 0.4, b2, eps, 0.0, 1, True, True)[0]                  # 1-beta1 >= 0.5
+    assert r['flags'] == _abi.ELX_HYPER_LERP_FROM_G
+    assert r['lerp_w'] == np.float32(np.float32(1 - 0.4) - np.float32(1.0))
+
+
+def test_stats_launch_blocks():
+    assert stats_launch_blocks(1) == 1 and stats_launch_blocks(16384) == 1 and stats_launch_blocks(16385) == 2
+    assert stats_launch_blocks(1 << 28) == 1024
+
+
+# ------------------------------------------------------------------------------------------------
+# chunk layout (CPU tensors)
+# ------------------------------------------------------------------------------------------------
+
+
+def test_chunk_append_close_and_valid_end():
+    """test/chunk/test_chunk.py: tensors are packed back to back and keep their values."""
+    a, b, c, d = torch.randn(2, 64), torch.randn(2, 2, 128), torch.randn(128), torch.randn(4, 32)
+    copies = [t.clone() for t in (a, b, c, d)]
+    chunk = ea.Chunk(None, 1024, torch.float, None, shard_device='cpu', temp_device='cpu')
+    assert chunk.chunk_size == 1024 and chunk.chunk_dtype == torch.float and chunk.shard_size == 1024
+    for t in (a, b, c, d):
+        chunk.append_tensor(t)
+    for t, cp in zip((a, b, c, d), copies):
+        assert torch.equal(t, cp)                      # still readable while the chunk is open
+    assert [(i.offset, i.end) for i in chunk.tensors_info.values()] == O.chunk_offsets([128, 512, 128, 128])
+    with pytest.raises(ea.ChunkFullError):
+        chunk.append_tensor(torch.randn(200))
+    chunk.close_chunk()
+    assert chunk.is_replica is False and chunk.is_init is False
+    assert chunk.utilized_size == 896 and chunk.valid_end == 896 == O.valid_end(896, 0, 1024) and chunk.n_valid == 896
+    flat = torch.cat([cp.flatten() for cp in copies])
+    assert torch.equal(chunk.shard[:896], flat) and torch.count_nonzero(chunk.shard[896:]) == 0
+    assert chunk.tensor_state_cnter[ea.TensorState.HOLD] == 4
+
+    full = ea.Chunk(None, 256, torch.float16, None, shard_device='cpu', temp_device='cpu')
+    full.append_tensor(torch.randn(256).half())
+    full.close_chunk()
+    assert full.valid_end == 257 and full.n_valid == 256              # sentinel of a completely used shard
+    with pytest.raises(AssertionError):
+        full.append_tensor(torch.randn(1).half())                     # closed
+    other = ea.Chunk(None, 256, torch.float, None, shard_device='cpu', temp_device='cpu')
+    with pytest.raises(AssertionError):
+        other.append_tensor(torch.randn(4).half())                    # dtype mismatch
+
+
+def test_chunk_pairing_and_meta_tensors():
+    p = ea.Chunk(None, 100, torch.float16, None, shard_device='cpu')
+    o = ea.Chunk(None, 100, torch.float, None, shard_device='cpu')
+    t16 = nn.Parameter(torch.empty(3, 7, dtype=torch.float16, device='meta'))
+    t32 = torch.empty(3, 7, dtype=torch.float, device='meta')
+    p.append_tensor(t16)
+    o.append_tensor(t32)
+    p.close_chunk()
+    o.close_chunk()
+    p.init_pair(o)
+    assert p.paired_chunk is o and o.paired_chunk is p
+    p.init_pair(o)                                                    # idempotent
+    assert p.tensors_info[t16].end == 21 and torch.count_nonzero(p.shard) == 0
+    third = ea.Chunk(None, 100, torch.float, None, shard_device='cpu')
+    with pytest.raises(AssertionError):
+        p.init_pair(third)
+    with pytest.raises(RuntimeError):                                 # flags come from the HIP kernels only
+        p.update_extra_reduce_info()
+    # a host-resident shard defers the refresh exactly like the reference (chunk.py:416-419)
+    p.optim_update()
+    assert p.optim_sync_flag is False
+
+
+class TinyNet(nn.Module):
+
+    def __init__(self):
+        super().__init__()
+        self.embed = nn.Embedding(20, 16)
+        self.norm = nn.LayerNorm(16)
+        self.fc = nn.Linear(16, 40)
+        self.out = nn.Linear(40, 20, bias=False)
+
+    def forward(self, x):
+        return self.out(torch.relu(self.fc(self.norm(self.embed(x))))).sum()
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+def test_module_builds_paired_chunks(dtype):
+    torch.manual_seed(0)
+    net = TinyNet()
+    originals = {n: p.detach().clone() for n, p in net.named_parameters()}
+    named = [(n, p.numel()) for n, p in net.named_parameters()]
+    sr = ea.greedy_search(named, 1024, dtype, shard_device=torch.device('cpu'))
+    assert [len(pl.name_list) for pl in sr.param_chunk_plans] == [len(g) for g in O.greedy_pack([s for _, s in named], 1024)]
+    module = ea.ElixirModule(net, sr, dtype=dtype)
+    assert module.use_amp == (dtype == torch.float16)
+    for pc in module.param_chunks:
+        oc = pc.paired_chunk
+        assert oc.chunk_dtype == torch.float32 and pc.chunk_dtype == dtype and oc.paired_chunk is pc
+        assert pc.chunk_size == oc.chunk_size == 1024 and pc.valid_end == oc.valid_end
+        # identical offsets in both chunks (module.py:120-127)
+        assert [(i.offset, i.end) for i in pc.tensors_info.values()] == [(i.offset, i.end) for i in oc.tensors_info.values()]
+        assert torch.equal(pc.shard, oc.shard.to(dtype))
+    for name, param in net.named_parameters():
+        pc = module.fetcher.get_one_chunk(param)
+        info = pc.tensors_info[param]
+        assert torch.equal(pc.paired_chunk.shard[info.offset:info.end], originals[name].flatten())    # fp32 master
+        assert param.dtype == dtype and torch.equal(param.data.flatten(), originals[name].flatten().to(dtype))
+    sd = module.state_dict()
+    for name, t in originals.items():
+        assert torch.equal(sd[name], t) and sd[name].dtype == torch.float32
+    assert module.state_dict(from_param=True)['fc.weight'].dtype == dtype
+
+
+def test_optimizer_ranges_groups_and_refusal_to_run_on_cpu():
+    torch.manual_seed(0)
+    net = TinyNet()
+    named = [(n, p.numel()) for n, p in net.named_parameters()]
+    module = ea.ElixirModule(net, ea.greedy_search(named, 1024, torch.float16, shard_device=torch.device('cpu')),
+                             dtype=torch.float16)
+    decay = [p for n, p in net.named_parameters() if p.dim() > 1]
+    exempt = [p for n, p in net.named_parameters() if p.dim() == 1]
+    inner = ea.HybridAdam([dict(params=decay, weight_decay=0.1), dict(params=exempt, weight_decay=0.0, lr=5e-4)], lr=1e-3)
+    opt = ea.ElixirOptimizer(module, inner, initial_scale=64, hysteresis=1, max_norm=1.0)
+    assert isinstance(opt.grad_scaler, ea.DynamicGradScaler) and opt.loss_scale == 64.0
+    assert all(c.l2_norm_flag for c in opt.param_chunk_set)
+    # every real parameter became one zero-size fake parameter with its (begin, end) in the shard
+    assert [len(g['params']) for g in opt.param_groups] == [len(decay), len(exempt)]
+    assert [g['weight_decay'] for g in opt.param_groups] == [0.1, 0.0] and opt.param_groups[1]['lr'] == 5e-4
+    for group, real in zip(opt.param_groups, (decay, exempt)):
+        for fake, p in zip(group['params'], real):
+            assert fake.numel() == 0
+            pc = module.fetcher.get_one_chunk(p)
+            info = pc.tensors_info[p]
+            assert opt.param_to_range[fake] == O.range_pair(info.offset, info.end, 0, pc.shard_size)
+            assert opt.param_to_optim_chunk[fake] is pc.paired_chunk
+    # fp32 / bf16 modules get the constant scaler
+    m32 = ea.ElixirModule(TinyNet(), ea.greedy_search(named, 1024, torch.float32, shard_device=torch.device('cpu')))
+    o32 = ea.ElixirOptimizer(m32, ea.HybridAdam(m32.parameters()))
+    assert isinstance(o32.grad_scaler, ea.ConstantGradScaler) and o32.loss_scale == 1.0
+    with pytest.raises(AssertionError):
+        ea.ElixirOptimizer(m32, ea.HybridAdam(m32.parameters()), max_norm=1.0, norm_type=1.0)
+    # no GPU, no step: the product has no CPU path
+    opt.mark_gradients_scaled()
+    with pytest.raises(RuntimeError, match='HIP'):
+        opt.step()
+    p = nn.Parameter(torch.zeros(4))
+    p.grad = torch.ones(4)
+    with pytest.raises(RuntimeError, match='GPU'):
+        ea.HybridAdam([p]).step()
+    with pytest.raises(NotImplementedError):
+        ea.HybridAdam([p], nvme_offload_fraction=0.5)
+
+
+def test_land_gradients_moves_grads_into_the_shards_on_cpu():
+    torch.manual_seed(0)
+    net = TinyNet()
+    named = [(n, p.numel()) for n, p in net.named_parameters()]
+    module = ea.ElixirModule(net, ea.greedy_search(named, 1024, torch.float32, shard_device=torch.device('cpu')))
+    loss = module(torch.randint(0, 20, (4, 8)))
+    loss.backward()
+    grads = {n: p.grad.detach().clone() for n, p in net.named_parameters()}
+    module.land_gradients(sync=False)
+    for name, param in net.named_parameters():
+        pc = module.fetcher.get_one_chunk(param)
+        info = pc.tensors_info[param]
+        assert torch.equal(pc.shard[info.offset:info.end], grads[name].flatten())
+        assert torch.count_nonzero(pc.shard[pc.utilized_size:]) == 0
+
+
+def test_workload_shapes():
+    for fn, tensors, total in ((S.gpt2_shapes, 148, 124_439_808), (S.opt_shapes, 388, 1_315_758_080),
+                               (S.llama_shapes, 291, 6_738_415_616)):
+        sh = fn()
+        assert len(sh) == tensors and sum(S.numel(s) for _, s in sh) == total
+        assert len({n for n, _ in sh}) == tensors
+
+
+def test_bench_refuses_more_than_one_gpu():
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--gpus', '2'], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True)
+    assert proc.returncode != 0 and 'ONE GPU' in proc.stderr
