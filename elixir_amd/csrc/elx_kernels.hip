@@ -11,16 +11,18 @@
 // Shape of the update launch, as measured on MI355X.  The update moves 14 B in and 14 B out per
 // element over four in-place regions.  HBM serves such a read/write mix best when the set of
 // addresses in flight is a tight, orderly moving window that is only just deep enough to cover
-// the memory latency; deeper queues cost bandwidth (full occupancy: ~5.5 TB/s; 40-60 KB in flight
-// per compute unit: 6.2-6.5 TB/s; a plain copy peaks at ~6.65 TB/s the same way, write-only traffic
-// falls from 7.2 to 6.2 TB/s between a shallow and a full queue).  Hence:
-//   * one wavefront per workgroup, one 512-element tile per workgroup, tiles handed out in
-//     address order by the dispatcher (a persistent grid-stride loop is much slower here);
+// the memory latency; deeper queues cost bandwidth (full occupancy: ~5.5 TB/s; about 40 KB in
+// flight per compute unit: 6.7 TB/s; a plain copy peaks at ~6.65 TB/s the same way, write-only
+// traffic falls from 7.2 to 6.2 TB/s between a shallow and a full queue).  Hence:
+//   * one wavefront per workgroup, one 256-element tile per workgroup (one access per stream per
+//     lane), tiles handed out in address order by the dispatcher (a persistent grid-stride loop is
+//     much slower here, and so are wider workgroups or more accesses per lane);
+//   * the common case is one straight line of code: with two or three wavefronts per SIMD there
+//     is nothing to hide a branch, a conditional load or a late table lookup behind;
 //   * every access is a fully coalesced 128-bit (fp32) / 64-bit (16-bit types) per-lane access,
 //     so one wavefront instruction covers one contiguous 1 KiB / 512 B span;
 //   * the number of resident workgroups per compute unit is capped through a dynamic LDS
-//     reservation (default 10: each wavefront spends part of its short life fetching its chunk
-//     record, so about 8 of them have memory requests in flight), not by the register file;
+//     reservation (default 12), not by the register file;
 //   * loads carry the non-temporal hint, stores go out non-temporal at agent scope.
 //
 // Arithmetic contract (what the parity tests pin): fp32 throughout, IEEE division and square
@@ -36,11 +38,11 @@ namespace {
 
 constexpr int kWave = 64;                              // one wavefront per update workgroup
 constexpr int kVec = 4;                                // elements per lane per access
-constexpr int kUnroll = 2;                             // independent accesses per lane per stream
+constexpr int kUnroll = 1;                             // independent accesses per lane per stream
 constexpr uint32_t kSpan = kWave * kVec;               // elements one wavefront access covers
-constexpr uint32_t kTile = kSpan * kUnroll;            // 512 elements per tile
+constexpr uint32_t kTile = kSpan * kUnroll;            // 256 elements per tile
 constexpr uint32_t kLdsPerCu = 160u * 1024u;           // gfx950
-constexpr uint32_t kDefaultBlocksPerCu = 10;
+constexpr uint32_t kDefaultBlocksPerCu = 12;
 constexpr uint32_t kMinBlocksPerCu = 3;                // keeps the reservation below 64 KiB
 constexpr uint32_t kMaxBlocksPerCu = 32;
 
@@ -167,19 +169,71 @@ struct Unscale {
     int mode;
 };
 
+// One element, with the three launch-uniform choices (unscale mode, L2 vs decoupled decay, which
+// end the lerp starts from) fixed at compile time: the tile loop below is then straight-line code.
+// With only two or three wavefronts per SIMD there is nothing to hide a branch behind.
+template <int MODE, bool L2, bool LERP_FROM_G>
+__device__ __forceinline__ void adam_elem_fixed(float g, float &p, float &m, float &v, const Hyper &h,
+                                                const Unscale &us) {
+    if (MODE == kDivMulInv)
+        g = g * us.inv_scale;
+    else if (MODE == kDivTrue)
+        g = g / us.div_scale;
+    p = p * h.decay_mul;                                   // AdamW: p *= 1 - lr*wd (1.0f otherwise)
+    if (L2) g = fmaf(h.l2_wd, p, g);                       // L2: g += wd*p
+    const float diff = g - m;
+    m = fmaf(h.lerp_w, diff, LERP_FROM_G ? g : m);         // m.lerp_(g, 1-beta1)
+    v = fmaf(h.omb2 * g, g, v * h.beta2);                  // v.mul_(beta2).addcmul_(g, g, 1-beta2)
+    const float denom = sqrtf(v) / h.bc2_sqrt + h.eps;     // sqrt(v)/sqrt(bc2) + eps
+    p = p + (h.neg_step * m) / denom;                      // p.addcdiv_(m, denom, -lr/bc1)
+}
+
+// The same element with the choices read at run time (the element-by-element path).
 __device__ __forceinline__ void adam_elem(float g, float &p, float &m, float &v, const Hyper &h, const Unscale &us) {
     if (us.mode == kDivMulInv)
         g = g * us.inv_scale;
     else if (us.mode == kDivTrue)
         g = g / us.div_scale;
-    p = p * h.decay_mul;                                   // AdamW: p *= 1 - lr*wd (1.0f otherwise)
-    if (h.flags & ELX_HYPER_L2) g = fmaf(h.l2_wd, p, g);  // L2: g += wd*p
+    p = p * h.decay_mul;
+    if (h.flags & ELX_HYPER_L2) g = fmaf(h.l2_wd, p, g);
     const float diff = g - m;
     const float base = (h.flags & ELX_HYPER_LERP_FROM_G) ? g : m;
-    m = fmaf(h.lerp_w, diff, base);                        // m.lerp_(g, 1-beta1)
-    v = fmaf(h.omb2 * g, g, v * h.beta2);                  // v.mul_(beta2).addcmul_(g, g, 1-beta2)
-    const float denom = sqrtf(v) / h.bc2_sqrt + h.eps;     // sqrt(v)/sqrt(bc2) + eps
-    p = p + (h.neg_step * m) / denom;                      // p.addcdiv_(m, denom, -lr/bc1)
+    m = fmaf(h.lerp_w, diff, base);
+    v = fmaf(h.omb2 * g, g, v * h.beta2);
+    const float denom = sqrtf(v) / h.bc2_sqrt + h.eps;
+    p = p + (h.neg_step * m) / denom;
+}
+
+template <int GD, int MODE, bool L2, bool LERP_FROM_G>
+__device__ __forceinline__ void tile_math(const typename Elem<GD>::vec4 (&G)[kUnroll], f32x4 (&P)[kUnroll],
+                                          f32x4 (&M)[kUnroll], f32x4 (&V)[kUnroll], const Hyper &h, const Unscale &us) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+        for (int k = 0; k < kVec; ++k) {
+            float g = Elem<GD>::to_f32(G[u][k]);
+            float p = P[u][k], m = M[u][k], v = V[u][k];
+            adam_elem_fixed<MODE, L2, LERP_FROM_G>(g, p, m, v, h, us);
+            P[u][k] = p;
+            M[u][k] = m;
+            V[u][k] = v;
+        }
+    }
+}
+
+template <int GD, int MODE>
+__device__ __forceinline__ void tile_math_flags(const typename Elem<GD>::vec4 (&G)[kUnroll], f32x4 (&P)[kUnroll],
+                                                f32x4 (&M)[kUnroll], f32x4 (&V)[kUnroll], const Hyper &h,
+                                                const Unscale &us) {
+    const bool l2 = h.flags & ELX_HYPER_L2, from_g = h.flags & ELX_HYPER_LERP_FROM_G;
+    if (!l2 && !from_g)
+        tile_math<GD, MODE, false, false>(G, P, M, V, h, us);
+    else if (l2 && !from_g)
+        tile_math<GD, MODE, true, false>(G, P, M, V, h, us);
+    else if (!l2 && from_g)
+        tile_math<GD, MODE, false, true>(G, P, M, V, h, us);
+    else
+        tile_math<GD, MODE, true, true>(G, P, M, V, h, us);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -300,43 +354,80 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
     const ElxChunk c = load_chunk_row(chunks + ci);
     const uint64_t base = (uint64_t)local_tile * kTile;
     if (base >= c.n_alloc) return;    // cannot happen with checked tables
-    const uint64_t left = c.n_alloc - base;
-    const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
-    const bool whole = (tile_n == kTile) && !scalar_only;
-
-    if (refresh_only || base >= c.n_valid) {    // nothing to update in this tile
-        if (whole)
-            tile_refresh_vec<LD>(c, base);
-        else
-            tile_scalar<GD, LD>(c, base, tile_n, 0, segs, hypers, us, true);
-        return;
-    }
 
     typedef typename Elem<GD>::vec4 gvec;
     typedef typename Elem<GD>::scalar gscalar;
-    gvec G[kUnroll];
-    f32x4 P[kUnroll], M[kUnroll], V[kUnroll];
-    const __amdgpu_buffer_rsrc_t pr = tile_rsrc(c.master + base, kTile * sizeof(float));
-    const __amdgpu_buffer_rsrc_t mr = tile_rsrc(c.m + base, kTile * sizeof(float));
-    const __amdgpu_buffer_rsrc_t vr = tile_rsrc(c.v + base, kTile * sizeof(float));
-    if (whole) {
+
+    // ---- the common case: a whole tile inside the valid head of the shard ---------------------
+    // Kept as one straight line (loads, table lookups, arithmetic, stores): with two or three
+    // wavefronts per SIMD there is nothing to hide a detour behind.
+    if (!scalar_only && !refresh_only && base + kTile <= c.n_valid) {
+        const __amdgpu_buffer_rsrc_t pr = tile_rsrc(c.master + base, kTile * sizeof(float));
+        const __amdgpu_buffer_rsrc_t mr = tile_rsrc(c.m + base, kTile * sizeof(float));
+        const __amdgpu_buffer_rsrc_t vr = tile_rsrc(c.v + base, kTile * sizeof(float));
+        // a NULL gradient reads as zero: an empty buffer returns 0 for every lane, without a branch
+        const __amdgpu_buffer_rsrc_t gr =
+            c.grad ? tile_rsrc(reinterpret_cast<const gscalar *>(c.grad) + base, kTile * sizeof(gscalar))
+                   : tile_rsrc(c.master, 0);
+        gvec G[kUnroll];
+        f32x4 P[kUnroll], M[kUnroll], V[kUnroll];
         // issue every load of the tile before looking at the segment table: the table lookups
         // below then overlap the memory latency
-        if (c.grad) {
-            const __amdgpu_buffer_rsrc_t gr = tile_rsrc(reinterpret_cast<const gscalar *>(c.grad) + base, kTile * sizeof(gscalar));
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) G[u] = TileIo<gvec>::load(gr, (threadIdx.x + u * kWave) * sizeof(gvec));
-        }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
+            G[u] = TileIo<gvec>::load(gr, (threadIdx.x + u * kWave) * sizeof(gvec));
             const uint32_t off = (threadIdx.x + u * kWave) * sizeof(f32x4);
             P[u] = TileIo<f32x4>::load(pr, off);
             M[u] = TileIo<f32x4>::load(mr, off);
             V[u] = TileIo<f32x4>::load(vr, off);
         }
+        // first segment of the chunk that ends after the start of the tile
+        uint32_t s = c.seg_begin, s_hi = c.seg_end;
+        while (s < s_hi) {
+            const uint32_t mid = (s + s_hi) >> 1;
+            if (segs[mid].end > base)
+                s_hi = mid;
+            else
+                s = mid + 1;
+        }
+        const bool has = s < c.seg_end;
+        const uint64_t sb = has ? segs[s].begin : ~0ull;
+        const uint64_t se = has ? segs[s].end : 0ull;
+        if (has && sb <= base && se >= base + kTile) {
+            const Hyper h = load_hyper(hypers + segs[s].hyper);
+            if (us.mode == kDivMulInv)
+                tile_math_flags<GD, kDivMulInv>(G, P, M, V, h, us);
+            else if (us.mode == kDivTrue)
+                tile_math_flags<GD, kDivTrue>(G, P, M, V, h, us);
+            else
+                tile_math_flags<GD, kDivNone>(G, P, M, V, h, us);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const uint32_t off = (threadIdx.x + u * kWave) * sizeof(f32x4);
+                TileIo<f32x4>::store(pr, off, P[u]);
+                TileIo<f32x4>::store(mr, off, M[u]);
+                TileIo<f32x4>::store(vr, off, V[u]);
+            }
+            store_lowp_vec<LD>(c, base, P);
+            return;
+        }
+        if (!has || sb >= base + kTile) {    // inside the valid head but owned by no segment
+            store_lowp_vec<LD>(c, base, P);
+            return;
+        }
+        // the tile straddles a segment boundary: redo it element by element below
     }
 
-    // first segment of the chunk that ends after the start of the tile
+    // ---- everything else ------------------------------------------------------------------------
+    const uint64_t left = c.n_alloc - base;
+    const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
+    if (refresh_only || base >= c.n_valid) {    // nothing to update in this tile
+        if (tile_n == kTile && !scalar_only)
+            tile_refresh_vec<LD>(c, base);
+        else
+            tile_scalar<GD, LD>(c, base, tile_n, 0, segs, hypers, us, true);
+        return;
+    }
     uint32_t s = c.seg_begin, s_hi = c.seg_end;
     while (s < s_hi) {
         const uint32_t mid = (s + s_hi) >> 1;
@@ -345,37 +436,7 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
         else
             s = mid + 1;
     }
-    const bool has = s < c.seg_end;
-    const uint64_t sb = has ? segs[s].begin : ~0ull;
-    const uint64_t se = has ? segs[s].end : 0ull;
-
-    if (whole && has && sb <= base && se >= base + kTile) {
-        const Hyper h = load_hyper(hypers + segs[s].hyper);
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-            for (int k = 0; k < kVec; ++k) {
-                float g = c.grad ? Elem<GD>::to_f32(G[u][k]) : 0.0f;
-                float p = P[u][k], m = M[u][k], v = V[u][k];
-                adam_elem(g, p, m, v, h, us);
-                P[u][k] = p;
-                M[u][k] = m;
-                V[u][k] = v;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const uint32_t off = (threadIdx.x + u * kWave) * sizeof(f32x4);
-            TileIo<f32x4>::store(pr, off, P[u]);
-            TileIo<f32x4>::store(mr, off, M[u]);
-            TileIo<f32x4>::store(vr, off, V[u]);
-        }
-        store_lowp_vec<LD>(c, base, P);
-    } else if (whole && (!has || sb >= base + kTile)) {
-        store_lowp_vec<LD>(c, base, P);    // inside the valid head but owned by no segment
-    } else {
-        tile_scalar<GD, LD>(c, base, tile_n, s, segs, hypers, us, false);
-    }
+    tile_scalar<GD, LD>(c, base, tile_n, s, segs, hypers, us, false);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -166,7 +166,7 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
  *   lowp_out = round-to-nearest-even(master)                       -- chunk.py:414
  * Replaces the inner optimizer's step over the fake parameters plus Chunk.optim_update.
  *   total_tiles, uniform_tiles_per_chunk   as returned by elx_check_tables for these tables
- *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (10).
+ *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (12).
  *                  The update streams best with a shallow, orderly queue of memory requests.
  */
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
