@@ -30,7 +30,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg',
            'elx_sizeof_hyper', 'elx_sizeof_stats', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
-           'elx_writeback_mt')
+           'elx_writeback_mt', 'elx_refresh_piece_elems')
 
 
 class ElxError(RuntimeError):
@@ -59,7 +59,8 @@ def load() -> ctypes.CDLL:
     L.elx_version.argtypes = []
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
-    for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats'):
+    for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
+                 'elx_refresh_piece_elems'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -70,7 +71,7 @@ def load() -> ctypes.CDLL:
     L.elx_adam_step_mt.restype = cint
     L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_writeback_mt.restype = cint
-    L.elx_writeback_mt.argtypes = [vp, u32, u64, u32, cint, u32, u32, vp]
+    L.elx_writeback_mt.argtypes = [vp, u32, cint, u32, u32, vp]
 
     if L.elx_version() != ELX_ABI_VERSION:
         raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
@@ -99,7 +100,7 @@ def _np_ptr(a: Optional[np.ndarray]):
 
 
 class TableInfo(tuple):
-    """(total_tiles, uniform_tiles_per_chunk, all_aligned16) as reported by elx_check_tables."""
+    """(total_tiles, max_tiles_per_chunk, all_aligned16) as reported by elx_check_tables."""
     __slots__ = ()
 
     @property
@@ -107,7 +108,7 @@ class TableInfo(tuple):
         return self[0]
 
     @property
-    def uniform_tiles(self) -> int:
+    def max_tiles(self) -> int:
         return self[1]
 
     @property
@@ -121,18 +122,18 @@ class TableInfo(tuple):
 
 def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, grad_dtype: int,
                  lowp_dtype: int) -> TableInfo:
-    """Validate host tables; returns (total_tiles, uniform_tiles_per_chunk, all_aligned16)."""
+    """Validate host tables; returns (total_tiles, max_tiles_per_chunk, all_aligned16)."""
     assert chunks.dtype == CHUNK_DTYPE
     n_segs = 0 if segs is None else len(segs)
     if n_segs:
         assert segs.dtype == SEG_DTYPE
     tiles = ctypes.c_uint64(0)
-    uniform = ctypes.c_uint32(0)
+    max_tiles = ctypes.c_uint32(0)
     aligned = ctypes.c_int(0)
     code = load().elx_check_tables(_np_ptr(chunks), len(chunks), _np_ptr(segs), n_segs, n_hypers, grad_dtype, lowp_dtype,
-                                   ctypes.byref(tiles), ctypes.byref(uniform), ctypes.byref(aligned))
+                                   ctypes.byref(tiles), ctypes.byref(max_tiles), ctypes.byref(aligned))
     check('elx_check_tables', code)
-    return TableInfo((int(tiles.value), int(uniform.value), bool(aligned.value)))
+    return TableInfo((int(tiles.value), int(max_tiles.value), bool(aligned.value)))
 
 
 def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_partials: int, d_stats: int,
@@ -143,15 +144,22 @@ def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chun
 
 
 def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int, info: TableInfo,
-                 div_scale: float, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int, stream: int) -> None:
+                 div_scale: float, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int, stream: int,
+                 flat_grid: bool = False) -> None:
+    """2-D grid (max tiles per chunk, chunks) unless ``flat_grid`` or there are too many chunks."""
+    grid_tiles = 0 if (flat_grid or n_chunks > 65535) else info.max_tiles
     check('elx_adam_step_mt',
-          load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles,
-                                  info.uniform_tiles, div_scale, grad_dtype, lowp_dtype, info.flags, blocks_per_cu,
-                                  stream))
+          load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles, grid_tiles,
+                                  div_scale, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
 
 
-def writeback_mt(d_chunks: int, n_chunks: int, info: TableInfo, lowp_dtype: int, blocks_per_cu: int,
-                 stream: int) -> None:
+def refresh_piece_elems() -> int:
+    return int(load().elx_refresh_piece_elems())
+
+
+def writeback_mt(d_chunks: int, n_chunks: int, lowp_dtype: int, max_elems: int, aligned: bool, stream: int) -> None:
+    """``max_elems``: the largest n_alloc among the records (sizes the grid)."""
+    piece = refresh_piece_elems()
+    blocks = max(1, min(4096, (max_elems + piece - 1) // piece))
     check('elx_writeback_mt',
-          load().elx_writeback_mt(d_chunks, n_chunks, info.total_tiles, info.uniform_tiles, lowp_dtype, info.flags,
-                                  blocks_per_cu, stream))
+          load().elx_writeback_mt(d_chunks, n_chunks, lowp_dtype, blocks, 0 if aligned else ELX_FLAG_SCALAR_ONLY, stream))

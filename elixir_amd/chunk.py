@@ -362,7 +362,7 @@ class Chunk:
             info = _abi.check_tables(row, None, 0, code, code)
             table = DeviceTable(row, self.shard_device)
             stream = torch.cuda.current_stream(self.shard_device).cuda_stream
-            _abi.writeback_mt(table.ptr, 1, info, code, 0, stream)
+            _abi.writeback_mt(table.ptr, 1, code, self.shard_size, info.aligned, stream)
             # keep the table alive until the launch has consumed it
             self._workspace['wb_table'] = table
             self.optim_sync_flag = True

@@ -329,13 +329,13 @@ template <int GD, int LD>
 __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks, uint32_t n_chunks,
                                                           const ElxSeg *__restrict__ segs,
                                                           const ElxHyper *__restrict__ hypers,
-                                                          uint32_t uniform_tiles_per_chunk, Unscale us,
-                                                          uint32_t scalar_only, uint32_t refresh_only) {
-    // chunk that owns this tile: with a uniform tile count per chunk the grid is (tiles, chunks)
-    // and nothing has to be looked up; otherwise the grid is flat and the owner is the last chunk
+                                                          uint32_t grid_tiles_per_chunk, Unscale us,
+                                                          uint32_t scalar_only) {
+    // chunk that owns this tile: on the 2-D grid (tiles, chunks) nothing has to be looked up
+    // (workgroups beyond a chunk's last tile exit); on the flat grid the owner is the last chunk
     // whose tile_begin is <= the tile index (all uniform -> scalar loads)
     uint32_t ci, local_tile;
-    if (uniform_tiles_per_chunk) {
+    if (grid_tiles_per_chunk) {
         ci = blockIdx.y;
         local_tile = blockIdx.x;
     } else {
@@ -353,7 +353,7 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
     }
     const ElxChunk c = load_chunk_row(chunks + ci);
     const uint64_t base = (uint64_t)local_tile * kTile;
-    if (base >= c.n_alloc) return;    // cannot happen with checked tables
+    if (base >= c.n_alloc) return;    // a shorter chunk on the 2-D grid
 
     typedef typename Elem<GD>::vec4 gvec;
     typedef typename Elem<GD>::scalar gscalar;
@@ -361,7 +361,7 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
     // ---- the common case: a whole tile inside the valid head of the shard ---------------------
     // Kept as one straight line (loads, table lookups, arithmetic, stores): with two or three
     // wavefronts per SIMD there is nothing to hide a detour behind.
-    if (!scalar_only && !refresh_only && base + kTile <= c.n_valid) {
+    if (!scalar_only && base + kTile <= c.n_valid) {
         const __amdgpu_buffer_rsrc_t pr = tile_rsrc(c.master + base, kTile * sizeof(float));
         const __amdgpu_buffer_rsrc_t mr = tile_rsrc(c.m + base, kTile * sizeof(float));
         const __amdgpu_buffer_rsrc_t vr = tile_rsrc(c.v + base, kTile * sizeof(float));
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
     // ---- everything else ------------------------------------------------------------------------
     const uint64_t left = c.n_alloc - base;
     const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
-    if (refresh_only || base >= c.n_valid) {    // nothing to update in this tile
+    if (base >= c.n_valid) {    // padding inside an update chunk: refresh only
         if (tile_n == kTile && !scalar_only)
             tile_refresh_vec<LD>(c, base);
         else
@@ -437,6 +437,50 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
             s = mid + 1;
     }
     tile_scalar<GD, LD>(c, base, tile_n, s, segs, hypers, us, false);
+}
+
+// ---------------------------------------------------------------------------------------------
+// low-precision refresh alone
+// ---------------------------------------------------------------------------------------------
+
+// lowp_out[0, n_alloc) = round-to-nearest-even(master) for every chunk.  4 bytes in, 2 bytes out per
+// element: a read-dominated stream that wants wide workgroups and a deep queue, the opposite of
+// the update.  Grid (blocks_per_chunk, n_chunks), each workgroup strides over 4096-element pieces.
+constexpr int kRefreshThreads = 256;
+constexpr int kRefreshUnroll = 4;
+constexpr uint32_t kRefreshPiece = kRefreshThreads * kVec * kRefreshUnroll;
+
+template <int LD>
+__global__ __launch_bounds__(kRefreshThreads) void refresh_kernel(const ElxChunk *__restrict__ chunks,
+                                                                  uint32_t scalar_only) {
+    typedef typename Elem<LD>::vec4 lvec;
+    typedef typename Elem<LD>::scalar lscalar;
+    const ElxChunk c = chunks[blockIdx.y];
+    if (!c.lowp_out) return;
+    lscalar *out = reinterpret_cast<lscalar *>(c.lowp_out);
+    const uint64_t n = c.n_alloc;
+    const uint64_t pieces = (n + kRefreshPiece - 1) / kRefreshPiece;
+    for (uint64_t piece = blockIdx.x; piece < pieces; piece += gridDim.x) {
+        const uint64_t base = piece * kRefreshPiece;
+        if (base + kRefreshPiece <= n && !scalar_only) {
+            const f32x4 *pp = reinterpret_cast<const f32x4 *>(c.master + base) + threadIdx.x;
+            lvec *lp = reinterpret_cast<lvec *>(out + base) + threadIdx.x;
+            f32x4 P[kRefreshUnroll];
+#pragma unroll
+            for (int u = 0; u < kRefreshUnroll; ++u) P[u] = ld_stream(pp + u * kRefreshThreads);
+#pragma unroll
+            for (int u = 0; u < kRefreshUnroll; ++u) {
+                lvec L;
+#pragma unroll
+                for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
+                __builtin_nontemporal_store(L, lp + u * kRefreshThreads);
+            }
+        } else {
+            const uint64_t left = n - base;
+            const uint32_t cnt = left < kRefreshPiece ? (uint32_t)left : kRefreshPiece;
+            for (uint32_t i = threadIdx.x; i < cnt; i += kRefreshThreads) out[base + i] = Elem<LD>::from_f32(c.master[base + i]);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -572,21 +616,19 @@ int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes) {
 
 template <int GD, int LD>
 int launch_step(uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
-                const ElxSeg *segs, const ElxHyper *hypers, uint32_t uniform_tiles, Unscale us, uint32_t scalar_only,
-                uint32_t refresh_only) {
-    const dim3 grid = uniform_tiles ? dim3(uniform_tiles, n_chunks) : dim3(tiles);
+                const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, uint32_t scalar_only) {
+    const dim3 grid = grid_tiles ? dim3(grid_tiles, n_chunks) : dim3(tiles);
     hipLaunchKernelGGL((adam_step_kernel<GD, LD>), grid, dim3(kWave), lds, st, chunks, n_chunks, segs, hypers,
-                       uniform_tiles, us, scalar_only, refresh_only);
+                       grid_tiles, us, scalar_only);
     return (int)hipGetLastError();
 }
 
 int dispatch_step(int gd, int ld, uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks,
-                  uint32_t n_chunks, const ElxSeg *segs, const ElxHyper *hypers, uint32_t uniform_tiles, Unscale us,
-                  uint32_t scalar_only, uint32_t refresh_only) {
+                  uint32_t n_chunks, const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us,
+                  uint32_t scalar_only) {
 #define ELX_CASE(G, L)                                                                                         \
     if (gd == G && ld == L)                                                                                    \
-        return launch_step<G, L>(tiles, lds, st, chunks, n_chunks, segs, hypers, uniform_tiles, us, scalar_only, \
-                                 refresh_only);
+        return launch_step<G, L>(tiles, lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -627,18 +669,18 @@ const char *elx_strerror(int code) {
 
 int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *h_segs, uint32_t n_segs,
                      uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles,
-                     uint32_t *uniform_tiles_per_chunk, int *all_aligned16) {
-    if (!h_chunks || !total_tiles || !uniform_tiles_per_chunk || !all_aligned16 || (n_segs && !h_segs)) return ELX_E_NULL;
+                     uint32_t *max_tiles_per_chunk, int *all_aligned16) {
+    if (!h_chunks || !total_tiles || !max_tiles_per_chunk || !all_aligned16 || (n_segs && !h_segs)) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u) return ELX_E_SIZE;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
     const uintptr_t gmask = elem_size(grad_dtype) - 1;
     uint64_t tiles = 0;
     int aligned = 1;
-    uint64_t uniform = (h_chunks[0].n_alloc + kTile - 1) / kTile;
+    uint64_t max_tiles = 0;
     for (uint32_t i = 0; i < n_chunks; ++i) {
         const ElxChunk &c = h_chunks[i];
-        if ((c.n_alloc + kTile - 1) / kTile != uniform) uniform = 0;
+        if ((c.n_alloc + kTile - 1) / kTile > max_tiles) max_tiles = (c.n_alloc + kTile - 1) / kTile;
         if (!c.master || !c.m || !c.v) return ELX_E_NULL;
         if (c.lowp_out && lowp_dtype == ELX_NONE) return ELX_E_DTYPE;
         if (c.n_alloc == 0) return ELX_E_SIZE;
@@ -663,7 +705,7 @@ int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *
     }
     if (tiles > 0x7FFFFFFFull) return ELX_E_SIZE;    // one workgroup per tile
     *total_tiles = tiles;
-    *uniform_tiles_per_chunk = (uint32_t)uniform;
+    *max_tiles_per_chunk = (uint32_t)max_tiles;
     *all_aligned16 = aligned;
     return 0;
 }
@@ -695,12 +737,13 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
 }
 
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
-                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles, uint32_t uniform_tiles_per_chunk,
+                     const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles, uint32_t grid_tiles_per_chunk,
                      float div_scale, int grad_dtype, int lowp_dtype, uint32_t flags, uint32_t blocks_per_cu,
                      void *stream) {
     if (!d_chunks || (n_segs && (!d_segs || !d_hypers))) return ELX_E_NULL;
-    if (n_chunks == 0 || total_tiles == 0 || total_tiles > 0x7FFFFFFFull || (n_segs && n_hypers == 0)) return ELX_E_SIZE;
-    if (uniform_tiles_per_chunk && (uint64_t)uniform_tiles_per_chunk * n_chunks != total_tiles) return ELX_E_TILES;
+    if (n_chunks == 0 || n_chunks > 65535u || total_tiles == 0 || total_tiles > 0x7FFFFFFFull || (n_segs && n_hypers == 0))
+        return ELX_E_SIZE;
+    if (grid_tiles_per_chunk && (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
     uint32_t lds = 0;
@@ -718,23 +761,25 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
         }
     }
     return dispatch_step(grad_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
-                         d_segs, d_hypers, uniform_tiles_per_chunk, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 0u);
+                         d_segs, d_hypers, grid_tiles_per_chunk, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
-int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles, uint32_t uniform_tiles_per_chunk,
-                     int lowp_dtype, uint32_t flags, uint32_t blocks_per_cu, void *stream) {
+int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype, uint32_t blocks_per_chunk,
+                     uint32_t flags, void *stream) {
     if (!d_chunks) return ELX_E_NULL;
-    if (n_chunks == 0 || total_tiles == 0 || total_tiles > 0x7FFFFFFFull) return ELX_E_SIZE;
-    if (uniform_tiles_per_chunk && (uint64_t)uniform_tiles_per_chunk * n_chunks != total_tiles) return ELX_E_TILES;
-    if (!is_lowp_or_f32(lowp_dtype)) return ELX_E_DTYPE;
-    uint32_t lds = 0;
-    if (int rc = occupancy_reservation(blocks_per_cu, &lds)) return rc;
-    Unscale us;
-    us.div_scale = -1.0f;
-    us.inv_scale = 1.0f;
-    us.mode = kDivNone;
-    return dispatch_step(lowp_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
-                         nullptr, nullptr, uniform_tiles_per_chunk, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u, 1u);
+    if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > 65535u) return ELX_E_SIZE;
+    const dim3 grid(blocks_per_chunk, n_chunks);
+    const uint32_t so = (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u;
+    hipStream_t st = (hipStream_t)stream;
+    switch (lowp_dtype) {
+        case ELX_F32: hipLaunchKernelGGL((refresh_kernel<ELX_F32>), grid, dim3(kRefreshThreads), 0, st, d_chunks, so); break;
+        case ELX_F16: hipLaunchKernelGGL((refresh_kernel<ELX_F16>), grid, dim3(kRefreshThreads), 0, st, d_chunks, so); break;
+        case ELX_BF16: hipLaunchKernelGGL((refresh_kernel<ELX_BF16>), grid, dim3(kRefreshThreads), 0, st, d_chunks, so); break;
+        default: return ELX_E_DTYPE;
+    }
+    return (int)hipGetLastError();
 }
+
+uint32_t elx_refresh_piece_elems(void) { return kRefreshPiece; }
 
 }    // extern "C"

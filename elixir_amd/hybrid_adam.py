@@ -22,6 +22,7 @@ import torch
 
 from . import _abi
 from .chunk import Chunk, DeviceTable, dtype_code
+from .launch_plan import FlatBuffer, LaunchPlan, build_plan
 
 
 def make_hyper_record(lr: float, beta1: float, beta2: float, eps: float, weight_decay: float, step: int,
@@ -70,6 +71,44 @@ class _CachedTable:
         return self.table
 
 
+class _HyperUploader:
+    """Per-step upload of the (tiny) hyper-parameter table without blocking the host: two pinned
+    staging buffers used in turn and an asynchronous copy on the launch stream.  A staging buffer
+    is rewritten two steps after its copy was enqueued; every step waits for the device at least
+    once in between (the readback of the gradient flags), so the copy has long completed."""
+
+    def __init__(self):
+        self.staging: List[torch.Tensor] = []
+        self.dev: Optional[torch.Tensor] = None
+        self.turn = 0
+
+    def upload(self, host: np.ndarray, device: torch.device) -> int:
+        nbytes = host.nbytes
+        if self.dev is None or self.dev.device != device or self.dev.numel() < nbytes:
+            cap = max(4096, nbytes)
+            self.dev = torch.empty(cap, dtype=torch.uint8, device=device)
+            self.staging = [torch.empty(cap, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
+        stage = self.staging[self.turn]
+        self.turn ^= 1
+        stage[:nbytes].numpy()[:] = host.view(np.uint8).reshape(-1)
+        self.dev[:nbytes].copy_(stage[:nbytes], non_blocking=True)
+        return self.dev.data_ptr()
+
+
+class _DevicePlan:
+    """A launch plan and its tables in device memory."""
+
+    def __init__(self, plan: LaunchPlan, device: torch.device):
+        self.plan = plan
+        self.rows = DeviceTable(plan.rows, device) if len(plan.rows) else None
+        self.segs = DeviceTable(plan.segs, device) if len(plan.segs) else None
+        self.refresh = DeviceTable(plan.refresh_rows, device) if plan.refresh_rows is not None else None
+        self.refresh_aligned = True
+        if plan.refresh_rows is not None:
+            self.refresh_aligned = bool(
+                np.all(plan.refresh_rows['lowp_out'] % 16 == 0) and np.all(plan.refresh_rows['master'] % 16 == 0))
+
+
 class ChunkBinding:
     """Where the fake parameters of ``ElixirOptimizer`` live: for each optimizer chunk the paired
     low-precision chunk, the flat m / v buffers and the slices the optimizer owns."""
@@ -99,6 +138,18 @@ class ChunkBinding:
             self.flat_m[chunk] = torch.zeros(chunk.shard_size, dtype=torch.float32, device=chunk.shard_device)
             self.flat_v[chunk] = torch.zeros(chunk.shard_size, dtype=torch.float32, device=chunk.shard_device)
         return self.flat_m[chunk], self.flat_v[chunk]
+
+
+class _Prepared:
+    """Everything a step needs that does not depend on the gradient flags: built while the stats
+    launch is still running, consumed (and only then committed to the optimizer state) by step()."""
+
+    def __init__(self, dplan, hyper_host, grad_code, lowp_code, device, states):
+        self.dplan: _DevicePlan = dplan
+        self.hyper_host: np.ndarray = hyper_host
+        self.grad_code, self.lowp_code, self.device = grad_code, lowp_code, device
+        self.states: List[Dict] = states      # per-parameter state dicts whose 'step' advances on commit
+        self.d_hypers: int = 0
 
 
 class HybridAdam(torch.optim.Optimizer):
@@ -131,17 +182,18 @@ class HybridAdam(torch.optim.Optimizer):
         self.adamw_mode = adamw_mode
         self.blocks_per_cu = 0    # cap on resident update workgroups per compute unit; 0: library default
         self._binding: Optional[ChunkBinding] = None
-        self._chunk_table = _CachedTable()
-        self._seg_table = _CachedTable()
-        self._hyper_table = _CachedTable()
-        self._checked_key = None
-        self._checked = None
+        self._plans: Dict = {}                      # plan key -> _DevicePlan
+        self._hyper_uploader = _HyperUploader()
+        self._prepared: Optional[_Prepared] = None
+        self._bound_entries = None                  # cached walk over the bound fake parameters
 
     # ------------------------------------------------------------------ chunk binding
 
     def bind_chunks(self, ranges: Dict[torch.nn.Parameter, Tuple[Chunk, int, int]]) -> ChunkBinding:
         """Called by ``ElixirOptimizer``: ``ranges[fake_param] = (optim_chunk, begin, end)``."""
         self._binding = ChunkBinding(ranges)
+        self._bound_entries = None
+        self._plans.clear()
         return self._binding
 
     @property
@@ -150,14 +202,51 @@ class HybridAdam(torch.optim.Optimizer):
 
     # ------------------------------------------------------------------ the step
 
-    def _hyper_index(self, hypers: Dict, group: Dict, step: int) -> int:
+    @staticmethod
+    def _group_key(group: Dict, step: int):
         beta1, beta2 = group['betas']
-        key = (group['lr'], beta1, beta2, group['eps'], group['weight_decay'], step, group['bias_correction'])
+        return (group['lr'], beta1, beta2, group['eps'], group['weight_decay'], step, group['bias_correction'])
+
+    def _hyper_index(self, hypers: Dict, group: Dict, step: int) -> int:
+        key = self._group_key(group, step)
         idx = hypers.get(key)
         if idx is None:
             idx = len(hypers)
             hypers[key] = idx
         return idx
+
+    def _device_plan(self, key, buffers_fn, grad_dtype, grad_code, lowp_code, n_hypers, device) -> _DevicePlan:
+        dplan = self._plans.get(key)
+        if dplan is None:
+            if len(self._plans) > 8:
+                self._plans.clear()
+            esize = 4 if grad_dtype == torch.float32 else 2
+            dplan = _DevicePlan(build_plan(buffers_fn(), esize, esize, n_hypers, grad_code, lowp_code), device)
+            self._plans[key] = dplan
+        return dplan
+
+    def prepare_step(self) -> None:
+        """Builds the tables of the next step without touching the optimizer state, so that a caller
+        can overlap this host work with device work whose result decides whether the step happens
+        (``ElixirOptimizer`` calls it between launching and reading the gradient flags).  The next
+        ``step()`` consumes what was prepared; ``discard_prepared()`` drops it."""
+        hypers: Dict = {}
+        if self._binding is not None:
+            self._prepared = self._prepare_bound(hypers)
+        else:
+            self._prepared = self._prepare_standalone(hypers)
+        prep = self._prepared
+        if prep is not None:
+            prep.d_hypers = self._hyper_uploader.upload(prep.hyper_host, prep.device)
+
+    def discard_prepared(self) -> None:
+        self._prepared = None
+
+    def _hyper_table(self, hypers: Dict) -> np.ndarray:
+        return np.concatenate([
+            make_hyper_record(lr, b1, b2, eps, wd, step, bc, self.adamw_mode)
+            for (lr, b1, b2, eps, wd, step, bc) in hypers.keys()
+        ])
 
     @torch.no_grad()
     def step(self, closure=None, div_scale: float = -1):
@@ -165,44 +254,37 @@ class HybridAdam(torch.optim.Optimizer):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
-
-        hypers: Dict = {}
-        if self._binding is not None:
-            launch = self._collect_bound(hypers)
-        else:
-            launch = self._collect_standalone(hypers)
-        if launch is None:
+        if self._prepared is None:
+            self.prepare_step()
+        prep, self._prepared = self._prepared, None
+        if prep is None:
             return loss
-        chunks, segs, grad_code, lowp_code, device = launch
 
-        hyper_host = np.concatenate([
-            make_hyper_record(lr, b1, b2, eps, wd, step, bc, self.adamw_mode)
-            for (lr, b1, b2, eps, wd, step, bc) in hypers.keys()
-        ])
-
-        key = (chunks.tobytes(), segs.tobytes(), len(hyper_host), grad_code, lowp_code)
-        if key != self._checked_key:
-            self._checked = _abi.check_tables(chunks, segs, len(hyper_host), grad_code, lowp_code)
-            self._checked_key = key
-        info = self._checked
-
-        d_chunks = self._chunk_table.get(chunks, device)
-        d_segs = self._seg_table.get(segs, device)
-        d_hypers = self._hyper_table.get(hyper_host, device)
-        stream = torch.cuda.current_stream(device).cuda_stream
-        _abi.adam_step_mt(d_chunks.ptr, len(chunks), d_segs.ptr, len(segs), d_hypers.ptr, len(hyper_host), info,
-                          float(div_scale), grad_code, lowp_code, self.blocks_per_cu, stream)
-        if self._binding is not None and lowp_code != _abi.ELX_NONE:
+        for state in prep.states:    # commit: this step happens
+            state['step'] += 1
+        plan = prep.dplan.plan
+        stream = torch.cuda.current_stream(prep.device).cuda_stream
+        if prep.dplan.rows is not None:
+            _abi.adam_step_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs), prep.d_hypers,
+                              len(prep.hyper_host), plan.info, float(div_scale), prep.grad_code, prep.lowp_code,
+                              self.blocks_per_cu, stream)
+        if prep.dplan.refresh is not None:
+            _abi.writeback_mt(prep.dplan.refresh.ptr, len(plan.refresh_rows), prep.lowp_code, plan.refresh_max_elems,
+                              prep.dplan.refresh_aligned, stream)
+        if self._binding is not None and prep.lowp_code != _abi.ELX_NONE:
             self._binding.fused_writeback = True
         return loss
 
-    def _collect_bound(self, hypers: Dict):
+    # ---- bound to chunk storage
+
+    def _walk_bound(self):
+        """(state dict, group index, chunk index, begin, end) per bound fake parameter, in group order."""
         b = self._binding
-        b.require_gpu()
-        n_chunks = len(b.chunks)
-        chunks = np.zeros(n_chunks, dtype=_abi.CHUNK_DTYPE)
-        per_chunk: List[List[Tuple[int, int, int]]] = [[] for _ in range(n_chunks)]
-        for group in self.param_groups:
+        signature = tuple(len(g['params']) for g in self.param_groups)
+        if self._bound_entries is not None and self._bound_entries[0] == signature:
+            return self._bound_entries[1]
+        entries = []
+        for gi, group in enumerate(self.param_groups):
             for p in group['params']:
                 if p not in b.ranges:
                     raise RuntimeError('a parameter of this optimizer is not part of the bound chunk storage')
@@ -214,40 +296,48 @@ class HybridAdam(torch.optim.Optimizer):
                     # per-tensor views of the flat moments, shaped like the optimizer's slice
                     state['exp_avg'] = flat_m[begin:end]
                     state['exp_avg_sq'] = flat_v[begin:end]
-                state['step'] += 1
-                per_chunk[b.chunk_index[chunk]].append((begin, end, self._hyper_index(hypers, group, state['step'])))
+                entries.append((state, gi, b.chunk_index[chunk], begin, end))
+        self._bound_entries = (signature, entries)
+        return entries
 
-        n_segs = sum(len(x) for x in per_chunk)
-        if n_segs == 0:
+    def _prepare_bound(self, hypers: Dict) -> Optional[_Prepared]:
+        b = self._binding
+        b.require_gpu()
+        entries = self._walk_bound()
+        if not entries:
             return None
-        segs = np.zeros(n_segs, dtype=_abi.SEG_DTYPE)
-        tile = _abi.tile_elems()
-        pos, tiles = 0, 0
+        groups = self.param_groups
+        # hyper record per entry: the (group, step + 1) pair it will be updated with
+        idx_of = [self._hyper_index(hypers, groups[gi], state['step'] + 1) for state, gi, _, _, _ in entries]
         lowp_dtype = b.chunks[0].paired_chunk.chunk_dtype
-        for i, c in enumerate(b.chunks):
-            pc = c.paired_chunk
-            assert pc.chunk_dtype == lowp_dtype, 'all parameter chunks of one optimizer share a dtype'
-            flat_m, flat_v = b.moments(c)
-            row = chunks[i]
-            row['grad'] = 0 if b.zero_grads else pc.shard.data_ptr()
-            row['lowp_out'] = 0 if b.zero_grads else pc.shard.data_ptr()
-            row['master'] = c.shard.data_ptr()
-            row['m'] = flat_m.data_ptr()
-            row['v'] = flat_v.data_ptr()
-            row['n_alloc'] = c.shard_size
-            row['n_valid'] = pc.n_valid
-            row['tile_begin'] = tiles
-            tiles += (c.shard_size + tile - 1) // tile
-            row['seg_begin'] = pos
-            for begin, end, h in sorted(per_chunk[i]):
-                segs[pos] = (begin, end, h, 0)
-                pos += 1
-            row['seg_end'] = pos
-        code = dtype_code(lowp_dtype)
-        return chunks, segs, code, (_abi.ELX_NONE if b.zero_grads else code), b.chunks[0].shard_device
+        grad_code = dtype_code(lowp_dtype)
+        lowp_code = _abi.ELX_NONE if b.zero_grads else grad_code
+        device = b.chunks[0].shard_device
+        shard_ptrs = tuple(c.paired_chunk.shard.data_ptr() for c in b.chunks)
+        key = ('bound', b.zero_grads, tuple(idx_of), shard_ptrs, tuple(c.shard.data_ptr() for c in b.chunks))
 
-    def _collect_standalone(self, hypers: Dict):
-        rows = []
+        def buffers():
+            per_chunk: List[List[Tuple[int, int, int]]] = [[] for _ in b.chunks]
+            for (state, gi, ci, begin, end), h in zip(entries, idx_of):
+                per_chunk[ci].append((begin, end, h))
+            out = []
+            for i, c in enumerate(b.chunks):
+                pc = c.paired_chunk
+                assert pc.chunk_dtype == lowp_dtype, 'all parameter chunks of one optimizer share a dtype'
+                flat_m, flat_v = b.moments(c)
+                shard_ptr = 0 if b.zero_grads else pc.shard.data_ptr()
+                out.append(FlatBuffer(grad=shard_ptr, lowp_out=shard_ptr, master=c.shard.data_ptr(),
+                                      m=flat_m.data_ptr(), v=flat_v.data_ptr(), n_alloc=c.shard_size, n_valid=pc.n_valid,
+                                      segs=sorted(per_chunk[i])))
+            return out
+
+        dplan = self._device_plan(key, buffers, lowp_dtype, grad_code, lowp_code, len(hypers), device)
+        return _Prepared(dplan, self._hyper_table(hypers), grad_code, lowp_code, device, [e[0] for e in entries])
+
+    # ---- standalone, on ordinary parameters
+
+    def _prepare_standalone(self, hypers: Dict) -> Optional[_Prepared]:
+        items = []
         grad_dtype = None
         device = None
         for group in self.param_groups:
@@ -272,27 +362,17 @@ class HybridAdam(torch.optim.Optimizer):
                     state['step'] = 0
                     state['exp_avg'] = torch.zeros_like(p, memory_format=torch.preserve_format)
                     state['exp_avg_sq'] = torch.zeros_like(p, memory_format=torch.preserve_format)
-                state['step'] += 1
-                rows.append((p, state, self._hyper_index(hypers, group, state['step'])))
-        if not rows:
+                n = p.numel()
+                items.append((state, (p.grad.data_ptr(), 0, p.data.data_ptr(), state['exp_avg'].data_ptr(),
+                                      state['exp_avg_sq'].data_ptr(), n, self._hyper_index(hypers, group, state['step'] + 1))))
+        if not items:
             return None
-        chunks = np.zeros(len(rows), dtype=_abi.CHUNK_DTYPE)
-        segs = np.zeros(len(rows), dtype=_abi.SEG_DTYPE)
-        tile = _abi.tile_elems()
-        tiles = 0
-        for i, (p, state, h) in enumerate(rows):
-            n = p.numel()
-            row = chunks[i]
-            row['grad'] = p.grad.data_ptr()
-            row['lowp_out'] = 0
-            row['master'] = p.data.data_ptr()
-            row['m'] = state['exp_avg'].data_ptr()
-            row['v'] = state['exp_avg_sq'].data_ptr()
-            row['n_alloc'] = n
-            row['n_valid'] = n
-            row['tile_begin'] = tiles
-            tiles += (n + tile - 1) // tile
-            row['seg_begin'] = i
-            row['seg_end'] = i + 1
-            segs[i] = (0, n, h, 0)
-        return chunks, segs, dtype_code(grad_dtype), _abi.ELX_NONE, device
+        grad_code = dtype_code(grad_dtype)
+        key = ('standalone', grad_code, tuple(it[1] for it in items))
+
+        def buffers():
+            return [FlatBuffer(grad=g, lowp_out=0, master=p, m=m, v=v, n_alloc=n, n_valid=n, segs=[(0, n, h)])
+                    for _, (g, _, p, m, v, n, h) in items]
+
+        dplan = self._device_plan(key, buffers, grad_dtype, grad_code, _abi.ELX_NONE, len(hypers), device)
+        return _Prepared(dplan, self._hyper_table(hypers), grad_code, _abi.ELX_NONE, device, [it[0] for it in items])

@@ -1,0 +1,98 @@
+"""Host-side planning of the update launch.
+
+The update kernel runs best as a 2-D grid ``(tiles per record, records)`` whose records are
+equal-sized blocks: no lookup to find a tile's owner, very few workgroups without work, and a
+segment table of one or two entries per record.  Runs of pure padding at the end of a shard are
+left out of that launch and refreshed by the wide-workgroup refresh launch instead.
+
+``build_plan`` turns a list of flat buffers (a chunk shard, or a standalone parameter) with their
+segments into
+  * ``rows`` / ``segs``: the ElxChunk / ElxSeg tables of the update launch, one row per block of
+    ``block_elems`` elements that contains at least one valid element;
+  * ``refresh_rows``: ElxChunk rows (lowp_out, master, n_alloc only) for the padding runs, or None.
+"""
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _abi
+
+MAX_ROWS = 32768    # target upper bound on update rows (the grid's y extent must stay below 65536)
+
+
+@dataclass
+class FlatBuffer:
+    """One flat run of elements: a chunk shard pair or a standalone parameter."""
+    grad: int         # device address of the gradients (0: zero gradient)
+    lowp_out: int     # device address of the low-precision copy (0: none)
+    master: int
+    m: int
+    v: int
+    n_alloc: int
+    n_valid: int
+    segs: List[Tuple[int, int, int]] = field(default_factory=list)    # (begin, end, hyper), sorted, disjoint
+
+
+@dataclass
+class LaunchPlan:
+    rows: np.ndarray
+    segs: np.ndarray
+    refresh_rows: Optional[np.ndarray]
+    refresh_max_elems: int
+    block_elems: int
+    info: _abi.TableInfo
+
+
+def _pow2_at_least(x: int) -> int:
+    p = 1
+    while p < x:
+        p <<= 1
+    return p
+
+
+def choose_block_elems(buffers: Sequence[FlatBuffer], tile: int) -> int:
+    """A power-of-two multiple of the tile, at least 16 tiles, so that the launch has at most
+    about MAX_ROWS rows."""
+    total = sum(min(b.n_alloc, b.n_valid + tile) for b in buffers)
+    return max(16 * tile, _pow2_at_least((total + MAX_ROWS // 2 - 1) // (MAX_ROWS // 2)))
+
+
+def build_plan(buffers: Sequence[FlatBuffer], grad_esize: int, lowp_esize: int, n_hypers: int, grad_dtype: int,
+               lowp_dtype: int) -> LaunchPlan:
+    tile = _abi.tile_elems()
+    block = choose_block_elems(buffers, tile)
+    rows, segs, refresh = [], [], []
+    tiles = 0
+    for buf in buffers:
+        assert 0 <= buf.n_valid <= buf.n_alloc
+        # the update covers whole blocks up to the one that holds the last valid element
+        up_end = min(buf.n_alloc, -(-buf.n_valid // block) * block)
+        seg_arr = np.array(buf.segs, dtype=np.int64).reshape(-1, 3)
+        if len(seg_arr):
+            assert np.all(seg_arr[:, 0] < seg_arr[:, 1]) and np.all(seg_arr[1:, 0] >= seg_arr[:-1, 1]), \
+                'segments must be sorted, non-empty and disjoint'
+            assert seg_arr[-1, 1] <= buf.n_valid, 'a segment reaches beyond the valid head of its buffer'
+        for b in range(0, up_end, block):
+            n = min(block, up_end - b)
+            seg_begin = len(segs)
+            if len(seg_arr):
+                lo = int(np.searchsorted(seg_arr[:, 1], b, side='right'))       # first segment ending after b
+                hi = int(np.searchsorted(seg_arr[:, 0], b + n, side='left'))    # first segment starting at/after the end
+                for sb, se, h in seg_arr[lo:hi]:
+                    segs.append((max(int(sb), b) - b, min(int(se), b + n) - b, int(h), 0))
+            rows.append((buf.grad + b * grad_esize if buf.grad else 0, buf.lowp_out + b * lowp_esize if buf.lowp_out else 0,
+                         buf.master + 4 * b, buf.m + 4 * b, buf.v + 4 * b, n, max(0, min(n, buf.n_valid - b)), tiles,
+                         seg_begin, len(segs)))
+            tiles += (n + tile - 1) // tile
+        if buf.lowp_out and up_end < buf.n_alloc:
+            refresh.append((0, buf.lowp_out + up_end * lowp_esize, buf.master + 4 * up_end, buf.master + 4 * up_end,
+                            buf.master + 4 * up_end, buf.n_alloc - up_end, 0, 0, 0, 0))
+    rows_np = np.array(rows, dtype=_abi.CHUNK_DTYPE) if rows else np.zeros(0, dtype=_abi.CHUNK_DTYPE)
+    segs_np = np.array(segs, dtype=_abi.SEG_DTYPE) if segs else np.zeros(0, dtype=_abi.SEG_DTYPE)
+    info = _abi.check_tables(rows_np, segs_np, n_hypers, grad_dtype, lowp_dtype) if len(rows_np) else None
+    refresh_np, refresh_max = None, 0
+    if refresh:
+        refresh_np = np.array(refresh, dtype=_abi.CHUNK_DTYPE)
+        refresh_max = int(refresh_np['n_alloc'].max())
+    return LaunchPlan(rows_np, segs_np, refresh_np, refresh_max, block, info)

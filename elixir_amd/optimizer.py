@@ -300,19 +300,20 @@ class ElixirOptimizer:
                 tiles += (c.shard_size + tile - 1) // tile
             code = dtype_code(gpu_chunks[0].chunk_dtype)
             info = _abi.check_tables(rows, None, 0, code, code)
-            self._wb_table = (DeviceTable(rows, gpu_chunks[0].shard_device), info, code)
-        table, info, code = self._wb_table
+            self._wb_table = (DeviceTable(rows, gpu_chunks[0].shard_device), info, code,
+                              max(c.shard_size for c in gpu_chunks))
+        table, info, code, max_elems = self._wb_table
         stream = torch.cuda.current_stream(table.dev.device).cuda_stream
-        _abi.writeback_mt(table.ptr, len(table), info, code, self.blocks_per_cu, stream)
+        _abi.writeback_mt(table.ptr, len(table), code, max_elems, info.aligned, stream)
         for c in gpu_chunks:
             c.optim_sync_flag = True
 
-    def _refresh_chunk_stats(self) -> None:
-        """Flags for every parameter chunk whose gradients landed without them: one launch over
-        the chunk list and one device-to-host copy."""
+    def _launch_chunk_stats(self):
+        """Enqueues the flags pass for every parameter chunk whose gradients landed without them:
+        one launch over the chunk list.  Returns what ``_collect_chunk_stats`` needs."""
         pending = [c for c in self._param_chunk_list if not c._stats_fresh]
         if not pending:
-            return
+            return None
         device = pending[0].shard_device
         if device.type != 'cuda':
             raise RuntimeError('gradient flags are computed by the HIP kernels: shards must be on the GPU')
@@ -328,9 +329,19 @@ class ElixirOptimizer:
         with self._timed('stats'):
             records = launch_grad_stats(rows, dtype_code(pending[0].chunk_dtype), device, table=table,
                                         workspace=self._stats_workspace)
+        return pending, records
+
+    def _collect_chunk_stats(self, launched) -> None:
+        """One device-to-host copy of 16 bytes per chunk: the only wait of the step."""
+        if launched is None:
+            return
+        pending, records = launched
         stats = read_grad_stats(records)
         for c, rec in zip(pending, stats):
             c._apply_stats(bool(rec['overflow']), float(rec['sumsq']))
+
+    def _refresh_chunk_stats(self) -> None:
+        self._collect_chunk_stats(self._launch_chunk_stats())
 
     def _timed(self, key: str):
         return _EventPair(self.kernel_events, key)
@@ -378,17 +389,25 @@ class ElixirOptimizer:
         return self.grad_scaler.scale_value
 
     def zero_grad(self, *args, **kwargs):
+        if self._binding is not None:
+            return None    # bound fake parameters never carry a .grad: nothing to drop
         return self.optim.zero_grad(set_to_none=True)
 
     # ------------------------------------------------------------------ the step
 
     def step(self, *args, **kwargs):
-        self._refresh_chunk_stats()
+        launched = self._launch_chunk_stats()
+        if self._binding is not None and not args and not kwargs:
+            # host work of the update launch, done while the flags pass runs on the device
+            self.optim.prepare_step()
+        self._collect_chunk_stats(launched)
         self._set_grad_ptr()
         found_inf = self._check_overflow()
         self.last_step_info = dict(found_inf=found_inf, combined_scale=None, total_norm=None)
 
         if found_inf:
+            if self._binding is not None:
+                self.optim.discard_prepared()
             self.optim_state = OptimState.UNSCALED    # no need to unscale grad
             self.grad_scaler.update(found_inf)    # update gradient scaler
             self._clear_optim_states()    # clear chunk states used for optimizer update

@@ -46,7 +46,7 @@ enum {
     ELX_E_SIZE = -7      /* a count is zero, out of its allowed range, or exceeds what a launch can address */
 };
 
-/* flags of elx_adam_step_mt */
+/* flags of elx_adam_step_mt and elx_writeback_mt */
 enum {
     ELX_FLAG_SCALAR_ONLY = 1u    /* take the element-by-element path for every tile (set by the host when
                                     elx_check_tables reports base pointers that are not 16-byte aligned) */
@@ -136,17 +136,16 @@ uint32_t elx_sizeof_stats(void);
  * Host-side validation of HOST copies of the tables, to be called once before they are uploaded:
  * NULL / dtype / range / ordering / tile checks as listed under the ELX_E_* codes.  On success
  * writes
- *   *total_tiles              the launch-wide tile count (one workgroup per tile, < 2^31),
- *   *uniform_tiles_per_chunk  the tile count of every chunk when they all agree, else 0
- *                             (lets the kernels find a tile's chunk with one division),
- *   *all_aligned16            whether every non-NULL base pointer is 16-byte aligned (if not, pass
- *                             ELX_FLAG_SCALAR_ONLY to the launches).
+ *   *total_tiles          the tile count over all chunks (one workgroup per tile, < 2^31),
+ *   *max_tiles_per_chunk  the largest tile count of any chunk (the x extent of the 2-D grid),
+ *   *all_aligned16        whether every non-NULL base pointer is 16-byte aligned (if not, pass
+ *                         ELX_FLAG_SCALAR_ONLY to the launches).
  * lowp_dtype may be ELX_NONE when no chunk has a lowp_out buffer.
  * Replaces the per-tensor asserts and range bookkeeping of optimizer.py:238-265 at the boundary.
  */
 int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *h_segs, uint32_t n_segs,
                      uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles,
-                     uint32_t *uniform_tiles_per_chunk, int *all_aligned16);
+                     uint32_t *max_tiles_per_chunk, int *all_aligned16);
 
 /*
  * Stats pass over grad[0, n_valid) of every chunk: replaces Chunk.set_overflow_flag and
@@ -162,26 +161,40 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
  * Fused update over every chunk: for each element inside a segment
  *   g = (float)grad; if (div_scale > 0) g /= div_scale;            -- the div_scale of optimizer.py:216
  *   Adam / AdamW on master, m, v with the segment's ElxHyper;
- * and for every element of the shard (padding included), when lowp_out is set,
+ * and for every element of the chunk (padding included), when lowp_out is set,
  *   lowp_out = round-to-nearest-even(master)                       -- chunk.py:414
  * Replaces the inner optimizer's step over the fake parameters plus Chunk.optim_update.
- *   total_tiles, uniform_tiles_per_chunk   as returned by elx_check_tables for these tables
+ *
+ * A "chunk" of this table need not be a whole shard: callers get the best throughput by listing
+ * equal-sized blocks of the shards that contain tensors as separate records and leaving runs of
+ * pure padding to elx_writeback_mt (the update wants a shallow queue of small tiles, the refresh
+ * a deep queue of large ones).
+ *   total_tiles            as returned by elx_check_tables for these tables
+ *   grid_tiles_per_chunk   0: flat grid of total_tiles workgroups, each finds its chunk by a search
+ *                          over tile_begin;  otherwise the launch is a 2-D grid
+ *                          (grid_tiles_per_chunk, n_chunks) without any lookup, and must be at least
+ *                          the max_tiles_per_chunk that elx_check_tables reported (n_chunks <= 65535)
  *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (12).
  *                  The update streams best with a shallow, orderly queue of memory requests.
  */
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
                      const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,
-                     uint32_t uniform_tiles_per_chunk, float div_scale, int grad_dtype, int lowp_dtype,
+                     uint32_t grid_tiles_per_chunk, float div_scale, int grad_dtype, int lowp_dtype,
                      uint32_t flags, uint32_t blocks_per_cu, void *stream);
 
 /*
  * Low-precision refresh alone: lowp_out[0, n_alloc) = round-to-nearest-even(master) for every
- * chunk.  The skip-step branch (optimizer.py:196-203 -> chunk.py:403-414) and state loading
- * (elixir/wrapper/module.py:343) use it.
+ * record (only lowp_out, master and n_alloc are read).  The skip-step branch
+ * (optimizer.py:196-203 -> chunk.py:403-414), state loading (elixir/wrapper/module.py:343) and the
+ * padding runs left out of an update launch use it.
+ *   blocks_per_chunk  workgroups per record, 1..65535; each strides over pieces of
+ *                     elx_refresh_piece_elems() elements
  */
-int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, uint64_t total_tiles,
-                     uint32_t uniform_tiles_per_chunk, int lowp_dtype, uint32_t flags, uint32_t blocks_per_cu,
-                     void *stream);
+int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype, uint32_t blocks_per_chunk,
+                     uint32_t flags, void *stream);
+
+/* Elements one workgroup of the refresh launch handles per stride. */
+uint32_t elx_refresh_piece_elems(void);
 
 #ifdef __cplusplus
 }

@@ -97,7 +97,7 @@ def test_check_tables_accepts_and_rejects():
     bad = row.copy(); bad['n_alloc'] = 0; bad['n_valid'] = 0; expect(-7, chunk=bad, segs=None)
 
 
-def test_check_tables_reports_alignment_and_uniformity():
+def test_check_tables_reports_alignment_and_tile_counts():
     tile = _abi.tile_elems()
     per = 8192 // tile
     rows = np.concatenate([_row(8192, 0x10000000), _row(8192, 0x20000000), _row(5000, 0x30000000)])
@@ -105,12 +105,11 @@ def test_check_tables_reports_alignment_and_uniformity():
     rows['seg_end'] = 0
     rows['tile_begin'] = [0, per, 2 * per]
     info = _abi.check_tables(rows, None, 0, _abi.ELX_F16, _abi.ELX_NONE)
-    assert info.total_tiles == 2 * per + (5000 + tile - 1) // tile and info.uniform_tiles == 0 and info.aligned
-    info = _abi.check_tables(rows[:2], None, 0, _abi.ELX_F16, _abi.ELX_NONE)
-    assert info.total_tiles == 2 * per and info.uniform_tiles == per
+    assert info.total_tiles == 2 * per + (5000 + tile - 1) // tile and info.max_tiles == per and info.aligned
+    info = _abi.check_tables(rows[2:], None, 0, _abi.ELX_F16, _abi.ELX_NONE) if False else info
     rows[1]['grad'] += 2    # 2-byte aligned only: legal for fp16, but not vectorisable
     info = _abi.check_tables(rows[:2], None, 0, _abi.ELX_F16, _abi.ELX_NONE)
-    assert not info.aligned and info.flags == _abi.ELX_FLAG_SCALAR_ONLY
+    assert info.total_tiles == 2 * per and not info.aligned and info.flags == _abi.ELX_FLAG_SCALAR_ONLY
 
 
 def test_launch_entry_points_reject_bad_arguments_before_launching():
@@ -124,5 +123,7 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, 9, _abi.ELX_NONE, 0, 0, None) == -2
     assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 2, None) == -7
     assert lib.elx_adam_step_mt(1, 2, None, 0, None, 0, 5, 2, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -6
-    assert lib.elx_writeback_mt(None, 1, 4, 0, _abi.ELX_F16, 0, 0, None) == -1
-    assert lib.elx_writeback_mt(1, 1, 4, 0, _abi.ELX_NONE, 0, 0, None) == -2
+    assert lib.elx_writeback_mt(None, 1, _abi.ELX_F16, 4, 0, None) == -1
+    assert lib.elx_writeback_mt(1, 1, _abi.ELX_NONE, 4, 0, None) == -2
+    assert lib.elx_writeback_mt(1, 1, _abi.ELX_F16, 0, 0, None) == -7
+    assert lib.elx_refresh_piece_elems() == 4096

@@ -271,3 +271,70 @@ def test_bench_refuses_more_than_one_gpu():
     proc = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--gpus', '2'], stdout=subprocess.PIPE,
                           stderr=subprocess.PIPE, text=True)
     assert proc.returncode != 0 and 'ONE GPU' in proc.stderr
+
+
+# ------------------------------------------------------------------------------------------------
+# launch plan
+# ------------------------------------------------------------------------------------------------
+
+
+def test_launch_plan_blocks_segments_and_padding():
+    from elixir_amd.launch_plan import FlatBuffer, build_plan
+    tile = _abi.tile_elems()
+    base = 0x40000000
+    # a 64 Ki-element buffer with 40,000 valid elements in three tensors; the rest is padding
+    buf = FlatBuffer(grad=base, lowp_out=base, master=base + (1 << 24), m=base + (2 << 24), v=base + (3 << 24),
+                     n_alloc=65536, n_valid=40000, segs=[(0, 5000, 0), (5000, 5003, 1), (5003, 40000, 0)])
+    plan = build_plan([buf], 2, 2, 2, _abi.ELX_F16, _abi.ELX_F16)
+    B = plan.block_elems
+    assert B % tile == 0 and B >= 16 * tile
+    n_rows = -(-40000 // B)
+    assert len(plan.rows) == n_rows and plan.info.max_tiles == B // tile
+    covered = 0
+    for i, row in enumerate(plan.rows):
+        b = i * B
+        assert row['master'] == buf.master + 4 * b and row['grad'] == buf.grad + 2 * b == row['lowp_out']
+        assert row['m'] == buf.m + 4 * b and row['v'] == buf.v + 4 * b
+        assert row['n_alloc'] == min(B, 65536 - b) and row['n_valid'] == max(0, min(row['n_alloc'], 40000 - b))
+        segs = plan.segs[row['seg_begin']:row['seg_end']]
+        # the row's segments are the buffer's segments clipped to the block and re-based
+        want = [(max(sb, b) - b, min(se, b + B) - b, h) for sb, se, h in buf.segs if se > b and sb < b + B]
+        assert [(int(s['begin']), int(s['end']), int(s['hyper'])) for s in segs] == want
+        covered += sum(int(s['end'] - s['begin']) for s in segs)
+    assert covered == 40000
+    # padding beyond the last update block goes to the refresh launch
+    up_end = min(65536, n_rows * B)
+    if up_end < 65536:
+        assert len(plan.refresh_rows) == 1 and plan.refresh_rows[0]['n_alloc'] == 65536 - up_end
+        assert plan.refresh_rows[0]['lowp_out'] == base + 2 * up_end and plan.refresh_rows[0]['master'] == buf.master + 4 * up_end
+    else:
+        assert plan.refresh_rows is None
+    # no low-precision copy, no refresh rows; zero valid elements, no update rows
+    solo = FlatBuffer(grad=base, lowp_out=0, master=base + (1 << 24), m=base + (2 << 24), v=base + (3 << 24),
+                      n_alloc=65536, n_valid=40000, segs=[(0, 40000, 0)])
+    assert build_plan([solo], 4, 4, 1, _abi.ELX_F32, _abi.ELX_NONE).refresh_rows is None
+    empty = FlatBuffer(grad=base, lowp_out=base, master=base + (1 << 24), m=base + (2 << 24), v=base + (3 << 24),
+                       n_alloc=65536, n_valid=0, segs=[])
+    plan = build_plan([empty], 2, 2, 1, _abi.ELX_F16, _abi.ELX_F16)
+    assert len(plan.rows) == 0 and plan.refresh_rows[0]['n_alloc'] == 65536
+
+
+def test_launch_plan_keeps_rows_bounded_for_the_large_workloads():
+    from elixir_amd.launch_plan import FlatBuffer, build_plan
+    from elixir_amd.module import greedy_groups
+    sizes = [S.numel(s) for _, s in S.llama_shapes()]
+    bufs = []
+    for k, grp in enumerate(greedy_groups(sizes, 256 << 20)):
+        off, segs = 0, []
+        for i in grp:
+            segs.append((off, off + sizes[i], 0))
+            off += sizes[i]
+        base = (k + 1) << 34
+        bufs.append(FlatBuffer(base, base, base + (1 << 32), base + (2 << 32), base + (3 << 32), 256 << 20, off, segs))
+    plan = build_plan(bufs, 2, 2, 1, _abi.ELX_F16, _abi.ELX_F16)
+    assert len(plan.rows) < 65536 and plan.info.max_tiles == plan.block_elems // _abi.tile_elems()
+    assert int(plan.rows['n_valid'].sum()) == sum(sizes)
+    padding = 27 * (256 << 20) - int(plan.rows['n_alloc'].sum())
+    assert padding == int(plan.refresh_rows['n_alloc'].sum()) and padding > 0
+    # few workgroups of the 2-D grid find no work
+    assert plan.info.max_tiles * len(plan.rows) - plan.info.total_tiles < 0.01 * plan.info.total_tiles
