@@ -86,13 +86,8 @@ struct Elem<ELX_BF16> {
     static __device__ __forceinline__ float to_f32(uint16_t b) {
         return __builtin_bit_cast(float, (uint32_t)b << 16);
     }
-    // round to nearest even on the bit pattern; NaN stays a quiet NaN
-    static __device__ __forceinline__ uint16_t from_f32(float x) {
-        uint32_t u = __builtin_bit_cast(uint32_t, x);
-        if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
-        u += 0x7FFFu + ((u >> 16) & 1u);
-        return (uint16_t)(u >> 16);
-    }
+    // v_cvt_pk_bf16_f32: round to nearest even, NaN stays a quiet NaN
+    static __device__ __forceinline__ uint16_t from_f32(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }
 };
 
 template <typename V>
