@@ -25,11 +25,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
 BYTES_UPDATE = 28               # per valid element: read g(2)+p,m,v(12); write p,m,v(12)+lowp(2)
 BYTES_STATS = 2                 # per valid element: the compulsory second read of g
-# HBM bytes per update launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
-# scaled by what the same counters read for a plain copy of known size (--calibrate-copy):
-# 96.375e9 read + 95.356e9 written for c5, i.e. the algorithmic bytes plus the refresh of the
-# chunk padding.  Counter runs cannot ride along with a timed run, hence a recorded figure.
-MEASURED_TRAFFIC_BYTES = {'c5': 191.73e9}
+# HBM bytes per adam_step_kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script, scaled by what the same counters read for a plain copy of known size (--calibrate-copy):
+# 94.411e9 read + 94.364e9 written for c5, i.e. the algorithmic 188.676e9 plus the padding inside
+# the last block of each chunk.  (The padding refresh launch moves another 1.984e9 + 0.992e9.)
+# Counter runs cannot ride along with a timed run, hence a recorded figure.
+MEASURED_TRAFFIC_BYTES = {'c5': 188.775e9}
 
 
 def cpu_baseline(built, sample_elems: int, steps: int = 3):
@@ -125,10 +126,11 @@ def main():
     opt.blocks_per_cu = args.blocks_per_cu
     n_valid = built.n_valid
 
-    step_s, upd_ms, stats_ms = [], [], []
+    step_s, upd_ms, stats_ms, adam_ms, refresh_ms = [], [], [], [], []
     for i in range(args.warmup + args.steps):
         built.land_gradients()
         opt.kernel_events = {}
+        opt.optim.kernel_events = {}
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         opt.step()
@@ -140,10 +142,16 @@ def main():
             ev = opt.kernel_events
             upd_ms.append(ev['update'][0].elapsed_time(ev['update'][1]))
             stats_ms.append(ev['stats'][0].elapsed_time(ev['stats'][1]))
+            iev = opt.optim.kernel_events
+            adam_ms.append(iev['adam_step'][0].elapsed_time(iev['adam_step'][1]))
+            refresh_ms.append(iev['refresh'][0].elapsed_time(iev['refresh'][1]) if 'refresh' in iev else 0.0)
     opt.kernel_events = None
+    opt.optim.kernel_events = None
 
     t_step = float(np.mean(step_s))
-    t_upd = float(np.mean(upd_ms)) * 1e-3
+    t_pair = float(np.mean(upd_ms)) * 1e-3        # update launch + padding refresh launch + host time between
+    t_upd = float(np.mean(adam_ms)) * 1e-3         # adam_step_kernel alone
+    t_refresh = float(np.mean(refresh_ms)) * 1e-3
     t_stats = float(np.mean(stats_ms)) * 1e-3
     upd_gbps = BYTES_UPDATE * n_valid / t_upd / 1e9
     out = {
@@ -187,6 +195,12 @@ def main():
             'traffic': MEASURED_TRAFFIC_BYTES.get(built.spec.name),
             'bytes_per_launch': BYTES_UPDATE * n_valid,
             'ms_per_launch': t_upd * 1e3,
+        },
+        'refresh_kernel': {
+            'what': 'low-precision refresh of the chunk padding left out of the update launch',
+            'ms_per_launch': t_refresh * 1e3,
+            'update_plus_refresh_ms': t_pair * 1e3,
+            'achieved_28B_over_both': BYTES_UPDATE * n_valid / t_pair / 1e9,
         },
         'stats_kernel': {
             'kernel': 'grad_stats_kernel+stats_finish_kernel',

@@ -186,6 +186,8 @@ class HybridAdam(torch.optim.Optimizer):
         self._hyper_uploader = _HyperUploader()
         self._prepared: Optional[_Prepared] = None
         self._bound_entries = None                  # cached walk over the bound fake parameters
+        # when set to a dict, step() records (begin, end) torch.cuda.Event pairs under 'adam_step' and 'refresh'
+        self.kernel_events = None
 
     # ------------------------------------------------------------------ chunk binding
 
@@ -264,13 +266,22 @@ class HybridAdam(torch.optim.Optimizer):
             state['step'] += 1
         plan = prep.dplan.plan
         stream = torch.cuda.current_stream(prep.device).cuda_stream
+        events = self.kernel_events
         if prep.dplan.rows is not None:
+            if events is not None:
+                events['adam_step'] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                events['adam_step'][0].record()
             _abi.adam_step_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs), prep.d_hypers,
                               len(prep.hyper_host), plan.info, float(div_scale), prep.grad_code, prep.lowp_code,
                               self.blocks_per_cu, stream)
+            if events is not None:
+                events['adam_step'][1].record()
         if prep.dplan.refresh is not None:
             _abi.writeback_mt(prep.dplan.refresh.ptr, len(plan.refresh_rows), prep.lowp_code, plan.refresh_max_elems,
                               prep.dplan.refresh_aligned, stream)
+            if events is not None:
+                events['refresh'] = (events['adam_step'][1], torch.cuda.Event(enable_timing=True))
+                events['refresh'][1].record()
         if self._binding is not None and prep.lowp_code != _abi.ELX_NONE:
             self._binding.fused_writeback = True
         return loss
