@@ -30,7 +30,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg',
            'elx_sizeof_hyper', 'elx_sizeof_stats', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
-           'elx_writeback_mt', 'elx_refresh_piece_elems')
+           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_land_grads_mt', 'elx_land_max_blocks')
 
 
 class ElxError(RuntimeError):
@@ -60,7 +60,7 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
-                 'elx_refresh_piece_elems'):
+                 'elx_refresh_piece_elems', 'elx_land_max_blocks'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -72,6 +72,8 @@ def load() -> ctypes.CDLL:
     L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_writeback_mt.restype = cint
     L.elx_writeback_mt.argtypes = [vp, u32, cint, u32, u32, vp]
+    L.elx_land_grads_mt.restype = cint
+    L.elx_land_grads_mt.argtypes = [vp, u32, cint, cint, flt, u32, vp, vp, u32, vp]
 
     if L.elx_version() != ELX_ABI_VERSION:
         raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
@@ -163,3 +165,14 @@ def writeback_mt(d_chunks: int, n_chunks: int, lowp_dtype: int, max_elems: int, 
     blocks = max(1, min(4096, (max_elems + piece - 1) // piece))
     check('elx_writeback_mt',
           load().elx_writeback_mt(d_chunks, n_chunks, lowp_dtype, blocks, 0 if aligned else ELX_FLAG_SCALAR_ONLY, stream))
+
+
+def land_max_blocks() -> int:
+    return int(load().elx_land_max_blocks())
+
+
+def land_grads_mt(d_rows: int, n_rows: int, src_dtype: int, dst_dtype: int, mul: float, blocks_per_row: int,
+                  d_partials: int, d_stats: int, aligned: bool, stream: int) -> None:
+    check('elx_land_grads_mt',
+          load().elx_land_grads_mt(d_rows, n_rows, src_dtype, dst_dtype, mul, blocks_per_row, d_partials, d_stats,
+                                   0 if aligned else ELX_FLAG_SCALAR_ONLY, stream))

@@ -118,6 +118,118 @@ def l2_norm_from_sumsq(sumsq: float) -> float:
     return float(np.float32(math.sqrt(sumsq)))**2
 
 
+def land_launch_blocks(n_alloc_max: int) -> int:
+    """Workgroups per row of the landing launch: one per 16 Ki elements, at most 1024."""
+    return int(max(1, min(LAND_BLOCKS_PER_ROW, _abi.land_max_blocks(), math.ceil(n_alloc_max / 16384))))
+
+
+LAND_BLOCKS_PER_ROW = 1024
+
+
+class StatsArena:
+    """Device ElxStats records that landing launches leave behind, one slot per chunk, so that the
+    optimizer step can fetch the flags of all chunks with one device-to-host copy."""
+    CAPACITY = 8192
+    _arenas: Dict[torch.device, 'StatsArena'] = {}
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self.itemsize = _abi.STATS_DTYPE.itemsize
+        self.buf = torch.zeros(self.CAPACITY * self.itemsize, dtype=torch.uint8, device=device)
+        self.next = 0
+
+    @classmethod
+    def get(cls, device: torch.device) -> 'StatsArena':
+        device = torch.device(device)
+        arena = cls._arenas.get(device)
+        if arena is None:
+            arena = cls._arenas[device] = StatsArena(device)
+        return arena
+
+    def new_slots(self, count: int) -> int:
+        """First index of ``count`` consecutive fresh slots."""
+        if self.next + count > self.CAPACITY:
+            raise RuntimeError(f'more than {self.CAPACITY} stats slots in use on {self.device}')
+        first = self.next
+        self.next += count
+        return first
+
+    def ptr(self, slot: int) -> int:
+        return self.buf.data_ptr() + slot * self.itemsize
+
+    def read(self, lo: int, hi: int) -> np.ndarray:
+        """Slots [lo, hi) on the host: one blocking copy."""
+        return self.buf[lo * self.itemsize:hi * self.itemsize].cpu().numpy().view(_abi.STATS_DTYPE).copy()
+
+
+def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float = 1.0) -> None:
+    """Fused gradient landing for a list of chunks in ONE launch: ``payloads[i]`` (``shard_size``
+    elements: the slice of the reduced payload that belongs to the shard; the chunk's dtype, or fp32)
+    overwrites ``chunks[i].shard`` while the overflow flag and the sum of squares of what now sits in
+    ``shard[:valid_end]`` are left in the chunk's slot of the device arena.  Nothing is read back
+    here; ``Chunk.overflow`` / ``Chunk.l2_norm`` (or the optimizer step, for all chunks at once)
+    fetch the records when they are needed.  Replaces chunk.py:309-315 + 345-356."""
+    if not chunks:
+        return
+    device = chunks[0].shard_device
+    if device.type != 'cuda':
+        raise RuntimeError('gradients land through the HIP kernels: shards must be on the GPU')
+    dst_code = dtype_code(chunks[0].chunk_dtype)
+    src_code = dtype_code(payloads[0].dtype)
+    for c, pl in zip(chunks, payloads):
+        assert not c.is_init
+        assert c.shard_device == device and pl.device == device and pl.is_contiguous()
+        assert dtype_code(c.chunk_dtype) == dst_code and dtype_code(pl.dtype) == src_code
+        assert pl.numel() == c.shard_size, 'the payload slice must cover the shard'
+    arena = StatsArena.get(device)
+    slots = [c._stats_slot for c in chunks]
+    if slots[0] is None or any(b is None or b != a + 1 for a, b in zip(slots, slots[1:])):
+        first = arena.new_slots(len(chunks))
+        for i, c in enumerate(chunks):
+            c._stats_slot = first + i
+    rows = np.zeros(len(chunks), dtype=_abi.CHUNK_DTYPE)
+    for i, (c, pl) in enumerate(zip(chunks, payloads)):
+        rows[i]['grad'] = pl.data_ptr()
+        rows[i]['lowp_out'] = c.shard.data_ptr()
+        rows[i]['n_alloc'] = c.shard_size
+        rows[i]['n_valid'] = c.n_valid
+    aligned = bool(np.all(rows['grad'] % 16 == 0) and np.all(rows['lowp_out'] % 16 == 0))
+    bpr = land_launch_blocks(int(rows['n_alloc'].max()))
+    ws = chunks[0]._workspace
+    need = len(rows) * bpr * arena.itemsize
+    buf = ws.get('land')
+    if buf is None or buf.numel() < need:
+        buf = ws['land'] = torch.empty(need, dtype=torch.uint8, device=device)
+    cached = ws.get('land_table')
+    if cached is None or not np.array_equal(cached.host, rows):
+        cached = ws['land_table'] = DeviceTable(rows, device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    _abi.land_grads_mt(cached.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
+                       arena.ptr(chunks[0]._stats_slot), aligned, stream)
+    for c in chunks:
+        c._overflow = False
+        c._l2_norm = None
+        c._stats_fresh = False
+        c._stats_pending = True
+
+
+def resolve_pending_stats(chunks: List['Chunk']) -> None:
+    """Fetches the landing records of every chunk in the list that has one outstanding: one copy
+    per device."""
+    by_device: Dict[torch.device, List['Chunk']] = {}
+    for c in chunks:
+        if c._stats_pending:
+            by_device.setdefault(c.shard_device, []).append(c)
+    for device, pending in by_device.items():
+        lo = min(c._stats_slot for c in pending)
+        hi = max(c._stats_slot for c in pending) + 1
+        records = StatsArena.get(device).read(lo, hi)
+        for c in pending:
+            rec = records[c._stats_slot - lo]
+            c._stats_pending = False
+            c._apply_stats(bool(rec['overflow']), float(rec['sumsq']))
+
+
 class Chunk:
     """A continuous memory block that stores a sequence of tensors (chunk.py:27-139).
 
@@ -187,11 +299,14 @@ class Chunk:
         self.optim_sync_flag = True
         # whether to record l2 norm for the gradient clipping calculation
         self.l2_norm_flag = False
-        self.l2_norm: Optional[float] = None
-        # whether it overflows after the reduction
-        self.overflow = False
+        # squared l2 norm / overflow of the reduced gradients; both are properties that first fetch
+        # the record a fused landing left on the device, if one is outstanding
+        self._l2_norm: Optional[float] = None
+        self._overflow = False
         # True once overflow / l2_norm describe the gradients that sit in the shard now
         self._stats_fresh = False
+        self._stats_slot: Optional[int] = None    # this chunk's record in the device arena
+        self._stats_pending = False               # a landing launch has written it, nobody has read it
         self._workspace: Dict = {}
 
     # ------------------------------------------------------------------ properties
@@ -199,6 +314,33 @@ class Chunk:
     @property
     def is_init(self) -> bool:
         return self._is_init
+
+    @property
+    def overflow(self) -> bool:
+        if self._stats_pending:
+            resolve_pending_stats([self])
+        return self._overflow
+
+    @overflow.setter
+    def overflow(self, value: bool) -> None:
+        self._overflow = bool(value)
+
+    @property
+    def l2_norm(self) -> Optional[float]:
+        if self._stats_pending:
+            resolve_pending_stats([self])
+        return self._l2_norm
+
+    @l2_norm.setter
+    def l2_norm(self, value: Optional[float]) -> None:
+        self._l2_norm = value
+
+    def invalidate_stats(self) -> None:
+        """The shard was written behind the chunk's back: forget flags and outstanding records."""
+        self._stats_pending = False
+        self._stats_fresh = False
+        self._overflow = False
+        self._l2_norm = None
 
     @property
     def shard_device(self) -> torch.device:
@@ -300,11 +442,11 @@ class Chunk:
 
     def set_overflow_flag(self, valid_tensor: Optional[torch.Tensor] = None) -> None:
         """chunk.py:214-216; here both flags come from one pass over ``shard[:valid_end]``."""
-        assert not self.overflow
+        assert not self._stats_pending and not self._overflow
         self._compute_stats()
 
     def set_l2_norm(self, valid_tensor: Optional[torch.Tensor] = None) -> None:
-        assert self.l2_norm is None, 'you are calculating the l2 norm twice'
+        assert not self._stats_pending and self._l2_norm is None, 'you are calculating the l2 norm twice'
         self._compute_stats()
 
     def _compute_stats(self) -> None:
@@ -315,27 +457,37 @@ class Chunk:
         self._apply_stats(bool(stats['overflow'][0]), float(stats['sumsq'][0]))
 
     def _apply_stats(self, overflow: bool, sumsq: float) -> None:
-        self.overflow = overflow
+        self._overflow = overflow
         if self.l2_norm_flag:
-            self.l2_norm = l2_norm_from_sumsq(sumsq)
+            self._l2_norm = l2_norm_from_sumsq(sumsq)
         self._stats_fresh = True
 
     def update_extra_reduce_info(self, block=None):
         """chunk.py:345-356: flags over the valid head of the reduced gradients.  On one process
-        those are the first ``valid_end`` elements of the shard."""
-        assert not self.overflow
-        assert self.l2_norm is None, 'you are calculating the l2 norm twice'
+        those are the first ``valid_end`` elements of the shard.  After a fused landing the record
+        already exists on the device and is only fetched; otherwise one stats pass runs."""
+        if self._stats_pending:
+            resolve_pending_stats([self])
+            return
+        assert not self._overflow
+        assert self._l2_norm is None, 'you are calculating the l2 norm twice'
         self._compute_stats()
 
     def reduce_chunk(self, payload: torch.Tensor, always_fp32: bool = False, sync: bool = True) -> None:
         """The tail of chunk.py:282-315 / 358-377 for a process group of size 1: the gradients that
-        backward accumulated in ``payload`` (``chunk_size`` elements) overwrite the shard; with
-        ``sync`` the flags are computed right away, otherwise the optimizer computes them for all
-        chunks in one launch at the top of the step."""
+        backward accumulated in ``payload`` (``chunk_size`` elements of the chunk's dtype, or fp32
+        for a reduction carried out in fp32) overwrite the shard.  The copy and the flags are one
+        launch; with ``sync`` the flags are fetched right away (as the reference's blocking
+        ``.item()`` calls do), otherwise they stay on the device until somebody reads
+        ``overflow`` / ``l2_norm`` or the optimizer step collects them for all chunks at once."""
         assert not self.is_init
         assert payload.numel() == self.chunk_size
-        self.shard.copy_(payload[self.shard_begin:self.shard_end])
-        self._stats_fresh = False
+        if self.shard_device.type == 'cuda':
+            land_chunks([self], [payload[self.shard_begin:self.shard_end]])
+        else:
+            # a host-resident shard: the landing is a transfer, and no flags come with it
+            self.shard.copy_(payload[self.shard_begin:self.shard_end])
+            self.invalidate_stats()
         if sync:
             self.update_extra_reduce_info()
 

@@ -586,6 +586,99 @@ __global__ __launch_bounds__(kStatsThreads) void stats_finish_kernel(const ElxSt
 }
 
 // ---------------------------------------------------------------------------------------------
+// gradient landing: payload -> shard, with the stats riding the copy
+// ---------------------------------------------------------------------------------------------
+
+// dst[0, n_alloc) = cast(src * mul) for every row, and the stats of dst[0, n_valid) -- the values as
+// they sit in the shard afterwards, which is what the flags of the reference are taken from.  A row
+// uses `grad` as the source, `lowp_out` as the destination.  With MUL the product is first rounded
+// to the source type (an in-place scaling of the payload), then cast.  Without MUL and with equal
+// types the bits are moved untouched.  Grid (blocks_per_row, n_rows); a workgroup strides over
+// tiles of 256 lanes x one 128-bit load x kLandUnroll.
+constexpr int kLandThreads = 256;
+constexpr int kLandUnroll = 2;
+constexpr uint32_t kMaxLandBlocks = 8192;
+
+template <int SD, int DD, bool MUL>
+__device__ __forceinline__ typename Elem<DD>::scalar land_elem(typename Elem<SD>::scalar x, float mul, float &as_f32) {
+    if constexpr (SD == DD && !MUL) {
+        as_f32 = Elem<SD>::to_f32(x);
+        return x;
+    } else {
+        float v = Elem<SD>::to_f32(x);
+        if constexpr (MUL) v = Elem<SD>::to_f32(Elem<SD>::from_f32(v * mul));
+        const typename Elem<DD>::scalar d = Elem<DD>::from_f32(v);
+        as_f32 = Elem<DD>::to_f32(d);
+        return d;
+    }
+}
+
+template <int SD, int DD, bool MUL>
+__global__ __launch_bounds__(kLandThreads) void land_grads_kernel(const ElxChunk *__restrict__ rows, uint32_t bpr,
+                                                                  float mul, ElxStats *__restrict__ partials,
+                                                                  uint32_t scalar_only) {
+    typedef typename Elem<SD>::scalar sscalar;
+    typedef typename Elem<DD>::scalar dscalar;
+    constexpr uint32_t kEpl = 16 / sizeof(sscalar);
+    constexpr uint32_t kLSpan = kLandThreads * kEpl;
+    constexpr uint32_t kLTile = kLSpan * kLandUnroll;
+    typedef sscalar svec __attribute__((ext_vector_type(kEpl)));
+    typedef dscalar dvec __attribute__((ext_vector_type(kEpl)));
+
+    const ElxChunk c = rows[blockIdx.y];
+    const sscalar *src = reinterpret_cast<const sscalar *>(c.grad);
+    dscalar *dst = reinterpret_cast<dscalar *>(c.lowp_out);
+    const uint64_t n = (src && dst) ? c.n_alloc : 0;
+    const uint64_t nv = c.n_valid < n ? c.n_valid : n;
+    const uint64_t n_tiles = (n + kLTile - 1) / kLTile;
+
+    double sum = 0.0;
+    float poison = 0.0f;
+    for (uint64_t t = blockIdx.x; t < n_tiles; t += bpr) {
+        const uint64_t base = t * kLTile;
+        float acc = 0.0f;
+        if (base + kLTile <= n && !scalar_only && (base + kLTile <= nv || base >= nv)) {
+            const bool counted = base < nv;    // wave-uniform
+            const svec *sp = reinterpret_cast<const svec *>(src + base) + threadIdx.x;
+            dvec *dp = reinterpret_cast<dvec *>(dst + base) + threadIdx.x;
+            svec S[kLandUnroll];
+#pragma unroll
+            for (int u = 0; u < kLandUnroll; ++u) S[u] = ld_stream(sp + u * kLandThreads);
+#pragma unroll
+            for (int u = 0; u < kLandUnroll; ++u) {
+                dvec D;
+                float F[kEpl];
+#pragma unroll
+                for (uint32_t k = 0; k < kEpl; ++k) D[k] = land_elem<SD, DD, MUL>(S[u][k], mul, F[k]);
+                __builtin_nontemporal_store(D, dp + u * kLandThreads);
+                if (counted) {
+#pragma unroll
+                    for (uint32_t k = 0; k < kEpl; ++k) stats_elem(F[k], acc, poison);
+                }
+            }
+        } else {
+            const uint64_t left = n - base;
+            const uint32_t tile_n = left < kLTile ? (uint32_t)left : kLTile;
+            for (uint32_t i = threadIdx.x; i < tile_n; i += kLandThreads) {
+                float f;
+                dst[base + i] = land_elem<SD, DD, MUL>(src[base + i], mul, f);
+                if (base + i < nv) stats_elem(f, acc, poison);
+            }
+        }
+        sum += (double)acc;
+    }
+    uint32_t flag = (poison != poison) ? 1u : 0u;
+    block_fold(sum, flag);
+    if (threadIdx.x == 0) {
+        ElxStats r;
+        r.sumsq = sum;
+        r.overflow = flag;
+        r.reserved = 0;
+        partials[(uint64_t)blockIdx.y * bpr + blockIdx.x] = r;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side of the ABI
 // ---------------------------------------------------------------------------------------------
 
@@ -776,5 +869,36 @@ int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype
 }
 
 uint32_t elx_refresh_piece_elems(void) { return kRefreshPiece; }
+
+int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, int dst_dtype, float mul,
+                      uint32_t blocks_per_row, ElxStats *d_partials, ElxStats *d_stats, uint32_t flags, void *stream) {
+    if (!d_rows || !d_partials || !d_stats) return ELX_E_NULL;
+    if (!is_lowp_or_f32(src_dtype) || !is_lowp_or_f32(dst_dtype)) return ELX_E_DTYPE;
+    if (src_dtype != dst_dtype && src_dtype != ELX_F32) return ELX_E_DTYPE;
+    if (n_rows == 0 || n_rows > 65535u || blocks_per_row == 0 || blocks_per_row > kMaxLandBlocks) return ELX_E_SIZE;
+    if (!(mul == mul) || mul <= 0.0f) return ELX_E_RANGE;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const dim3 grid(blocks_per_row, n_rows), block(kLandThreads);
+    const uint32_t so = (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u;
+#define ELX_LAND(S, D)                                                                                          \
+    if (src_dtype == S && dst_dtype == D) {                                                                     \
+        if (mul == 1.0f)                                                                                        \
+            hipLaunchKernelGGL((land_grads_kernel<S, D, false>), grid, block, 0, st, d_rows, blocks_per_row, mul, d_partials, so); \
+        else                                                                                                    \
+            hipLaunchKernelGGL((land_grads_kernel<S, D, true>), grid, block, 0, st, d_rows, blocks_per_row, mul, d_partials, so);  \
+    }
+    ELX_LAND(ELX_F32, ELX_F32)
+    ELX_LAND(ELX_F16, ELX_F16)
+    ELX_LAND(ELX_BF16, ELX_BF16)
+    ELX_LAND(ELX_F32, ELX_F16)
+    ELX_LAND(ELX_F32, ELX_BF16)
+#undef ELX_LAND
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_rows), dim3(kStatsThreads), 0, st, d_partials, blocks_per_row, d_stats);
+    return (int)hipGetLastError();
+}
+
+uint32_t elx_land_max_blocks(void) { return kMaxLandBlocks; }
 
 }    // extern "C"

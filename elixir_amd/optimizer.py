@@ -29,7 +29,7 @@ import torch
 from torch.nn import Parameter
 
 from . import _abi
-from .chunk import Chunk, DeviceTable, dtype_code, launch_grad_stats, read_grad_stats
+from .chunk import Chunk, DeviceTable, dtype_code, launch_grad_stats, read_grad_stats, resolve_pending_stats
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
 from .hybrid_adam import HybridAdam
 
@@ -311,7 +311,7 @@ class ElixirOptimizer:
     def _launch_chunk_stats(self):
         """Enqueues the flags pass for every parameter chunk whose gradients landed without them:
         one launch over the chunk list.  Returns what ``_collect_chunk_stats`` needs."""
-        pending = [c for c in self._param_chunk_list if not c._stats_fresh]
+        pending = [c for c in self._param_chunk_list if not c._stats_fresh and not c._stats_pending]
         if not pending:
             return None
         device = pending[0].shard_device
@@ -333,6 +333,7 @@ class ElixirOptimizer:
 
     def _collect_chunk_stats(self, launched) -> None:
         """One device-to-host copy of 16 bytes per chunk: the only wait of the step."""
+        resolve_pending_stats(self._param_chunk_list)    # records left behind by fused landings
         if launched is None:
             return
         pending, records = launched
@@ -355,9 +356,7 @@ class ElixirOptimizer:
 
     def _clear_optim_states(self) -> None:
         for param_chunk in self.param_chunk_set:
-            param_chunk.overflow = False
-            param_chunk.l2_norm = None
-            param_chunk._stats_fresh = False
+            param_chunk.invalidate_stats()
 
     def _calc_global_norm(self) -> float:
         """optimizer.py:149-164 on one process: the per-group sum passes through a one-element fp32
@@ -403,7 +402,8 @@ class ElixirOptimizer:
         self._collect_chunk_stats(launched)
         self._set_grad_ptr()
         found_inf = self._check_overflow()
-        self.last_step_info = dict(found_inf=found_inf, combined_scale=None, total_norm=None)
+        self.last_step_info = dict(found_inf=found_inf, combined_scale=None, total_norm=None,
+                                   chunk_overflow=[bool(c.overflow) for c in self._param_chunk_list])
 
         if found_inf:
             if self._binding is not None:

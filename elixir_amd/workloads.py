@@ -11,6 +11,7 @@ import numpy as np
 import torch
 
 from . import shapes as S
+from .chunk import land_chunks
 from .hybrid_adam import HybridAdam
 from .module import ElixirModule, greedy_search
 from .optimizer import ElixirOptimizer
@@ -57,17 +58,22 @@ class BuiltWorkload:
     n_valid: int = 0
     n_alloc: int = 0
 
-    def land_gradients(self) -> None:
+    def land_gradients(self, fused: bool = False) -> None:
         """Puts the saved gradients back into the low-precision shards (what backward and the
-        chunk reduction leave behind) and declares them scaled."""
-        for pc, g in zip(self.module.param_chunks, self.grads):
-            pc.shard.copy_(g)
-            pc._stats_fresh = False
+        chunk reduction leave behind) and declares them scaled.  ``fused``: through the landing
+        launch that also leaves the flags of every chunk on the device, so that the step needs no
+        pass of its own over the gradients; otherwise a plain copy, flags unknown."""
+        if fused:
+            land_chunks(self.module.param_chunks, self.grads)
+        else:
+            for pc, g in zip(self.module.param_chunks, self.grads):
+                pc.shard.copy_(g)
+                pc.invalidate_stats()
         self.optimizer.mark_gradients_scaled()
 
 
 def build(name: str, device: Optional[torch.device] = None, seed: int = 1234, shapes: Optional[List[S.NamedShape]] = None,
-          chunk_size: Optional[int] = None) -> BuiltWorkload:
+          chunk_size: Optional[int] = None, hysteresis: Optional[int] = None) -> BuiltWorkload:
     spec = WORKLOADS[name]
     device = device or torch.device('cuda', torch.cuda.current_device())
     named = list(shapes if shapes is not None else spec.shapes())
@@ -83,8 +89,8 @@ def build(name: str, device: Optional[torch.device] = None, seed: int = 1234, sh
         groups.append(dict(params=exempt, weight_decay=0.0))
     inner = HybridAdam(groups, lr=spec.lr, betas=spec.betas, eps=spec.eps, weight_decay=spec.weight_decay,
                        adamw_mode=spec.adamw_mode)
-    opt = ElixirOptimizer(module, inner, initial_scale=spec.loss_scale, hysteresis=spec.hysteresis,
-                          max_norm=spec.max_norm)
+    opt = ElixirOptimizer(module, inner, initial_scale=spec.loss_scale,
+                          hysteresis=spec.hysteresis if hysteresis is None else hysteresis, max_norm=spec.max_norm)
     if module.use_amp:
         assert opt.loss_scale == spec.loss_scale
 

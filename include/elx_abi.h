@@ -196,6 +196,28 @@ int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype
 /* Elements one workgroup of the refresh launch handles per stride. */
 uint32_t elx_refresh_piece_elems(void);
 
+/*
+ * Gradient landing with the stats riding the copy: for every row
+ *   lowp_out[i] = cast_dst(grad[i])                          for i in [0, n_alloc)
+ * and d_stats[row] = overflow flag and sum of squares of lowp_out[0, n_valid) as stored.  Replaces the
+ * tail of Chunk.reduce, `__update_shard(reduce_buffer, self.shard)` (elixir/chunk/core/chunk.py:309-315,
+ * 484-489), fused with Chunk.update_extra_reduce_info (chunk.py:345-356): the flags are known when
+ * the gradients have landed, and the optimizer step needs no pass of its own over them.
+ * A row reads `grad` (the payload slice that belongs to this shard, n_alloc elements of src_dtype),
+ * `lowp_out` (the shard, n_alloc elements of dst_dtype), n_alloc and n_valid; nothing else.
+ *   src_dtype / dst_dtype  equal, or fp32 -> fp16 / bf16 (a payload reduced in fp32, chunk.py:291-296)
+ *   mul        1.0f: plain copy / cast.  Otherwise each element is multiplied in fp32, rounded to
+ *              src_dtype and then cast, as the in-place `reduce_buffer /= pg_size` of chunk.py:299
+ *              does on the device for mul = 1.0f / pg_size.  Must be finite and > 0.
+ *   blocks_per_row  workgroups per row, 1..elx_land_max_blocks()
+ *   d_partials workspace of n_rows * blocks_per_row ElxStats records (contents ignored)
+ *   d_stats    n_rows results; fixed reduction order
+ */
+int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, int dst_dtype, float mul,
+                      uint32_t blocks_per_row, ElxStats *d_partials, ElxStats *d_stats, uint32_t flags, void *stream);
+
+uint32_t elx_land_max_blocks(void);
+
 #ifdef __cplusplus
 }
 #endif

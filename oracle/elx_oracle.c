@@ -14,6 +14,8 @@
  *   orc_sumsq           float64 brute force used to check the norm
  *   orc_l2norm_sq_ref   elixir/chunk/core/chunk.py:218-221   (float().norm(2).item()**2)
  *   orc_writeback       elixir/chunk/core/chunk.py:403-414   (shard.copy_(fp32 shard): RNE cast)
+ *   orc_land            elixir/chunk/core/chunk.py:299,309-315,484-489  (reduce_buffer /= pg_size on
+ *                       the device, then shard.copy_(reduce_buffer[shard_begin:shard_end]))
  *   orc_adam            elixir/wrapper/optimizer.py:211-216 -> inner optimizer step with
  *                       div_scale.  The inner optimizer (ColossalAI HybridAdam) is not part
  *                       of the reference tree; its published update rule is
@@ -172,6 +174,38 @@ void orc_writeback(const float *master, void *lowp, int dtype, uint64_t n) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < (int64_t)n; ++i)
         out[i] = orc_f32_to_lowp(master[i], dtype);
+}
+
+/* ---------- gradient landing (chunk.py:299, 309-315, 484-489) ---------- */
+
+/*
+ * dst[i] = cast_dd(src[i]) for i in [0, n).  With mul != 1 the element is first scaled the way an
+ * in-place `payload /= pg_size` scales it on the device: the tensor is multiplied by the fp32
+ * reciprocal of the host scalar (mul = 1.0f / pg_size) in fp32 and rounded back to the payload's
+ * own type; the cast to the shard's type follows.  Equal types and mul == 1: the bits move
+ * untouched (a copy does not canonicalise NaN payloads).  Allowed pairs: sd == dd, or sd == fp32.
+ */
+void orc_land(const void *src, int sd, void *dst, int dd, uint64_t n, float mul) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)n; ++i) {
+        if (sd == dd && mul == 1.0f) {
+            if (sd == 0)
+                ((uint32_t *)dst)[i] = ((const uint32_t *)src)[i];
+            else
+                ((uint16_t *)dst)[i] = ((const uint16_t *)src)[i];
+            continue;
+        }
+        float v = load_grad(src, sd, (uint64_t)i);
+        if (mul != 1.0f) {
+            v = v * mul;
+            if (sd != 0)
+                v = orc_lowp_to_f32(orc_f32_to_lowp(v, sd), sd);
+        }
+        if (dd == 0)
+            ((float *)dst)[i] = v;
+        else
+            ((uint16_t *)dst)[i] = orc_f32_to_lowp(v, dd);
+    }
 }
 
 /* ---------- stages 1+4: unscale and Adam / AdamW ---------- */

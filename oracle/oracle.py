@@ -64,6 +64,8 @@ def lib():
         L.orc_l2norm_sq_ref.argtypes = [vp, cint, u64]
         L.orc_writeback.restype = None
         L.orc_writeback.argtypes = [vp, vp, cint, u64]
+        L.orc_land.restype = None
+        L.orc_land.argtypes = [vp, cint, vp, cint, u64, flt]
         L.orc_adam.restype = None
         L.orc_adam.argtypes = [vp, cint, vp, vp, vp, u64, dbl, dbl, dbl, dbl, dbl, i64, cint, cint, flt]
         L.orc_adam_f64.restype = None
@@ -121,6 +123,17 @@ def writeback(master: np.ndarray, dtype: int) -> np.ndarray:
     assert master.dtype == np.float32
     out = np.empty(master.shape, dtype=np.float32 if dtype == F32 else np.uint16)
     lib().orc_writeback(_ptr(master), _ptr(out), dtype, master.size)
+    return out
+
+
+def land(src: np.ndarray, src_dtype: int, dst_dtype: int, mul: float = 1.0) -> np.ndarray:
+    """chunk.py:299,309-315,484-489 -- the payload as it sits in the shard after landing: scaled by
+    ``mul`` in the payload's own type (``mul = float32(1/pg_size)``; 1.0 on one GPU), then cast to
+    the shard's type."""
+    _check_grad(src, src_dtype)
+    assert src_dtype == dst_dtype or src_dtype == F32
+    out = np.empty(src.shape, dtype=np.float32 if dst_dtype == F32 else np.uint16)
+    lib().orc_land(_ptr(src), src_dtype, _ptr(out), dst_dtype, src.size, float(np.float32(mul)))
     return out
 
 

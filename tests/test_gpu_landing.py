@@ -1,0 +1,304 @@
+"""Gradient landing fused with the flags (elixir/chunk/core/chunk.py:299,309-315,345-356,484-489):
+the payload overwrites the shard, and the overflow flag and squared norm of what now sits in
+``shard[:valid_end]`` come out of the same pass.
+
+Bars: the landed shard is bit-identical to the oracle's (and to torch's own device ops where torch
+has the op); the overflow flag is exact; the sum of squares is within 1e-6 relative of the float64
+brute force (the summation order differs).
+"""
+import numpy as np
+import pytest
+import torch
+
+import elixir_amd as ea
+from elixir_amd import _abi, workloads
+from elixir_amd.chunk import DeviceTable, StatsArena, land_chunks
+from oracle import oracle as O
+
+from helpers import CODE, build_workload, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+PAIRS = [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32),
+         (torch.float32, torch.float16), (torch.float32, torch.bfloat16)]
+
+
+def _land(src: torch.Tensor, dst: torch.Tensor, n_valid: int, mul: float = 1.0, blocks: int = 0):
+    """One row through the C ABI; returns (overflow, sumsq)."""
+    n = dst.numel()
+    assert src.numel() == n
+    row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+    row['grad'], row['lowp_out'], row['n_alloc'], row['n_valid'] = src.data_ptr(), dst.data_ptr(), n, n_valid
+    table = DeviceTable(row, dst.device)
+    bpr = blocks or max(1, min(1024, -(-n // 16384)))
+    ws = torch.empty((bpr + 1) * _abi.STATS_DTYPE.itemsize, dtype=torch.uint8, device=dst.device)
+    aligned = src.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0
+    _abi.land_grads_mt(table.ptr, 1, CODE[src.dtype], CODE[dst.dtype], mul, bpr, ws.data_ptr(),
+                       ws.data_ptr() + bpr * _abi.STATS_DTYPE.itemsize, aligned,
+                       torch.cuda.current_stream().cuda_stream)
+    rec = ws[bpr * _abi.STATS_DTYPE.itemsize:].cpu().numpy().view(_abi.STATS_DTYPE)
+    return bool(rec['overflow'][0]), float(rec['sumsq'][0])
+
+
+def _payload(n, dtype, seed, scale=3.0):
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    return (torch.randn(n, generator=g, device=DEV) * scale).to(dtype)
+
+
+@pytest.mark.parametrize('sd,dd', PAIRS)
+@pytest.mark.parametrize('n', [1, 7, 4095, 4096, 8192 * 4 + 5, (1 << 20) + 3, (1 << 22) + 12345])
+def test_landing_matches_oracle(oracle, sd, dd, n):
+    src = _payload(n, sd, n)
+    nv = max(1, n - n // 5)                       # a padded tail
+    if nv < n:
+        src[nv:] = float('inf')                   # garbage in the padding: copied, never counted
+    dst = torch.full((n,), 7.0, dtype=dd, device=DEV)
+    flag, sumsq = _land(src, dst, nv)
+    want = oracle.land(to_np(src), CODE[sd], CODE[dd])
+    got = to_np(dst)
+    assert np.array_equal(got.view(np.uint32 if dd == torch.float32 else np.uint16),
+                          want.view(np.uint32 if dd == torch.float32 else np.uint16))
+    assert flag is False and oracle.overflow(want[:nv], CODE[dd]) is False
+    ref = oracle.sumsq(want[:nv], CODE[dd])
+    assert abs(sumsq - ref) <= 1e-6 * ref, (sumsq, ref)
+    # and what torch's own copy leaves in the shard
+    assert torch.equal(dst[:nv], src[:nv].to(dd))
+
+
+@pytest.mark.parametrize('sd,dd', PAIRS)
+@pytest.mark.parametrize('bad', [float('inf'), float('-inf'), float('nan')])
+def test_landing_flags_nonfinite(oracle, sd, dd, bad):
+    n = 100_000
+    for pos in (0, n // 2 + 1, n - 1):
+        src = _payload(n, sd, pos)
+        src[pos] = bad
+        dst = torch.zeros(n, dtype=dd, device=DEV)
+        flag, _ = _land(src, dst, n)
+        assert flag is True, (pos, bad)
+        # just outside the valid head it does not count
+        flag, _ = _land(src, dst, pos)
+        assert flag is False, (pos, bad)
+
+
+def test_landing_overflow_born_in_the_cast():
+    """An fp32 payload that is finite but too large for fp16: the shard holds inf after landing, and
+    the flag is taken from the shard (chunk.py:345-356), so it must be set.  bf16 keeps it finite."""
+    n = 50_000
+    src = _payload(n, torch.float32, 3)
+    src[12345] = 70000.0
+    dst = torch.zeros(n, dtype=torch.float16, device=DEV)
+    flag, _ = _land(src, dst, n)
+    assert flag is True and torch.isinf(dst[12345])
+    dst = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    flag, sumsq = _land(src, dst, n)
+    assert flag is False
+    assert abs(sumsq - float(dst.double().square().sum())) <= 1e-6 * sumsq
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_landing_same_type_keeps_every_bit_pattern(dtype):
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    src = bits.view(dtype).repeat(3).to(DEV)          # signalling NaNs, both zeros, subnormals
+    dst = torch.zeros_like(src)
+    flag, _ = _land(src, dst, src.numel())
+    assert flag is True
+    assert torch.equal(dst.view(torch.int16), src.view(torch.int16))
+
+
+@pytest.mark.parametrize('sd,dd', PAIRS)
+@pytest.mark.parametrize('pg', [2, 3, 6, 8])
+def test_landing_scaled_like_torchs_device_division(oracle, sd, dd, pg):
+    """``reduce_buffer /= pg_size`` (chunk.py:299) as torch runs it on the device, then the copy into
+    the shard: the same bits, powers of two or not."""
+    n = (1 << 18) + 77
+    src = _payload(n, sd, pg, scale=50.0)
+    src[:6] = torch.tensor([0.0, -0.0, 65504.0, -6e-8, 1e-3, 3.0], device=DEV).to(sd)
+    want = src.clone()
+    want /= pg
+    want = want.to(dd)
+    dst = torch.zeros(n, dtype=dd, device=DEV)
+    flag, sumsq = _land(src, dst, n, mul=float(np.float32(1.0) / np.float32(pg)))
+    view = torch.int32 if dd == torch.float32 else torch.int16
+    assert torch.equal(dst.view(view), want.view(view))
+    assert flag is False
+    ref = float(want.double().square().sum())
+    assert abs(sumsq - ref) <= 1e-6 * ref
+    got = to_np(dst)
+    ora = oracle.land(to_np(src), CODE[sd], CODE[dd], mul=float(np.float32(1.0) / np.float32(pg)))
+    assert np.array_equal(got.view(np.uint8), ora.view(np.uint8))
+
+
+@pytest.mark.parametrize('sd,dd', [(torch.float16, torch.float16), (torch.float32, torch.bfloat16)])
+def test_landing_unaligned_bases(oracle, sd, dd):
+    n = 70_001
+    src_full = _payload(n + 3, sd, 1)
+    dst_full = torch.zeros(n + 1, dtype=dd, device=DEV)
+    src, dst = src_full[3:], dst_full[1:]
+    flag, sumsq = _land(src, dst, n - 5)
+    want = oracle.land(to_np(src), CODE[sd], CODE[dd])
+    assert np.array_equal(to_np(dst).view(np.uint8), want.view(np.uint8))
+    ref = oracle.sumsq(want[:n - 5], CODE[dd])
+    assert flag is False and abs(sumsq - ref) <= 1e-6 * ref
+    assert float(dst_full[0]) == 0.0
+
+
+def test_landing_is_reproducible_and_independent_of_the_grid(oracle):
+    n = (1 << 21) + 999
+    src = _payload(n, torch.float16, 8)
+    dst = torch.zeros_like(src)
+    first = _land(src, dst, n)
+    assert _land(src, dst, n) == first
+    ref = oracle.sumsq(to_np(src), O.F16)
+    for blocks in (1, 3, 64, 4096):
+        flag, sumsq = _land(src, dst, n, blocks=blocks)
+        assert flag is False and abs(sumsq - ref) <= 1e-6 * ref
+        assert torch.equal(dst, src)
+
+
+def test_abi_rejects_bad_landing_arguments():
+    src = torch.zeros(16, dtype=torch.float16, device=DEV)
+    dst = torch.zeros(16, dtype=torch.float32, device=DEV)
+    with pytest.raises(_abi.ElxError):
+        _land(src, dst, 16)                              # low precision -> fp32 is not a landing
+    dst = torch.zeros(16, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(_abi.ElxError):
+        _land(src, dst, 16)                              # fp16 -> bf16
+    dst = torch.zeros(16, dtype=torch.float16, device=DEV)
+    for mul in (0.0, -1.0, float('nan')):
+        with pytest.raises(_abi.ElxError):
+            _land(src, dst, 16, mul=mul)
+    with pytest.raises(_abi.ElxError):
+        _land(src, dst, 16, blocks=_abi.land_max_blocks() + 1)
+
+
+# ------------------------------------------------------------------------------------------------
+# through Chunk / ElixirOptimizer
+# ------------------------------------------------------------------------------------------------
+
+
+def _tiny():
+    return [('a.weight', (300, 41)), ('a.bias', (41,)), ('b.weight', (129, 77)), ('n.weight', (77,)),
+            ('c.weight', (311, 33)), ('c.bias', (33,))]
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('sync', [True, False])
+def test_reduce_chunk_lands_and_flags(oracle, dtype, sync):
+    module, opt, _ = build_workload(_tiny(), 16384, dtype, seed=2, loss_scale=64.0, initial_scale=64.0, max_norm=1.0)
+    chunks = module.param_chunks
+    assert len(chunks) >= 2
+    payloads = [_payload(pc.chunk_size, dtype, 10 + i, scale=0.5) for i, pc in enumerate(chunks)]
+    for pl, pc in zip(payloads, chunks):
+        pl[pc.utilized_size:] = 0
+    payloads[1][5] = float('inf')
+    for pc, pl in zip(chunks, payloads):
+        pc.invalidate_stats()
+        pc.reduce_chunk(pl, sync=sync)
+        assert pc._stats_pending is (not sync)
+    for i, (pc, pl) in enumerate(zip(chunks, payloads)):
+        assert torch.equal(pc.shard.view(torch.int16), pl.view(torch.int16))
+        assert pc.overflow is (i == 1)
+        assert pc._stats_pending is False
+        want = oracle.l2norm_sq_ref(to_np(pl)[:pc.n_valid], CODE[dtype])
+        if i != 1:
+            assert abs(pc.l2_norm - want) <= 1e-6 * want
+        # reading again does not touch the device record
+        assert pc.overflow is (i == 1)
+
+
+def test_fused_landing_then_step_equals_plain_landing_then_step(oracle):
+    """The step after a fused landing launches no stats pass and gives the same bits."""
+    dtype = torch.float16
+    runs = []
+    for fused in (False, True):
+        module, opt, _ = build_workload(_tiny(), 16384, dtype, seed=5, loss_scale=128.0, initial_scale=128.0)
+        payloads = [_payload(pc.chunk_size, dtype, 20 + i, scale=0.1) for i, pc in enumerate(module.param_chunks)]
+        for pl, pc in zip(payloads, module.param_chunks):
+            pl[pc.utilized_size:] = 0
+        if fused:
+            land_chunks(module.param_chunks, payloads)
+            assert all(pc._stats_pending for pc in module.param_chunks)
+        else:
+            for pc, pl in zip(module.param_chunks, payloads):
+                pc.shard.copy_(pl)
+                pc.invalidate_stats()
+        opt.mark_gradients_scaled()
+        opt.kernel_events = {}
+        opt.step()
+        assert ('stats' in opt.kernel_events) is (not fused)
+        assert opt.last_step_info['found_inf'] is False and opt.last_step_info['combined_scale'] == 128.0
+        runs.append([(pc.paired_chunk.shard.clone(), pc.shard.clone(), *[t.clone() for t in
+                                                                        opt._binding.moments(pc.paired_chunk)])
+                     for pc in module.param_chunks])
+    for a, b in zip(*runs):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+
+
+def test_fused_landing_overflow_skips_the_step(oracle):
+    dtype = torch.float16
+    module, opt, _ = build_workload(_tiny(), 16384, dtype, seed=6, loss_scale=64.0, initial_scale=64.0, hysteresis=1)
+    payloads = [_payload(pc.chunk_size, dtype, 30 + i, scale=0.1) for i, pc in enumerate(module.param_chunks)]
+    for pl, pc in zip(payloads, module.param_chunks):
+        pl[pc.utilized_size:] = 0
+    last = module.param_chunks[-1]
+    payloads[-1][last.n_valid - 1] = float('nan')
+    before = [pc.paired_chunk.shard.clone() for pc in module.param_chunks]
+    land_chunks(module.param_chunks, payloads)
+    opt.mark_gradients_scaled()
+    opt.step()
+    assert opt.last_step_info['found_inf'] is True and opt.loss_scale == 32.0
+    assert opt.last_step_info['chunk_overflow'] == [False] * (len(payloads) - 1) + [True]
+    for pc, p0 in zip(module.param_chunks, before):
+        assert torch.equal(pc.paired_chunk.shard, p0)
+        assert torch.equal(pc.shard, p0.to(dtype))
+        assert pc._stats_pending is False and pc.overflow is False
+
+
+def test_fp32_payload_lands_in_low_precision_chunks(oracle):
+    """A reduction carried out in fp32 (chunk.py:291-296,314): the fp32 buffer is cast on landing."""
+    dtype = torch.bfloat16
+    module, opt, _ = build_workload(_tiny(), 16384, dtype, seed=7, loss_scale=1.0)
+    pc = module.param_chunks[0]
+    pl = _payload(pc.chunk_size, torch.float32, 40, scale=0.3)
+    pc.invalidate_stats()
+    pc.reduce_chunk(pl, always_fp32=True, sync=True)
+    assert torch.equal(pc.shard, pl.to(dtype))
+    assert pc.overflow is False
+
+
+def test_full_size_fused_landing_c5_properties():
+    """LLaMA-7B chunk set: 27 chunks land in one launch; the shards equal the payloads, the flags and
+    the global norm equal those of the separate stats pass (norm: 1e-6, summation order differs),
+    and the step that follows launches no stats pass."""
+    built = workloads.build('c5', seed=77)
+    opt, module = built.optimizer, built.module
+    built.land_gradients(fused=False)
+    opt.kernel_events = {}
+    opt.step()
+    plain = dict(opt.last_step_info)
+    assert 'stats' in opt.kernel_events
+
+    built.land_gradients(fused=True)
+    for pc, g in zip(module.param_chunks, built.grads):
+        assert torch.equal(pc.shard.view(torch.int16), g.view(torch.int16))
+    opt.kernel_events = {}
+    opt.step()
+    fused = opt.last_step_info
+    assert 'stats' not in opt.kernel_events
+    assert fused['found_inf'] is False and plain['found_inf'] is False
+    assert abs(fused['total_norm'] - plain['total_norm']) <= 1e-6 * plain['total_norm']
+    assert all(st['step'] == 2 for st in opt.state.values())
+    for pc in module.param_chunks:
+        assert torch.equal(pc.shard, pc.paired_chunk.shard.to(torch.float16))
+
+    # an overflow in the last valid element of the last chunk, and garbage in the padding behind it
+    last = module.param_chunks[-1]
+    built.grads[-1][last.n_valid - 1] = float('-inf')
+    built.grads[0][module.param_chunks[0].n_valid:] = float('nan')
+    built.land_gradients(fused=True)
+    opt.step()
+    assert opt.last_step_info['found_inf'] is True
+    assert opt.last_step_info['chunk_overflow'] == [False] * 26 + [True]
+    assert all(st['step'] == 2 for st in opt.state.values())

@@ -340,3 +340,81 @@ def test_valid_end_and_range_rules():
     assert O.range_pair(400, 700, 512, 512) == (0, 188)
     assert O.range_pair(100, 300, 512, 512)[0] >= O.range_pair(100, 300, 512, 512)[1]    # empty on this shard
     assert O.chunk_offsets([5, 7, 1]) == [(0, 5), (5, 12), (12, 13)]
+
+
+# ------------------------------------------------------------------------------------------------
+# gradient landing
+# ------------------------------------------------------------------------------------------------
+
+
+def _special_payload(n, dtype, seed):
+    """Random values across the whole range of the type plus the special ones."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n, generator=g) * torch.exp(torch.randn(n, generator=g) * 6.0)
+    x[:12] = torch.tensor([0.0, -0.0, float('inf'), float('-inf'), float('nan'), 65504.0, 65520.0, -65536.0, 6e-8,
+                           -6.1e-5, 1e-40, 3.3e38])
+    return x.to(dtype)
+
+
+@pytest.mark.parametrize('dtype', ['f16', 'bf16', 'f32'])
+def test_landing_same_type_moves_the_bits(oracle, dtype):
+    # every 16-bit pattern (signalling NaNs included) comes out as it went in
+    if dtype == 'f32':
+        src = np.random.default_rng(0).integers(0, 2**32, 100000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        out = oracle.land(src, CODE[dtype], CODE[dtype])
+        assert np.array_equal(out.view(np.uint32), src.view(np.uint32))
+    else:
+        src = np.arange(65536, dtype=np.uint16)
+        assert np.array_equal(oracle.land(src, CODE[dtype], CODE[dtype]), src)
+
+
+@pytest.mark.parametrize('dtype', ['f16', 'bf16'])
+def test_landing_from_fp32_is_torchs_cast(oracle, dtype):
+    x = _special_payload(200000, torch.float32, 1)
+    want = bits_of(x.to(TORCH[dtype]))
+    got = oracle.land(x.numpy().copy(), O.F32, CODE[dtype])
+    nan = np.isnan(x.numpy())
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.all(np.isnan(oracle.lowp_to_f32(got[nan], CODE[dtype])))
+
+
+@pytest.mark.parametrize('dtype', ['f16', 'bf16', 'f32'])
+@pytest.mark.parametrize('pg', [2, 4, 8, 64])
+def test_landing_scaled_by_a_power_of_two_is_torchs_inplace_division(oracle, dtype, pg):
+    # payload /= pg_size (chunk.py:299): for a power of two the division and the multiplication by
+    # the reciprocal are the same correctly rounded result, so torch's CPU division pins it
+    x = _special_payload(200000, TORCH[dtype], pg)
+    want = x.clone()
+    want /= pg
+    src = bits_of(x)
+    got = oracle.land(src, CODE[dtype], CODE[dtype], mul=1.0 / pg)
+    wb = bits_of(want)
+    if dtype == 'f32':
+        nan = np.isnan(wb)
+        assert np.array_equal(got.view(np.uint32)[~nan], wb.view(np.uint32)[~nan]) and np.all(np.isnan(got[nan]))
+    else:
+        nan = np.isnan(oracle.lowp_to_f32(wb, CODE[dtype]))
+        assert np.array_equal(got[~nan], wb[~nan])
+        assert np.all(np.isnan(oracle.lowp_to_f32(got[nan], CODE[dtype])))
+
+
+@pytest.mark.parametrize('dtype', ['f16', 'bf16'])
+def test_landing_fp32_payload_scaled_then_cast(oracle, dtype):
+    # the always-fp32 reduction (chunk.py:291-299,314): fp32 payload / pg, then shard.copy_ casts
+    x = _special_payload(100000, torch.float32, 9)
+    want = x.clone()
+    want /= 4
+    wb = bits_of(want.to(TORCH[dtype]))
+    got = oracle.land(x.numpy().copy(), O.F32, CODE[dtype], mul=0.25)
+    nan = np.isnan(x.numpy())
+    assert np.array_equal(got[~nan], wb[~nan])
+
+
+def test_landing_rounds_twice_not_once(oracle):
+    # a value where rounding the product to fp16 first matters is impossible for powers of two, so
+    # use mul = 1/3: (fp16(x) * f32(1/3)) -> fp16 must equal the two-step result computed with numpy
+    x = np.random.default_rng(4).standard_normal(50000).astype(np.float16)
+    third = np.float32(1.0) / np.float32(3.0)
+    want = (x.astype(np.float32) * third).astype(np.float16)
+    got = oracle.land(x.view(np.uint16), O.F16, O.F16, mul=float(third))
+    assert np.array_equal(got, want.view(np.uint16))
