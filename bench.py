@@ -81,6 +81,66 @@ def cpu_baseline(built, sample_elems: int, steps: int = 3):
     }
 
 
+def fused_landing_leg(built, steps):
+    """The same step when the gradients arrive through the landing launch that leaves the flags on
+    the device: the step then holds no pass over the gradients (28 B per valid element).  Reports
+    the landing launch itself next to the plain device copy it replaces (both outside the step)."""
+    opt = built.optimizer
+    chunks = built.module.param_chunks
+    n_alloc, n_valid = built.n_alloc, built.n_valid
+    esize = built.grads[0].element_size()
+
+    def timed(fn):
+        b, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        b.record()
+        fn()
+        e.record()
+        e.synchronize()
+        return b.elapsed_time(e) * 1e-3
+
+    def plain():
+        for pc, g in zip(chunks, built.grads):
+            pc.shard.copy_(g)
+
+    plain_s, land_s, step_s = [], [], []
+    for i in range(steps + 1):
+        t_plain = timed(plain)
+        for pc in chunks:
+            pc.invalidate_stats()
+        t_land = timed(lambda: built.land_gradients(fused=True))
+        opt.kernel_events = {}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert opt.last_step_info['found_inf'] is False and 'stats' not in opt.kernel_events
+        if i > 0:
+            plain_s.append(t_plain)
+            land_s.append(t_land)
+            step_s.append(dt)
+    opt.kernel_events = None
+    t_step, t_land, t_plain = float(np.mean(step_s)), float(np.mean(land_s)), float(np.mean(plain_s))
+    return {
+        'what': 'gradients landed by land_grads_kernel (copy + flags in one pass, outside the step); '
+                'the step fetches the flags and runs the update',
+        'steps': steps,
+        'ms_per_step': t_step * 1e3,
+        'elements_per_sec': n_valid / t_step,
+        'step_gbps_28B': BYTES_UPDATE * n_valid / t_step / 1e9,
+        'step_frac_28B': BYTES_UPDATE * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
+        'land_kernel': {
+            'kernel': 'land_grads_kernel+stats_finish_kernel',
+            'ms_per_launch': t_land * 1e3,
+            'bytes_per_launch': 2 * esize * n_alloc,
+            'achieved': 2 * esize * n_alloc / t_land / 1e9,
+            'unit': 'GB/s',
+            'frac': 2 * esize * n_alloc / t_land / 1e9 / HBM_PEAK_GBPS,
+            'plain_copy_ms': t_plain * 1e3,
+        },
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -93,6 +153,9 @@ def main():
     ap.add_argument('--calibrate-copy', type=float, default=0.0,
                     help='instead of the benchmark, run three plain device copies of this many GiB (a kernel of '
                     'known traffic, to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit')
+    ap.add_argument('--landing-steps', type=int, default=5,
+                    help='steps of the additional leg in which the gradients arrive through the fused landing '
+                    'launch (0: skip the leg)')
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -211,6 +274,8 @@ def main():
         },
         'build_s': t_build,
     }
+    if args.landing_steps > 0:
+        out['fused_landing'] = fused_landing_leg(built, args.landing_steps)
     if args.cpu_sample > 0:
         out['cpu_baseline'] = cpu_baseline(built, args.cpu_sample)
     print(json.dumps(out))

@@ -30,7 +30,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg',
            'elx_sizeof_hyper', 'elx_sizeof_stats', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
-           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_land_grads_mt', 'elx_land_max_blocks')
+           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_land_grads_mt', 'elx_land_max_blocks', 'elx_land_tile_elems', 'elx_land_fold_blocks')
 
 
 class ElxError(RuntimeError):
@@ -60,7 +60,7 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
-                 'elx_refresh_piece_elems', 'elx_land_max_blocks'):
+                 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -72,6 +72,8 @@ def load() -> ctypes.CDLL:
     L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_writeback_mt.restype = cint
     L.elx_writeback_mt.argtypes = [vp, u32, cint, u32, u32, vp]
+    L.elx_land_tile_elems.restype = u32
+    L.elx_land_tile_elems.argtypes = [cint]
     L.elx_land_grads_mt.restype = cint
     L.elx_land_grads_mt.argtypes = [vp, u32, cint, cint, flt, u32, vp, vp, u32, vp]
 
@@ -171,8 +173,22 @@ def land_max_blocks() -> int:
     return int(load().elx_land_max_blocks())
 
 
+def land_tile_elems(src_dtype: int) -> int:
+    return int(load().elx_land_tile_elems(src_dtype))
+
+
+def land_fold_blocks() -> int:
+    return int(load().elx_land_fold_blocks())
+
+
+def land_workspace_records(n_rows: int, blocks_per_row: int) -> int:
+    """ElxStats records the landing launch needs as workspace."""
+    return n_rows * (blocks_per_row + land_fold_blocks())
+
+
 def land_grads_mt(d_rows: int, n_rows: int, src_dtype: int, dst_dtype: int, mul: float, blocks_per_row: int,
-                  d_partials: int, d_stats: int, aligned: bool, stream: int) -> None:
+                  d_partials: int, d_stats: int, aligned: bool, stream: int, blocks_per_cu: int = 0) -> None:
+    flags = (0 if aligned else ELX_FLAG_SCALAR_ONLY) | ((blocks_per_cu & 0xFF) << 8)
     check('elx_land_grads_mt',
           load().elx_land_grads_mt(d_rows, n_rows, src_dtype, dst_dtype, mul, blocks_per_row, d_partials, d_stats,
-                                   0 if aligned else ELX_FLAG_SCALAR_ONLY, stream))
+                                   flags, stream))

@@ -118,12 +118,13 @@ def l2_norm_from_sumsq(sumsq: float) -> float:
     return float(np.float32(math.sqrt(sumsq)))**2
 
 
-def land_launch_blocks(n_alloc_max: int) -> int:
-    """Workgroups per row of the landing launch: one per 16 Ki elements, at most 1024."""
-    return int(max(1, min(LAND_BLOCKS_PER_ROW, _abi.land_max_blocks(), math.ceil(n_alloc_max / 16384))))
+def land_launch_blocks(n_alloc_max: int, src_dtype: int) -> int:
+    """Workgroups per row of the landing launch: one per tile."""
+    tile = _abi.land_tile_elems(src_dtype)
+    return int(max(1, min(_abi.land_max_blocks(), (n_alloc_max + tile - 1) // tile)))
 
 
-LAND_BLOCKS_PER_ROW = 1024
+LAND_BLOCKS_PER_CU = 0    # 0: the library default
 
 
 class StatsArena:
@@ -194,9 +195,9 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
         rows[i]['n_alloc'] = c.shard_size
         rows[i]['n_valid'] = c.n_valid
     aligned = bool(np.all(rows['grad'] % 16 == 0) and np.all(rows['lowp_out'] % 16 == 0))
-    bpr = land_launch_blocks(int(rows['n_alloc'].max()))
+    bpr = land_launch_blocks(int(rows['n_alloc'].max()), src_code)
     ws = chunks[0]._workspace
-    need = len(rows) * bpr * arena.itemsize
+    need = _abi.land_workspace_records(len(rows), bpr) * arena.itemsize
     buf = ws.get('land')
     if buf is None or buf.numel() < need:
         buf = ws['land'] = torch.empty(need, dtype=torch.uint8, device=device)
@@ -205,7 +206,7 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
         cached = ws['land_table'] = DeviceTable(rows, device)
     stream = torch.cuda.current_stream(device).cuda_stream
     _abi.land_grads_mt(cached.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
-                       arena.ptr(chunks[0]._stats_slot), aligned, stream)
+                       arena.ptr(chunks[0]._stats_slot), aligned, stream, LAND_BLOCKS_PER_CU)
     for c in chunks:
         c._overflow = False
         c._l2_norm = None

@@ -593,11 +593,19 @@ __global__ __launch_bounds__(kStatsThreads) void stats_finish_kernel(const ElxSt
 // they sit in the shard afterwards, which is what the flags of the reference are taken from.  A row
 // uses `grad` as the source, `lowp_out` as the destination.  With MUL the product is first rounded
 // to the source type (an in-place scaling of the payload), then cast.  Without MUL and with equal
-// types the bits are moved untouched.  Grid (blocks_per_row, n_rows); a workgroup strides over
-// tiles of 256 lanes x one 128-bit load x kLandUnroll.
-constexpr int kLandThreads = 256;
-constexpr int kLandUnroll = 2;
-constexpr uint32_t kMaxLandBlocks = 8192;
+// types the bits are moved untouched.
+//
+// A copy is a 1:1 read/write stream like the update, and wants the same shape: one wavefront per
+// workgroup, one tile per workgroup (4 x 128-bit loads per lane: 4 KiB of source), residency capped
+// through the LDS reservation, tiles handed out in address order by the dispatcher.  Grid
+// (blocks_per_row, n_rows); when a row has more tiles than blocks a workgroup takes several
+// (stride gridDim.x).  Every workgroup leaves one ElxStats partial, folded afterwards in a fixed
+// order by stats_fold_kernel / stats_finish_kernel.
+constexpr int kLandUnroll = 4;
+constexpr uint32_t kMaxLandBlocks = 1u << 20;
+constexpr uint32_t kDefaultLandBlocksPerCu = 10;
+constexpr uint32_t kFoldBlocks = 64;           // first-stage workgroups per row when partials are many
+constexpr uint32_t kFoldThreshold = 2048;      // partials per row above which the fold has two stages
 
 template <int SD, int DD, bool MUL>
 __device__ __forceinline__ typename Elem<DD>::scalar land_elem(typename Elem<SD>::scalar x, float mul, float &as_f32) {
@@ -613,68 +621,116 @@ __device__ __forceinline__ typename Elem<DD>::scalar land_elem(typename Elem<SD>
     }
 }
 
+template <int BYTES>
+struct LaneIo;
+template <>
+struct LaneIo<16> {
+    typedef u32x4 raw;
+    static __device__ __forceinline__ raw load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxLoad);
+    }
+    static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, raw x) {
+        __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)off, 0, kAuxStore);
+    }
+};
+template <>
+struct LaneIo<8> {
+    typedef u32x2 raw;
+    static __device__ __forceinline__ raw load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kAuxLoad);
+    }
+    static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, raw x) {
+        __builtin_amdgcn_raw_buffer_store_b64(x, r, (int)off, 0, kAuxStore);
+    }
+};
+
 template <int SD, int DD, bool MUL>
-__global__ __launch_bounds__(kLandThreads) void land_grads_kernel(const ElxChunk *__restrict__ rows, uint32_t bpr,
-                                                                  float mul, ElxStats *__restrict__ partials,
-                                                                  uint32_t scalar_only) {
+__global__ __launch_bounds__(kWave) void land_grads_kernel(const ElxChunk *__restrict__ rows, float mul,
+                                                           ElxStats *__restrict__ partials, uint32_t scalar_only) {
     typedef typename Elem<SD>::scalar sscalar;
     typedef typename Elem<DD>::scalar dscalar;
-    constexpr uint32_t kEpl = 16 / sizeof(sscalar);
-    constexpr uint32_t kLSpan = kLandThreads * kEpl;
+    constexpr uint32_t kEpl = 16 / sizeof(sscalar);              // elements per lane per 128-bit load
+    constexpr uint32_t kLSpan = kWave * kEpl;
     constexpr uint32_t kLTile = kLSpan * kLandUnroll;
+    constexpr int kDstBytes = (int)(kEpl * sizeof(dscalar));     // 16, or 8 for fp32 -> 16-bit
     typedef sscalar svec __attribute__((ext_vector_type(kEpl)));
     typedef dscalar dvec __attribute__((ext_vector_type(kEpl)));
 
-    const ElxChunk c = rows[blockIdx.y];
+    const ElxChunk c = load_chunk_row(rows + blockIdx.y);
     const sscalar *src = reinterpret_cast<const sscalar *>(c.grad);
     dscalar *dst = reinterpret_cast<dscalar *>(c.lowp_out);
     const uint64_t n = (src && dst) ? c.n_alloc : 0;
     const uint64_t nv = c.n_valid < n ? c.n_valid : n;
-    const uint64_t n_tiles = (n + kLTile - 1) / kLTile;
 
+    float acc = 0.0f, poison = 0.0f;
     double sum = 0.0;
-    float poison = 0.0f;
-    for (uint64_t t = blockIdx.x; t < n_tiles; t += bpr) {
-        const uint64_t base = t * kLTile;
-        float acc = 0.0f;
+    for (uint64_t base = (uint64_t)blockIdx.x * kLTile; base < n; base += (uint64_t)gridDim.x * kLTile) {
         if (base + kLTile <= n && !scalar_only && (base + kLTile <= nv || base >= nv)) {
-            const bool counted = base < nv;    // wave-uniform
-            const svec *sp = reinterpret_cast<const svec *>(src + base) + threadIdx.x;
-            dvec *dp = reinterpret_cast<dvec *>(dst + base) + threadIdx.x;
+            const __amdgpu_buffer_rsrc_t sr = tile_rsrc(src + base, kLTile * sizeof(sscalar));
+            const __amdgpu_buffer_rsrc_t dr = tile_rsrc(dst + base, kLTile * sizeof(dscalar));
             svec S[kLandUnroll];
 #pragma unroll
-            for (int u = 0; u < kLandUnroll; ++u) S[u] = ld_stream(sp + u * kLandThreads);
+            for (int u = 0; u < kLandUnroll; ++u)
+                S[u] = __builtin_bit_cast(svec, LaneIo<16>::load(sr, (threadIdx.x + u * kWave) * 16u));
+            float F[kLandUnroll][kEpl];
 #pragma unroll
             for (int u = 0; u < kLandUnroll; ++u) {
                 dvec D;
-                float F[kEpl];
 #pragma unroll
-                for (uint32_t k = 0; k < kEpl; ++k) D[k] = land_elem<SD, DD, MUL>(S[u][k], mul, F[k]);
-                __builtin_nontemporal_store(D, dp + u * kLandThreads);
-                if (counted) {
+                for (uint32_t k = 0; k < kEpl; ++k) D[k] = land_elem<SD, DD, MUL>(S[u][k], mul, F[u][k]);
+                LaneIo<kDstBytes>::store(dr, (threadIdx.x + u * kWave) * (uint32_t)kDstBytes,
+                                         __builtin_bit_cast(typename LaneIo<kDstBytes>::raw, D));
+            }
+            if (base < nv) {    // wave-uniform: the tile lies inside the valid head
 #pragma unroll
-                    for (uint32_t k = 0; k < kEpl; ++k) stats_elem(F[k], acc, poison);
-                }
+                for (int u = 0; u < kLandUnroll; ++u)
+#pragma unroll
+                    for (uint32_t k = 0; k < kEpl; ++k) stats_elem(F[u][k], acc, poison);
             }
         } else {
             const uint64_t left = n - base;
             const uint32_t tile_n = left < kLTile ? (uint32_t)left : kLTile;
-            for (uint32_t i = threadIdx.x; i < tile_n; i += kLandThreads) {
+            for (uint32_t i = threadIdx.x; i < tile_n; i += kWave) {
                 float f;
                 dst[base + i] = land_elem<SD, DD, MUL>(src[base + i], mul, f);
                 if (base + i < nv) stats_elem(f, acc, poison);
             }
         }
         sum += (double)acc;
+        acc = 0.0f;
     }
-    uint32_t flag = (poison != poison) ? 1u : 0u;
+    sum = wave_sum(sum);
+    const uint32_t flag = __ballot(poison != poison) != 0ull ? 1u : 0u;
+    if (threadIdx.x == 0) {
+        ElxStats r;
+        r.sumsq = sum;
+        r.overflow = flag;
+        r.reserved = 0;
+        partials[(uint64_t)blockIdx.y * gridDim.x + blockIdx.x] = r;
+    }
+}
+
+// First stage of a long fold: workgroup j of row y folds its contiguous share of the row's `bpr`
+// partials into mid[y * gridDim.x + j].
+__global__ __launch_bounds__(kStatsThreads) void stats_fold_kernel(const ElxStats *__restrict__ partials, uint32_t bpr,
+                                                                   ElxStats *__restrict__ mid) {
+    const ElxStats *row = partials + (uint64_t)blockIdx.y * bpr;
+    const uint32_t share = (bpr + gridDim.x - 1) / gridDim.x;
+    const uint32_t lo = blockIdx.x * share;
+    const uint32_t hi = lo + share < bpr ? lo + share : bpr;
+    double sum = 0.0;
+    uint32_t flag = 0;
+    for (uint32_t i = lo + threadIdx.x; i < hi; i += kStatsThreads) {
+        sum += row[i].sumsq;
+        flag |= row[i].overflow;
+    }
     block_fold(sum, flag);
     if (threadIdx.x == 0) {
         ElxStats r;
         r.sumsq = sum;
         r.overflow = flag;
         r.reserved = 0;
-        partials[(uint64_t)blockIdx.y * bpr + blockIdx.x] = r;
+        mid[(uint64_t)blockIdx.y * gridDim.x + blockIdx.x] = r;
     }
 }
 
@@ -876,16 +932,21 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, in
     if (!is_lowp_or_f32(src_dtype) || !is_lowp_or_f32(dst_dtype)) return ELX_E_DTYPE;
     if (src_dtype != dst_dtype && src_dtype != ELX_F32) return ELX_E_DTYPE;
     if (n_rows == 0 || n_rows > 65535u || blocks_per_row == 0 || blocks_per_row > kMaxLandBlocks) return ELX_E_SIZE;
-    if (!(mul == mul) || mul <= 0.0f) return ELX_E_RANGE;
+    if (!(mul == mul) || mul <= 0.0f || mul > 3.0e38f) return ELX_E_RANGE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const dim3 grid(blocks_per_row, n_rows), block(kLandThreads);
+    const dim3 grid(blocks_per_row, n_rows), block(kWave);
     const uint32_t so = (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u;
-#define ELX_LAND(S, D)                                                                                          \
-    if (src_dtype == S && dst_dtype == D) {                                                                     \
-        if (mul == 1.0f)                                                                                        \
-            hipLaunchKernelGGL((land_grads_kernel<S, D, false>), grid, block, 0, st, d_rows, blocks_per_row, mul, d_partials, so); \
-        else                                                                                                    \
-            hipLaunchKernelGGL((land_grads_kernel<S, D, true>), grid, block, 0, st, d_rows, blocks_per_row, mul, d_partials, so);  \
+    uint32_t lds = 0;
+    int rc = occupancy_reservation(((flags >> 8) & 0xFFu) ? ((flags >> 8) & 0xFFu) : kDefaultLandBlocksPerCu, &lds);
+    if (rc) return rc;
+    rc = ELX_E_DTYPE;
+#define ELX_LAND(S, D)                                                                                       \
+    if (src_dtype == S && dst_dtype == D) {                                                                  \
+        if (mul == 1.0f)                                                                                     \
+            hipLaunchKernelGGL((land_grads_kernel<S, D, false>), grid, block, lds, st, d_rows, mul, d_partials, so); \
+        else                                                                                                 \
+            hipLaunchKernelGGL((land_grads_kernel<S, D, true>), grid, block, lds, st, d_rows, mul, d_partials, so);  \
+        rc = (int)hipGetLastError();                                                                         \
     }
     ELX_LAND(ELX_F32, ELX_F32)
     ELX_LAND(ELX_F16, ELX_F16)
@@ -893,11 +954,23 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, in
     ELX_LAND(ELX_F32, ELX_F16)
     ELX_LAND(ELX_F32, ELX_BF16)
 #undef ELX_LAND
-    int rc = (int)hipGetLastError();
     if (rc) return rc;
-    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_rows), dim3(kStatsThreads), 0, st, d_partials, blocks_per_row, d_stats);
+    if (blocks_per_row > kFoldThreshold) {
+        ElxStats *mid = d_partials + (uint64_t)n_rows * blocks_per_row;
+        hipLaunchKernelGGL(stats_fold_kernel, dim3(kFoldBlocks, n_rows), dim3(kStatsThreads), 0, st, d_partials,
+                           blocks_per_row, mid);
+        rc = (int)hipGetLastError();
+        if (rc) return rc;
+        hipLaunchKernelGGL(stats_finish_kernel, dim3(n_rows), dim3(kStatsThreads), 0, st, mid, kFoldBlocks, d_stats);
+    } else {
+        hipLaunchKernelGGL(stats_finish_kernel, dim3(n_rows), dim3(kStatsThreads), 0, st, d_partials, blocks_per_row, d_stats);
+    }
     return (int)hipGetLastError();
 }
+
+uint32_t elx_land_tile_elems(int src_dtype) { return kWave * (16u / elem_size(src_dtype)) * kLandUnroll; }
+
+uint32_t elx_land_fold_blocks(void) { return kFoldBlocks; }
 
 uint32_t elx_land_max_blocks(void) { return kMaxLandBlocks; }
 

@@ -209,14 +209,22 @@ uint32_t elx_refresh_piece_elems(void);
  *   mul        1.0f: plain copy / cast.  Otherwise each element is multiplied in fp32, rounded to
  *              src_dtype and then cast, as the in-place `reduce_buffer /= pg_size` of chunk.py:299
  *              does on the device for mul = 1.0f / pg_size.  Must be finite and > 0.
- *   blocks_per_row  workgroups per row, 1..elx_land_max_blocks()
- *   d_partials workspace of n_rows * blocks_per_row ElxStats records (contents ignored)
+ *   blocks_per_row  workgroups per row, 1..elx_land_max_blocks().  One workgroup lands one tile of
+ *              elx_land_tile_elems(src_dtype) elements at a time; the launch streams best with one
+ *              tile per workgroup, blocks_per_row = ceil(max n_alloc / tile); with fewer, a workgroup
+ *              takes several tiles
+ *   d_partials workspace of n_rows * (blocks_per_row + elx_land_fold_blocks()) ElxStats records
+ *              (contents ignored)
  *   d_stats    n_rows results; fixed reduction order
+ *   flags      ELX_FLAG_SCALAR_ONLY when a base pointer is not 16-byte aligned; bits 8..15: cap on
+ *              resident workgroups per compute unit, 3..32 (0 = the library default, 10)
  */
 int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, int dst_dtype, float mul,
                       uint32_t blocks_per_row, ElxStats *d_partials, ElxStats *d_stats, uint32_t flags, void *stream);
 
 uint32_t elx_land_max_blocks(void);
+uint32_t elx_land_tile_elems(int src_dtype);
+uint32_t elx_land_fold_blocks(void);
 
 #ifdef __cplusplus
 }

@@ -30,13 +30,15 @@ def _land(src: torch.Tensor, dst: torch.Tensor, n_valid: int, mul: float = 1.0, 
     row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
     row['grad'], row['lowp_out'], row['n_alloc'], row['n_valid'] = src.data_ptr(), dst.data_ptr(), n, n_valid
     table = DeviceTable(row, dst.device)
-    bpr = blocks or max(1, min(1024, -(-n // 16384)))
-    ws = torch.empty((bpr + 1) * _abi.STATS_DTYPE.itemsize, dtype=torch.uint8, device=dst.device)
+    tile = _abi.land_tile_elems(CODE[src.dtype])
+    bpr = blocks or max(1, -(-n // tile))
+    recs = _abi.land_workspace_records(1, bpr)
+    ws = torch.empty((recs + 1) * _abi.STATS_DTYPE.itemsize, dtype=torch.uint8, device=dst.device)
     aligned = src.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0
     _abi.land_grads_mt(table.ptr, 1, CODE[src.dtype], CODE[dst.dtype], mul, bpr, ws.data_ptr(),
-                       ws.data_ptr() + bpr * _abi.STATS_DTYPE.itemsize, aligned,
+                       ws.data_ptr() + recs * _abi.STATS_DTYPE.itemsize, aligned,
                        torch.cuda.current_stream().cuda_stream)
-    rec = ws[bpr * _abi.STATS_DTYPE.itemsize:].cpu().numpy().view(_abi.STATS_DTYPE)
+    rec = ws[recs * _abi.STATS_DTYPE.itemsize:].cpu().numpy().view(_abi.STATS_DTYPE)
     return bool(rec['overflow'][0]), float(rec['sumsq'][0])
 
 
@@ -150,7 +152,7 @@ def test_landing_is_reproducible_and_independent_of_the_grid(oracle):
     first = _land(src, dst, n)
     assert _land(src, dst, n) == first
     ref = oracle.sumsq(to_np(src), O.F16)
-    for blocks in (1, 3, 64, 4096):
+    for blocks in (1, 3, 64, 2049, 4096):
         flag, sumsq = _land(src, dst, n, blocks=blocks)
         assert flag is False and abs(sumsq - ref) <= 1e-6 * ref
         assert torch.equal(dst, src)

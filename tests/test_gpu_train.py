@@ -102,6 +102,7 @@ def test_fp16_training_matches_master_weight_amp_and_recovers_from_overflow():
         if poison:
             pc = module.param_chunks[0]
             pc.shard[7] = float('inf')
+            pc.invalidate_stats()    # the shard changed behind the chunk's back: flags from the landing are stale
         opt.step()
         assert opt.last_step_info['found_inf'] == poison
         module.materialize_params()
