@@ -121,6 +121,37 @@ def fused_landing_leg(built, steps):
             step_s.append(dt)
     opt.kernel_events = None
     t_step, t_land, t_plain = float(np.mean(step_s)), float(np.mean(land_s)), float(np.mean(plain_s))
+
+    # the same landing straight from per-tensor gradients (views of the saved buffers stand in for
+    # the .grad tensors), next to what it replaces: a zeroed payload per chunk, one slice copy per
+    # tensor, and the copy of the payload into the shard
+    from elixir_amd.chunk import land_tensors
+    grads = {}
+    for pc, g in zip(chunks, built.grads):
+        for t, info in pc.tensors_info.items():
+            grads[t] = g[info.offset:info.end]
+
+    def slice_copies():
+        for pc in chunks:
+            payload = torch.zeros(pc.chunk_size, dtype=pc.chunk_dtype, device=pc.shard_device)
+            for t, info in pc.tensors_info.items():
+                payload[info.offset:info.end].copy_(grads[t])
+            pc.shard.copy_(payload)
+
+    pt_gpu, pt_wall, sc_gpu = [], [], []
+    for i in range(steps + 1):
+        a = timed(slice_copies)
+        for pc in chunks:
+            pc.invalidate_stats()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        b = timed(lambda: land_tensors(chunks, lambda t: grads[t]))
+        w = time.perf_counter() - t0
+        if i > 0:
+            sc_gpu.append(a)
+            pt_gpu.append(b)
+            pt_wall.append(w)
+    assert not any(pc.overflow for pc in chunks)
     return {
         'what': 'gradients landed by land_grads_kernel (copy + flags in one pass, outside the step); '
                 'the step fetches the flags and runs the update',
@@ -137,6 +168,12 @@ def fused_landing_leg(built, steps):
             'unit': 'GB/s',
             'frac': 2 * esize * n_alloc / t_land / 1e9 / HBM_PEAK_GBPS,
             'plain_copy_ms': t_plain * 1e3,
+        },
+        'per_tensor_landing': {
+            'what': 'the same launch fed by one row list over the %d per-tensor gradients (no payload)' % len(grads),
+            'ms_launch_to_done': float(np.mean(pt_gpu)) * 1e3,
+            'ms_wall_with_table_build': float(np.mean(pt_wall)) * 1e3,
+            'zero_payload_slice_copies_and_shard_copy_ms': float(np.mean(sc_gpu)) * 1e3,
         },
     }
 

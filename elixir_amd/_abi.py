@@ -75,7 +75,7 @@ def load() -> ctypes.CDLL:
     L.elx_land_tile_elems.restype = u32
     L.elx_land_tile_elems.argtypes = [cint]
     L.elx_land_grads_mt.restype = cint
-    L.elx_land_grads_mt.argtypes = [vp, u32, cint, cint, flt, u32, vp, vp, u32, vp]
+    L.elx_land_grads_mt.argtypes = [vp, u32, vp, u32, cint, cint, flt, u32, vp, vp, u32, vp]
 
     if L.elx_version() != ELX_ABI_VERSION:
         raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
@@ -181,14 +181,15 @@ def land_fold_blocks() -> int:
     return int(load().elx_land_fold_blocks())
 
 
-def land_workspace_records(n_rows: int, blocks_per_row: int) -> int:
+def land_workspace_records(n_rows: int, blocks_per_row: int, n_slots: int = 0) -> int:
     """ElxStats records the landing launch needs as workspace."""
-    return n_rows * (blocks_per_row + land_fold_blocks())
+    return n_rows * blocks_per_row + (n_slots or n_rows) * land_fold_blocks()
 
 
 def land_grads_mt(d_rows: int, n_rows: int, src_dtype: int, dst_dtype: int, mul: float, blocks_per_row: int,
-                  d_partials: int, d_stats: int, aligned: bool, stream: int, blocks_per_cu: int = 0) -> None:
+                  d_partials: int, d_stats: int, aligned: bool, stream: int, blocks_per_cu: int = 0,
+                  d_slot_offsets: int = 0, n_slots: int = 0) -> None:
     flags = (0 if aligned else ELX_FLAG_SCALAR_ONLY) | ((blocks_per_cu & 0xFF) << 8)
     check('elx_land_grads_mt',
-          load().elx_land_grads_mt(d_rows, n_rows, src_dtype, dst_dtype, mul, blocks_per_row, d_partials, d_stats,
-                                   flags, stream))
+          load().elx_land_grads_mt(d_rows, n_rows, d_slot_offsets or None, n_slots, src_dtype, dst_dtype, mul,
+                                   blocks_per_row, d_partials, d_stats, flags, stream))

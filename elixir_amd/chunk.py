@@ -214,6 +214,112 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
         c._stats_pending = True
 
 
+def _land_block_elems(total: int, tile: int) -> int:
+    """Rows of a per-tensor landing are blocks of this many elements: a power of two, at least 16
+    tiles, chosen so that the launch stays below about 32 Ki rows."""
+    block = 16 * tile
+    while block * 16384 < total:
+        block <<= 1
+    return block
+
+
+def land_rows(pieces, n_slots: int, block: int, ssize: int, dsize: int):
+    """The row table of a per-tensor landing.  ``pieces``: (slot, source address or 0 for zeros,
+    destination address, element count), the pieces of one slot consecutive and slots ascending.
+    Every piece becomes ceil(count / block) rows.  Returns (rows, slot_offsets) where the rows
+    [slot_offsets[s], slot_offsets[s + 1]) belong to slot s."""
+    per_slot = np.zeros(n_slots + 1, dtype=np.int64)
+    if not pieces:
+        return np.zeros(0, dtype=_abi.CHUNK_DTYPE), per_slot.astype(np.uint32)
+    slot, src, dst, count = (np.array(col, dtype=np.uint64) for col in zip(*pieces))
+    n_rows = (count + np.uint64(block - 1)) // np.uint64(block)
+    first_row = np.concatenate(([0], np.cumsum(n_rows)[:-1])).astype(np.uint64)
+    total = int(n_rows.sum())
+    piece = np.repeat(np.arange(len(pieces)), n_rows.astype(np.int64))
+    start = (np.arange(total, dtype=np.uint64) - first_row[piece]) * np.uint64(block)    # element offset in the piece
+    rows = np.zeros(total, dtype=_abi.CHUNK_DTYPE)
+    has_src = src[piece] != 0
+    rows['grad'] = np.where(has_src, src[piece] + start * np.uint64(ssize), 0)
+    rows['lowp_out'] = dst[piece] + start * np.uint64(dsize)
+    rows['n_alloc'] = np.minimum(np.uint64(block), count[piece] - start)
+    rows['n_valid'] = np.where(has_src, rows['n_alloc'], 0)
+    np.add.at(per_slot, slot.astype(np.int64) + 1, n_rows.astype(np.int64))
+    return rows, np.cumsum(per_slot).astype(np.uint32)
+
+
+def land_tensors(chunks: List['Chunk'], grad_of, mul: float = 1.0) -> None:
+    """Lands chunks straight from the per-tensor gradients, in ONE launch for the whole list:
+    ``grad_of(tensor)`` is the gradient of a tensor of the chunk (contiguous, on the shard's device,
+    all of one dtype: the chunk's or fp32).  Every gradient is copied (cast) into its slice of the
+    shard, what no tensor covers is zeroed, and the flags of each chunk are left in its slot of the
+    device arena, as ``land_chunks`` leaves them.  Replaces the per-parameter copies of
+    chunk.py:386-393 / module.py:177-190, the intermediate payload, and chunk.py:309-315 + 345-356.
+
+    Each gradient is listed as rows of equal blocks (the last one shorter); a slice whose byte
+    offset in the shard is not a multiple of 16 is moved element by element by its workgroups."""
+    if not chunks:
+        return
+    device = chunks[0].shard_device
+    if device.type != 'cuda':
+        raise RuntimeError('gradients land through the HIP kernels: shards must be on the GPU')
+    dst_dtype = chunks[0].chunk_dtype
+    dst_code = dtype_code(dst_dtype)
+    dsize = chunks[0].shard.element_size()
+    src_dtype = None
+    pieces = []    # (chunk index, src address or 0, begin in the shard, element count)
+    for ci, c in enumerate(chunks):
+        assert not c.is_init and c.shard_device == device and c.chunk_dtype == dst_dtype
+        covered = 0
+        for tensor, info in sorted(c.tensors_info.items(), key=lambda kv: kv[1].offset):
+            g = grad_of(tensor)
+            assert g is not None, 'every tensor of a chunk needs a gradient before the chunk can land'
+            assert g.device == device and g.is_contiguous() and g.numel() == info.end - info.offset
+            src_dtype = src_dtype or g.dtype
+            assert g.dtype == src_dtype, 'all gradients of one landing must have one dtype'
+            begin, end = max(info.offset, c.shard_begin) - c.shard_begin, min(info.end, c.shard_end) - c.shard_begin
+            if begin >= end:
+                continue
+            if begin > covered:
+                pieces.append((ci, 0, covered, begin - covered))
+            pieces.append((ci, g.data_ptr() + (begin + c.shard_begin - info.offset) * g.element_size(), begin, end - begin))
+            covered = end
+        if covered < c.shard_size:
+            pieces.append((ci, 0, covered, c.shard_size - covered))
+    src_code = dtype_code(src_dtype if src_dtype is not None else dst_dtype)
+    ssize = 4 if src_code == _abi.ELX_F32 else 2
+    tile = _abi.land_tile_elems(src_code)
+    block = _land_block_elems(sum(c.shard_size for c in chunks), tile)
+
+    rows, slot_offsets = land_rows([(ci, src, chunks[ci].shard.data_ptr() + begin * dsize, count)
+                                    for ci, src, begin, count in pieces], len(chunks), block, ssize, dsize)
+    if len(rows) > 65535:
+        raise RuntimeError(f'{len(rows)} rows in one landing launch: land fewer chunks at a time')
+
+    arena = StatsArena.get(device)
+    slots = [c._stats_slot for c in chunks]
+    if slots[0] is None or any(b is None or b != a + 1 for a, b in zip(slots, slots[1:])):
+        first = arena.new_slots(len(chunks))
+        for i, c in enumerate(chunks):
+            c._stats_slot = first + i
+    bpr = max(1, (int(rows['n_alloc'].max()) + tile - 1) // tile)
+    ws = chunks[0]._workspace
+    need = _abi.land_workspace_records(len(rows), bpr, len(chunks)) * arena.itemsize
+    buf = ws.get('land')
+    if buf is None or buf.numel() < need:
+        buf = ws['land'] = torch.empty(need, dtype=torch.uint8, device=device)
+    table = ws['land_table'] = DeviceTable(rows, device)
+    offsets = ws['land_offsets'] = torch.from_numpy(slot_offsets.view(np.int32).copy()).to(device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    _abi.land_grads_mt(table.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
+                       arena.ptr(chunks[0]._stats_slot), True, stream, LAND_BLOCKS_PER_CU,
+                       d_slot_offsets=offsets.data_ptr(), n_slots=len(chunks))
+    for c in chunks:
+        c._overflow = False
+        c._l2_norm = None
+        c._stats_fresh = False
+        c._stats_pending = True
+
+
 def resolve_pending_stats(chunks: List['Chunk']) -> None:
     """Fetches the landing records of every chunk in the list that has one outstanding: one copy
     per device."""

@@ -657,16 +657,19 @@ __global__ __launch_bounds__(kWave) void land_grads_kernel(const ElxChunk *__res
     typedef dscalar dvec __attribute__((ext_vector_type(kEpl)));
 
     const ElxChunk c = load_chunk_row(rows + blockIdx.y);
-    const sscalar *src = reinterpret_cast<const sscalar *>(c.grad);
+    const sscalar *src = reinterpret_cast<const sscalar *>(c.grad);    // NULL: the source is all zeros
     dscalar *dst = reinterpret_cast<dscalar *>(c.lowp_out);
-    const uint64_t n = (src && dst) ? c.n_alloc : 0;
+    const uint64_t n = dst ? c.n_alloc : 0;
     const uint64_t nv = c.n_valid < n ? c.n_valid : n;
+    // 128-bit accesses need both ends of the row on a 16-byte boundary (tiles keep that alignment)
+    const bool vec_ok = !scalar_only && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
 
     float acc = 0.0f, poison = 0.0f;
     double sum = 0.0;
     for (uint64_t base = (uint64_t)blockIdx.x * kLTile; base < n; base += (uint64_t)gridDim.x * kLTile) {
-        if (base + kLTile <= n && !scalar_only && (base + kLTile <= nv || base >= nv)) {
-            const __amdgpu_buffer_rsrc_t sr = tile_rsrc(src + base, kLTile * sizeof(sscalar));
+        if (base + kLTile <= n && vec_ok && (base + kLTile <= nv || base >= nv)) {
+            // an empty resource returns zero for every lane: the NULL source without a branch
+            const __amdgpu_buffer_rsrc_t sr = tile_rsrc(src ? src + base : nullptr, src ? kLTile * sizeof(sscalar) : 0u);
             const __amdgpu_buffer_rsrc_t dr = tile_rsrc(dst + base, kLTile * sizeof(dscalar));
             svec S[kLandUnroll];
 #pragma unroll
@@ -692,7 +695,8 @@ __global__ __launch_bounds__(kWave) void land_grads_kernel(const ElxChunk *__res
             const uint32_t tile_n = left < kLTile ? (uint32_t)left : kLTile;
             for (uint32_t i = threadIdx.x; i < tile_n; i += kWave) {
                 float f;
-                dst[base + i] = land_elem<SD, DD, MUL>(src[base + i], mul, f);
+                const sscalar x = src ? src[base + i] : sscalar(0);
+                dst[base + i] = land_elem<SD, DD, MUL>(x, mul, f);
                 if (base + i < nv) stats_elem(f, acc, poison);
             }
         }
@@ -710,19 +714,33 @@ __global__ __launch_bounds__(kWave) void land_grads_kernel(const ElxChunk *__res
     }
 }
 
-// First stage of a long fold: workgroup j of row y folds its contiguous share of the row's `bpr`
-// partials into mid[y * gridDim.x + j].
+// Folding the partials of a landing launch.  The partials are laid out [row][bpr]; the rows that
+// feed one output record ("slot") are consecutive, so a slot owns one contiguous run of partials:
+// rows [offsets[slot], offsets[slot + 1]) when an offsets table is given, row `slot` otherwise.
+__device__ __forceinline__ void slot_range(const uint32_t *__restrict__ offsets, uint32_t slot, uint32_t bpr,
+                                           uint64_t &begin, uint64_t &count) {
+    const uint32_t r0 = offsets ? offsets[slot] : slot;
+    const uint32_t r1 = offsets ? offsets[slot + 1] : slot + 1;
+    begin = (uint64_t)r0 * bpr;
+    count = (uint64_t)(r1 - r0) * bpr;
+}
+
+// First stage: workgroup j of slot y folds its contiguous share of the slot's partials into
+// mid[y * gridDim.x + j].  Second stage: stats_finish_kernel over gridDim.x records per slot.
 __global__ __launch_bounds__(kStatsThreads) void stats_fold_kernel(const ElxStats *__restrict__ partials, uint32_t bpr,
+                                                                   const uint32_t *__restrict__ offsets,
                                                                    ElxStats *__restrict__ mid) {
-    const ElxStats *row = partials + (uint64_t)blockIdx.y * bpr;
-    const uint32_t share = (bpr + gridDim.x - 1) / gridDim.x;
-    const uint32_t lo = blockIdx.x * share;
-    const uint32_t hi = lo + share < bpr ? lo + share : bpr;
+    uint64_t begin, count;
+    slot_range(offsets, blockIdx.y, bpr, begin, count);
+    const uint64_t share = (count + gridDim.x - 1) / gridDim.x;
+    const uint64_t lo = blockIdx.x * share;
+    const uint64_t hi = lo + share < count ? lo + share : count;
+    const ElxStats *run = partials + begin;
     double sum = 0.0;
     uint32_t flag = 0;
-    for (uint32_t i = lo + threadIdx.x; i < hi; i += kStatsThreads) {
-        sum += row[i].sumsq;
-        flag |= row[i].overflow;
+    for (uint64_t i = lo + threadIdx.x; i < hi; i += kStatsThreads) {
+        sum += run[i].sumsq;
+        flag |= run[i].overflow;
     }
     block_fold(sum, flag);
     if (threadIdx.x == 0) {
@@ -926,12 +944,15 @@ int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype
 
 uint32_t elx_refresh_piece_elems(void) { return kRefreshPiece; }
 
-int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, int dst_dtype, float mul,
-                      uint32_t blocks_per_row, ElxStats *d_partials, ElxStats *d_stats, uint32_t flags, void *stream) {
+int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d_slot_offsets, uint32_t n_slots,
+                      int src_dtype, int dst_dtype, float mul, uint32_t blocks_per_row, ElxStats *d_partials,
+                      ElxStats *d_stats, uint32_t flags, void *stream) {
     if (!d_rows || !d_partials || !d_stats) return ELX_E_NULL;
     if (!is_lowp_or_f32(src_dtype) || !is_lowp_or_f32(dst_dtype)) return ELX_E_DTYPE;
     if (src_dtype != dst_dtype && src_dtype != ELX_F32) return ELX_E_DTYPE;
     if (n_rows == 0 || n_rows > 65535u || blocks_per_row == 0 || blocks_per_row > kMaxLandBlocks) return ELX_E_SIZE;
+    if (!d_slot_offsets) n_slots = n_rows;
+    if (n_slots == 0 || n_slots > n_rows) return ELX_E_SIZE;
     if (!(mul == mul) || mul <= 0.0f || mul > 3.0e38f) return ELX_E_RANGE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const dim3 grid(blocks_per_row, n_rows), block(kWave);
@@ -955,16 +976,17 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, in
     ELX_LAND(ELX_F32, ELX_BF16)
 #undef ELX_LAND
     if (rc) return rc;
-    if (blocks_per_row > kFoldThreshold) {
-        ElxStats *mid = d_partials + (uint64_t)n_rows * blocks_per_row;
-        hipLaunchKernelGGL(stats_fold_kernel, dim3(kFoldBlocks, n_rows), dim3(kStatsThreads), 0, st, d_partials,
-                           blocks_per_row, mid);
-        rc = (int)hipGetLastError();
-        if (rc) return rc;
-        hipLaunchKernelGGL(stats_finish_kernel, dim3(n_rows), dim3(kStatsThreads), 0, st, mid, kFoldBlocks, d_stats);
-    } else {
+    // one slot per row and few partials: the finish alone; otherwise two stages
+    if (!d_slot_offsets && blocks_per_row <= kFoldThreshold) {
         hipLaunchKernelGGL(stats_finish_kernel, dim3(n_rows), dim3(kStatsThreads), 0, st, d_partials, blocks_per_row, d_stats);
+        return (int)hipGetLastError();
     }
+    ElxStats *mid = d_partials + (uint64_t)n_rows * blocks_per_row;
+    hipLaunchKernelGGL(stats_fold_kernel, dim3(kFoldBlocks, n_slots), dim3(kStatsThreads), 0, st, d_partials,
+                       blocks_per_row, d_slot_offsets, mid);
+    rc = (int)hipGetLastError();
+    if (rc) return rc;
+    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_slots), dim3(kStatsThreads), 0, st, mid, kFoldBlocks, d_stats);
     return (int)hipGetLastError();
 }
 

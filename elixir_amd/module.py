@@ -16,7 +16,7 @@ from typing import Any, Dict, Iterable, List, Mapping, NamedTuple, Optional, Seq
 import torch
 import torch.nn as nn
 
-from .chunk import Chunk, ChunkGroup, gpu_device
+from .chunk import Chunk, ChunkGroup, gpu_device, land_tensors
 
 
 class ChunkPlan(NamedTuple):
@@ -219,12 +219,28 @@ class ElixirModule(nn.Module):
         self.module.zero_grad(set_to_none=True)
 
     def land_gradients(self, sync: bool = False) -> None:
-        """module.py:177-190 + chunk.py:358-393 for one process: each parameter's gradient is
-        copied into its slice of a full-size payload (zero elsewhere, as the replicated block of the
-        reference is after a gather of zero padding), and the payload overwrites the shard.  With
-        ``sync`` the flags are computed per chunk here, otherwise by the optimizer in one launch."""
+        """module.py:177-190 + chunk.py:358-393 for one process: every parameter's gradient goes
+        into its slice of the chunk's shard, what no parameter covers becomes zero (as the
+        replicated block of the reference is after a gather of zero padding), and the flags of every
+        chunk are taken in the same pass.  GPU-resident chunks land in one launch straight from the
+        ``.grad`` tensors; host-resident ones through a full-size payload and a transfer.  With
+        ``sync`` the flags are fetched here, otherwise when somebody reads them (the optimizer step
+        does, for all chunks at once)."""
         assert not self.synthetic
+        on_gpu = [c for c in self.param_chunks if c.shard_device.type == 'cuda']
+        if on_gpu:
+
+            def grad_of(param):
+                assert param.grad is not None, 'every parameter of a chunk needs a gradient before the reduction'
+                return param.grad.data.contiguous()
+
+            land_tensors(on_gpu, grad_of)
+            if sync:
+                for chunk in on_gpu:
+                    chunk.update_extra_reduce_info()
         for chunk in self.param_chunks:
+            if chunk.shard_device.type == 'cuda':
+                continue
             payload = torch.zeros(chunk.chunk_size, dtype=chunk.chunk_dtype, device=chunk.shard_device)
             for param, info in chunk.tensors_info.items():
                 assert param.grad is not None, 'every parameter of a chunk needs a gradient before the reduction'

@@ -203,8 +203,15 @@ uint32_t elx_refresh_piece_elems(void);
  * tail of Chunk.reduce, `__update_shard(reduce_buffer, self.shard)` (elixir/chunk/core/chunk.py:309-315,
  * 484-489), fused with Chunk.update_extra_reduce_info (chunk.py:345-356): the flags are known when
  * the gradients have landed, and the optimizer step needs no pass of its own over them.
- * A row reads `grad` (the payload slice that belongs to this shard, n_alloc elements of src_dtype),
- * `lowp_out` (the shard, n_alloc elements of dst_dtype), n_alloc and n_valid; nothing else.
+ * A row reads `grad` (the source: n_alloc elements of src_dtype; NULL = all zeros), `lowp_out` (the
+ * destination: n_alloc elements of dst_dtype), n_alloc and n_valid; nothing else.  A row can be a whole
+ * shard with the payload slice that belongs to it, or any piece of one: listing every tensor's
+ * gradient as rows (cut into equal blocks) with the gaps and the padding as zero rows lands a chunk
+ * straight from the per-parameter gradients, which also replaces the copies of
+ * Chunk.copy_tensor_to_chunk_slice (chunk.py:386-393) and the intermediate payload.
+ *   d_slot_offsets / n_slots  NULL: one result record per row (n_slots is ignored).  Otherwise
+ *              n_slots + 1 ascending row indices: the rows [offsets[s], offsets[s+1]) feed d_stats[s]
+ *              (the rows of one chunk are consecutive), offsets[0] = 0, offsets[n_slots] = n_rows
  *   src_dtype / dst_dtype  equal, or fp32 -> fp16 / bf16 (a payload reduced in fp32, chunk.py:291-296)
  *   mul        1.0f: plain copy / cast.  Otherwise each element is multiplied in fp32, rounded to
  *              src_dtype and then cast, as the in-place `reduce_buffer /= pg_size` of chunk.py:299
@@ -213,14 +220,16 @@ uint32_t elx_refresh_piece_elems(void);
  *              elx_land_tile_elems(src_dtype) elements at a time; the launch streams best with one
  *              tile per workgroup, blocks_per_row = ceil(max n_alloc / tile); with fewer, a workgroup
  *              takes several tiles
- *   d_partials workspace of n_rows * (blocks_per_row + elx_land_fold_blocks()) ElxStats records
- *              (contents ignored)
- *   d_stats    n_rows results; fixed reduction order
- *   flags      ELX_FLAG_SCALAR_ONLY when a base pointer is not 16-byte aligned; bits 8..15: cap on
- *              resident workgroups per compute unit, 3..32 (0 = the library default, 10)
+ *   d_partials workspace of n_rows * blocks_per_row + n_slots * elx_land_fold_blocks() ElxStats
+ *              records (contents ignored)
+ *   d_stats    n_slots results; fixed reduction order
+ *   flags      ELX_FLAG_SCALAR_ONLY forces the element-by-element path (rows whose ends are not both
+ *              16-byte aligned take it by themselves); bits 8..15: cap on resident workgroups per
+ *              compute unit, 3..32 (0 = the library default, 10)
  */
-int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, int src_dtype, int dst_dtype, float mul,
-                      uint32_t blocks_per_row, ElxStats *d_partials, ElxStats *d_stats, uint32_t flags, void *stream);
+int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d_slot_offsets, uint32_t n_slots,
+                      int src_dtype, int dst_dtype, float mul, uint32_t blocks_per_row, ElxStats *d_partials,
+                      ElxStats *d_stats, uint32_t flags, void *stream);
 
 uint32_t elx_land_max_blocks(void);
 uint32_t elx_land_tile_elems(int src_dtype);

@@ -304,3 +304,110 @@ def test_full_size_fused_landing_c5_properties():
     assert opt.last_step_info['found_inf'] is True
     assert opt.last_step_info['chunk_overflow'] == [False] * 26 + [True]
     assert all(st['step'] == 2 for st in opt.state.values())
+
+
+# ------------------------------------------------------------------------------------------------
+# landing straight from the per-tensor gradients
+# ------------------------------------------------------------------------------------------------
+
+
+def _odd():
+    """Sizes that leave most slices off the 16-byte grid, a tensor larger than one block, tiny ones."""
+    return [('w0', (5, 3)), ('w1', (1000, 37)), ('b1', (37,)), ('w2', (333, 129)), ('s', (1,)), ('w3', (64, 64)),
+            ('w4', (700, 100)), ('b4', (100,)), ('w5', (257, 255))]
+
+
+def _expected_shards(module, grads, dtype):
+    out = []
+    for pc in module.param_chunks:
+        want = torch.zeros(pc.shard_size, dtype=dtype, device=DEV)
+        for t, info in pc.tensors_info.items():
+            want[info.offset:info.end] = grads[t].flatten().to(dtype)
+        out.append(want)
+    return out
+
+
+@pytest.mark.parametrize('shapes', ['odd', 'aligned'])
+@pytest.mark.parametrize('gdtype,dtype', [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+                                          (torch.float32, torch.bfloat16), (torch.float32, torch.float32)])
+def test_land_tensors_matches_slice_copies(oracle, shapes, gdtype, dtype):
+    from elixir_amd.chunk import land_tensors
+    named = _odd() if shapes == 'odd' else [(f't{i}', (8 * (i + 1), 24 + 8 * (i % 5))) for i in range(40)]
+    module, opt, _ = build_workload(named, 1 << 17, dtype, seed=3, loss_scale=1.0, max_norm=1.0)
+    assert len(module.param_chunks) >= 2
+    params = list(module.parameters())
+    grads = {p: _payload(p.numel(), gdtype, 100 + i, scale=0.7).view(p.shape) for i, p in enumerate(params)}
+    for pc in module.param_chunks:
+        pc.shard.fill_(float('nan'))                   # whatever sat there, padding included, is overwritten
+        pc.invalidate_stats()
+    land_tensors(module.param_chunks, lambda t: grads[t])
+    view = torch.int32 if dtype == torch.float32 else torch.int16
+    for pc, want in zip(module.param_chunks, _expected_shards(module, grads, dtype)):
+        assert pc._stats_pending
+        assert torch.equal(pc.shard.view(view), want.view(view))
+        ref = oracle.l2norm_sq_ref(to_np(want)[:pc.n_valid], CODE[dtype])
+        assert pc.overflow is False
+        assert abs(pc.l2_norm - ref) <= 1e-6 * ref
+
+
+def test_land_tensors_flags_the_right_chunk(oracle):
+    from elixir_amd.chunk import land_tensors
+    dtype = torch.float16
+    module, opt, _ = build_workload(_odd(), 1 << 17, dtype, seed=4, loss_scale=1.0)
+    params = list(module.parameters())
+    for victim in (0, len(params) // 2, len(params) - 1):
+        grads = {p: _payload(p.numel(), dtype, 200 + i, scale=0.7).view(p.shape) for i, p in enumerate(params)}
+        grads[params[victim]].view(-1)[-1] = float('nan')
+        for pc in module.param_chunks:
+            pc.invalidate_stats()
+        land_tensors(module.param_chunks, lambda t: grads[t])
+        owner = module.fetcher.get_one_chunk(params[victim])
+        assert [pc.overflow for pc in module.param_chunks] == [pc is owner for pc in module.param_chunks]
+
+
+def test_land_tensors_then_step_equals_payload_landing_then_step(oracle):
+    from elixir_amd.chunk import land_tensors
+    dtype = torch.float16
+    runs = []
+    for per_tensor in (False, True):
+        module, opt, _ = build_workload(_odd(), 1 << 17, dtype, seed=5, loss_scale=256.0, initial_scale=256.0)
+        params = list(module.parameters())
+        grads = {p: _payload(p.numel(), dtype, 300 + i, scale=0.2).view(p.shape) for i, p in enumerate(params)}
+        if per_tensor:
+            land_tensors(module.param_chunks, lambda t: grads[t])
+        else:
+            land_chunks(module.param_chunks, _expected_shards(module, grads, dtype))
+        opt.mark_gradients_scaled()
+        opt.kernel_events = {}
+        opt.step()
+        assert 'stats' not in opt.kernel_events and opt.last_step_info['found_inf'] is False
+        runs.append([(pc.paired_chunk.shard.clone(), pc.shard.clone()) for pc in module.param_chunks])
+    for a, b in zip(*runs):
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_full_size_per_tensor_landing_c5():
+    """LLaMA-7B: 291 gradients (views of the saved buffers stand in for the .grad tensors) land in
+    27 chunks with one launch; shards, flags and norm as after the payload landing."""
+    from elixir_amd.chunk import land_tensors
+    built = workloads.build('c5', seed=78)
+    opt, module = built.optimizer, built.module
+    grads = {}
+    for pc, g in zip(module.param_chunks, built.grads):
+        g[pc.utilized_size:] = 0
+        for t, info in pc.tensors_info.items():
+            grads[t] = g[info.offset:info.end]
+    built.land_gradients(fused=True)
+    want = [(pc.overflow, pc.l2_norm) for pc in module.param_chunks]
+    for pc in module.param_chunks:
+        pc.shard.fill_(1.0)
+        pc.invalidate_stats()
+    land_tensors(module.param_chunks, lambda t: grads[t])
+    for pc, g, (ovf, l2) in zip(module.param_chunks, built.grads, want):
+        assert torch.equal(pc.shard.view(torch.int16), g.view(torch.int16))
+        assert pc.overflow is ovf is False
+        assert abs(pc.l2_norm - l2) <= 1e-6 * l2
+    opt.mark_gradients_scaled()
+    opt.kernel_events = {}
+    opt.step()
+    assert 'stats' not in opt.kernel_events and opt.last_step_info['found_inf'] is False

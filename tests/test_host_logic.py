@@ -338,3 +338,30 @@ def test_launch_plan_keeps_rows_bounded_for_the_large_workloads():
     assert padding == int(plan.refresh_rows['n_alloc'].sum()) and padding > 0
     # few workgroups of the 2-D grid find no work
     assert plan.info.max_tiles * len(plan.rows) - plan.info.total_tiles < 0.01 * plan.info.total_tiles
+
+
+def test_land_rows_tile_every_piece_exactly():
+    from elixir_amd.chunk import land_rows, _land_block_elems
+    block = 4096
+    pieces = [(0, 1 << 30, 1 << 40, 10000), (0, 0, (1 << 40) + 20000, 5000), (1, 1 << 31, 1 << 41, 4096),
+              (2, 1 << 32, 1 << 42, 1), (2, 0, (1 << 42) + 2, 8193)]
+    rows, offsets = land_rows(pieces, 3, block, ssize=4, dsize=2)
+    assert offsets.tolist() == [0, 3 + 2, 3 + 2 + 1, 3 + 2 + 1 + 1 + 3]
+    k = 0
+    for slot, src, dst, count in pieces:
+        left = count
+        done = 0
+        while left > 0:
+            r = rows[k]
+            n = min(block, left)
+            assert r['n_alloc'] == n and r['n_valid'] == (n if src else 0)
+            assert r['grad'] == (src + 4 * done if src else 0) and r['lowp_out'] == dst + 2 * done
+            assert offsets[slot] <= k < offsets[slot + 1]
+            done += n
+            left -= n
+            k += 1
+    assert k == len(rows)
+    # block choice: a power of two of at least 16 tiles that keeps a 7.2 G element set below 32 Ki rows
+    assert _land_block_elems(1000, 2048) == 16 * 2048
+    b = _land_block_elems(7_247_757_312, 2048)
+    assert b & (b - 1) == 0 and 7_247_757_312 // b < 16384 <= 7_247_757_312 // (b // 2)
