@@ -538,6 +538,24 @@ class Chunk:
     def get_tensors(self) -> List[torch.Tensor]:
         return list(self.tensors_info.keys())
 
+    def get_cpu_copy(self, only_rank_0: bool = False) -> List[torch.Tensor]:
+        """chunk.py:426-447 on one process: a CPU copy of every tensor of the chunk, in order,
+        shaped like the tensor."""
+        assert not self.is_init
+        return [self.shard[info.offset:info.end].view(info.fake_data.shape if info.fake_data is not None else t.shape)
+                .cpu() for t, info in self.tensors_info.items()]
+
+    def load_tensors(self, tensor_list: List[Optional[torch.Tensor]], only_rank_0: bool = False) -> None:
+        """chunk.py:449-473 on one process: values for the tensors of the chunk, in order (None =
+        keep), written into the shard."""
+        assert not self.is_init
+        assert len(tensor_list) == len(self.tensors_info)
+        for info, load_tensor in zip(self.tensors_info.values(), tensor_list):
+            if load_tensor is None:
+                continue
+            self.shard[info.offset:info.end].copy_(load_tensor.data.flatten())
+        self.invalidate_stats()
+
     # ------------------------------------------------------------------ gradient landing and flags
 
     def _stats_row(self) -> np.ndarray:

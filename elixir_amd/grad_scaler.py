@@ -117,9 +117,13 @@ class DynamicGradScaler(BaseGradScaler):
             self._scale = min(self._scale, self._max_scale)
 
     def state_dict(self) -> Dict:
+        """The scale, the factors and the hysteresis as the scaler this class mirrors saves them, and
+        what a resumed run needs besides: both counters, the growth interval and the clamps."""
         return dict(scale=self.scale, growth_factor=self._growth_factor, backoff_factor=self._backoff_factor,
                     hysteresis=self._hysteresis, growth_step=self._growth_step,
-                    hysteresis_step=self._hysteresis_step)
+                    hysteresis_step=self._hysteresis_step, growth_interval=self._growth_interval,
+                    min_scale=None if self._min_scale is None else float(self._min_scale),
+                    max_scale=None if self._max_scale is None else float(self._max_scale))
 
     def load_state_dict(self, state_dict: Dict) -> None:
         self._scale = np.float32(float(state_dict['scale']))
@@ -128,3 +132,8 @@ class DynamicGradScaler(BaseGradScaler):
         self._hysteresis = state_dict['hysteresis']
         self._growth_step = state_dict.get('growth_step', 0)
         self._hysteresis_step = state_dict.get('hysteresis_step', 0)
+        self._growth_interval = state_dict.get('growth_interval', self._growth_interval)
+        if 'min_scale' in state_dict:
+            self._min_scale = None if state_dict['min_scale'] is None else np.float32(state_dict['min_scale'])
+        if 'max_scale' in state_dict:
+            self._max_scale = None if state_dict['max_scale'] is None else np.float32(state_dict['max_scale'])

@@ -288,6 +288,61 @@ class HybridAdam(torch.optim.Optimizer):
 
     # ---- bound to chunk storage
 
+    # ---- checkpoint of the optimizer state
+
+    def _ensure_state(self) -> None:
+        """Bound fake parameters get their (step, exp_avg, exp_avg_sq) entries -- views of the flat
+        per-chunk moments -- before the first step, so that a fresh optimizer can save or load."""
+        if self._binding is not None:
+            self._walk_bound()
+
+    def state_dict(self):
+        """torch's packed layout (``state`` keyed by the running index of the parameter over the
+        groups, ``param_groups`` with those indices).  ``exp_avg`` / ``exp_avg_sq`` are CPU copies,
+        detached from the flat storage; with bound chunks they are the 1-D slices this process owns."""
+        self._ensure_state()
+        packed = super().state_dict()
+        # torch hands out the optimizer's own per-parameter dicts: build new ones, never edit those
+        packed['state'] = {
+            pid: {key: (value.detach().to('cpu', copy=True) if torch.is_tensor(value) else value)
+                  for key, value in st.items()}
+            for pid, st in packed['state'].items()
+        }
+        return packed
+
+    def load_state_dict(self, state_dict) -> None:
+        """Restores what ``state_dict`` saved, IN PLACE: the moments are copied into the flat
+        per-chunk buffers (or the existing per-parameter tensors) the update launch reads, never
+        replaced by new tensors; step counts and group hyper-parameters are taken over."""
+        self._ensure_state()
+        groups, saved_groups = self.param_groups, state_dict['param_groups']
+        if len(groups) != len(saved_groups) or any(
+                len(g['params']) != len(sg['params']) for g, sg in zip(groups, saved_groups)):
+            raise ValueError('loaded state dict has a different number of parameter groups or parameters')
+        id_to_param = {}
+        for g, sg in zip(groups, saved_groups):
+            for p, pid in zip(g['params'], sg['params']):
+                id_to_param[pid] = p
+            for key, value in sg.items():
+                if key != 'params':
+                    g[key] = value
+        for pid, saved in state_dict['state'].items():
+            p = id_to_param[int(pid)]
+            state = self.state[p]
+            for key in ('exp_avg', 'exp_avg_sq'):
+                if key not in saved:
+                    continue
+                if key not in state:    # a standalone parameter that has not stepped yet
+                    state[key] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                src = saved[key]
+                if src.numel() != state[key].numel():
+                    raise ValueError(f'parameter {pid}: saved {key} has {src.numel()} elements, '
+                                     f'this optimizer holds {state[key].numel()}')
+                state[key].copy_(src.reshape(state[key].shape))
+            step = saved.get('step', 0)
+            state['step'] = int(step.item()) if torch.is_tensor(step) else int(step)
+        self._prepared = None
+
     def _walk_bound(self):
         """(state dict, group index, chunk index, begin, end) per bound fake parameter, in group order."""
         b = self._binding

@@ -178,10 +178,21 @@ class ElixirOptimizer:
         return self.optim.add_param_group(*args, **kwargs)
 
     def state_dict(self):
-        return self.optim.state_dict()
+        """The inner optimizer's state in torch's packed layout (step, exp_avg, exp_avg_sq per fake
+        parameter -- the slice of each tensor this process owns -- and the group hyper-parameters),
+        plus the loss scaler under ``grad_scaler``.  The reference forwards to the inner optimizer
+        and loses the scaler; resuming a mixed-precision run needs both."""
+        packed = self.optim.state_dict()
+        packed['grad_scaler'] = self.grad_scaler.state_dict()
+        return packed
 
-    def load_state_dict(self, *args, **kwargs):
-        return self.optim.load_state_dict(*args, **kwargs)
+    def load_state_dict(self, state_dict, *args, **kwargs):
+        state_dict = dict(state_dict)
+        scaler_state = state_dict.pop('grad_scaler', None)
+        ret = self.optim.load_state_dict(state_dict, *args, **kwargs)
+        if scaler_state is not None:
+            self.grad_scaler.load_state_dict(scaler_state)
+        return ret
 
     # ------------------------------------------------------------------ set-up
 

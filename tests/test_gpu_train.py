@@ -126,3 +126,57 @@ def test_state_dict_round_trip_and_load():
     for k in new:
         assert torch.equal(back[k], new[k])
         assert torch.equal(module.state_dict(from_param=True)[k], new[k].bfloat16())
+
+
+def test_resume_from_checkpoint_is_bit_identical():
+    """Train, save weights + optimizer state + scaler, go on; a fresh module and optimizer that load
+    the checkpoint and see the same batches end with the same bits.  The save point sits right after
+    a skipped step with hysteresis 2, so the scaler's counters matter."""
+    torch.manual_seed(3)
+    base = Net().to(DEV)
+
+    def run(model, steps, gen, opt_pair=None, poison_at=()):
+        module, opt = opt_pair or wrap(model, torch.float16, initial_scale=512.0, hysteresis=2, growth_interval=3)
+        for step in steps:
+            x = batch(gen)
+            opt.zero_grad()
+            opt.backward(module(x))
+            if step in poison_at:
+                pc = module.param_chunks[-1]
+                pc.shard[pc.n_valid - 1] = float('-inf')
+                pc.invalidate_stats()
+            opt.step()
+            module.materialize_params()
+        return module, opt
+
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    module, opt = run(copy.deepcopy(base), range(0, 4), gen, poison_at=(3,))
+    assert opt.last_step_info['found_inf'] is True and opt.loss_scale == 1024.0    # grew at step 3 (0-2 clean), armed, not backed off
+    weights = module.state_dict()
+    ckpt = opt.state_dict()
+    gen_state = gen.get_state()
+    # the saved moments are copies: going on must not change them
+    frozen = {i: st['exp_avg'].clone() for i, st in ckpt['state'].items()}
+    module, opt = run(None, range(4, 9), gen, opt_pair=(module, opt), poison_at=(5,))
+    assert all(torch.equal(frozen[i], st['exp_avg']) for i, st in ckpt['state'].items())
+    # 3: armed; 4: clean; 5: second overflow of the window -> 512; 6-8: three clean steps -> 1024 again
+    assert opt.loss_scale == 1024.0 and opt.grad_scaler._growth_step == 0
+
+    gen2 = torch.Generator(device=DEV).manual_seed(0)
+    gen2.set_state(gen_state)
+    fresh_module, fresh_opt = wrap(copy.deepcopy(base), torch.float16, initial_scale=2.0, hysteresis=1)
+    fresh_module.load_state_dict(weights)
+    fresh_opt.load_state_dict(ckpt)
+    assert fresh_opt.loss_scale == 1024.0
+    fresh_module, fresh_opt = run(None, range(4, 9), gen2, opt_pair=(fresh_module, fresh_opt), poison_at=(5,))
+
+    assert fresh_opt.loss_scale == opt.loss_scale == 1024.0
+    for a, b in zip(module.param_chunks, fresh_module.param_chunks):
+        assert torch.equal(a.paired_chunk.shard, b.paired_chunk.shard) and torch.equal(a.shard, b.shard)
+        for x, y in zip(opt._binding.moments(a.paired_chunk), fresh_opt._binding.moments(b.paired_chunk)):
+            assert torch.equal(x, y)
+    sa, sb = opt.state_dict(), fresh_opt.state_dict()
+    assert [st['step'] for st in sa['state'].values()] == [st['step'] for st in sb['state'].values()] == [7] * len(
+        sa['state'])
+    assert sa['grad_scaler']['growth_step'] == sb['grad_scaler']['growth_step']
+    assert sa['grad_scaler']['hysteresis_step'] == sb['grad_scaler']['hysteresis_step']

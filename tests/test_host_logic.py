@@ -365,3 +365,80 @@ def test_land_rows_tile_every_piece_exactly():
     assert _land_block_elems(1000, 2048) == 16 * 2048
     b = _land_block_elems(7_247_757_312, 2048)
     assert b & (b - 1) == 0 and 7_247_757_312 // b < 16384 <= 7_247_757_312 // (b // 2)
+
+
+# ------------------------------------------------------------------------------------------------
+# checkpoint of the optimizer state (no GPU: host-resident shards can be saved and loaded, not stepped)
+# ------------------------------------------------------------------------------------------------
+
+
+def _cpu_optimizer(seed):
+    torch.manual_seed(seed)
+    net = TinyNet()
+    named = [(n, p.numel()) for n, p in net.named_parameters()]
+    module = ea.ElixirModule(net, ea.greedy_search(named, 1024, torch.float16, shard_device=torch.device('cpu')),
+                             dtype=torch.float16)
+    decay = [p for p in net.parameters() if p.dim() > 1]
+    exempt = [p for p in net.parameters() if p.dim() == 1]
+    inner = ea.HybridAdam([dict(params=decay, weight_decay=0.1), dict(params=exempt, weight_decay=0.0)], lr=1e-3)
+    return module, ea.ElixirOptimizer(module, inner, initial_scale=1024.0, hysteresis=2, growth_interval=7)
+
+
+def test_optimizer_state_dict_round_trip_keeps_flat_storage():
+    module, opt = _cpu_optimizer(0)
+    sd0 = opt.state_dict()
+    n_params = sum(len(g['params']) for g in opt.param_groups)
+    assert set(sd0) == {'state', 'param_groups', 'grad_scaler'} and len(sd0['state']) == n_params
+    assert all(st['step'] == 0 and st['exp_avg'].device.type == 'cpu' for st in sd0['state'].values())
+
+    # invent a state: moments, step counts, changed hyper-parameters, a scaler in mid-flight
+    gen = torch.Generator().manual_seed(1)
+    for i, st in sd0['state'].items():
+        st['exp_avg'] = torch.randn(st['exp_avg'].shape, generator=gen)
+        st['exp_avg_sq'] = torch.rand(st['exp_avg_sq'].shape, generator=gen)
+        st['step'] = 5 + i
+    sd0['param_groups'][0]['lr'] = 3e-4
+    sd0['param_groups'][1]['betas'] = (0.8, 0.95)
+    sd0['grad_scaler'].update(scale=torch.tensor([256.0]), growth_step=3, hysteresis_step=1)
+
+    flat_before = {c: (opt._binding.moments(c)[0].data_ptr(), opt._binding.moments(c)[1].data_ptr())
+                   for c in opt._binding.chunks}
+    opt.load_state_dict(sd0)
+    assert opt.loss_scale == 256.0 and opt.grad_scaler._growth_step == 3 and opt.grad_scaler._hysteresis_step == 1
+    assert opt.param_groups[0]['lr'] == 3e-4 and opt.param_groups[1]['betas'] == (0.8, 0.95)
+    sd1 = opt.state_dict()
+    for i, st in sd0['state'].items():
+        assert sd1['state'][i]['step'] == st['step']
+        assert torch.equal(sd1['state'][i]['exp_avg'], st['exp_avg'])
+        assert torch.equal(sd1['state'][i]['exp_avg_sq'], st['exp_avg_sq'])
+    # the values went INTO the flat per-chunk buffers: same storage, and the per-tensor views see them
+    for c, (pm, pv) in flat_before.items():
+        m, v = opt._binding.moments(c)
+        assert (m.data_ptr(), v.data_ptr()) == (pm, pv)
+    k = 0
+    for group in opt.param_groups:
+        for fake in group['params']:
+            chunk, (b, e) = opt.param_to_optim_chunk[fake], opt.param_to_range[fake]
+            assert torch.equal(opt._binding.moments(chunk)[0][b:e], sd0['state'][k]['exp_avg'])
+            k += 1
+
+    other_module, other = _cpu_optimizer(0)
+    bad = opt.state_dict()
+    bad['param_groups'][0]['params'] = bad['param_groups'][0]['params'][:-1]
+    with pytest.raises(ValueError):
+        other.load_state_dict(bad)
+
+
+def test_chunk_cpu_copy_and_load_tensors():
+    a, b = torch.randn(3, 5), torch.randn(7)
+    chunk = ea.Chunk(None, 32, torch.float, None, shard_device='cpu', temp_device='cpu')
+    chunk.append_tensor(a)
+    chunk.append_tensor(b)
+    chunk.close_chunk()
+    ca, cb = chunk.get_cpu_copy()
+    assert ca.shape == (3, 5) and cb.shape == (7,)
+    assert torch.equal(ca.flatten(), chunk.shard[:15]) and torch.equal(cb, chunk.shard[15:22])
+    new_b = torch.arange(7.0)
+    chunk.load_tensors([None, new_b])
+    assert torch.equal(chunk.shard[:15], ca.flatten()) and torch.equal(chunk.shard[15:22], new_b)
+    assert torch.count_nonzero(chunk.shard[22:]) == 0
