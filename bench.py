@@ -178,6 +178,52 @@ def fused_landing_leg(built, steps):
     }
 
 
+def offload_gather_leg(mi_elements):
+    """Source copy of the gather for ONE host-resident chunk of ``mi_elements`` Mi elements whose
+    refresh was deferred: the cast kernel reading the pinned fp32 shard in place, against the staged
+    form (fp32 shard to the GPU, then a cast copy).  Bound by the host link, not by HBM."""
+    import elixir_amd as ea
+    n = mi_elements << 20
+    p = ea.Chunk(None, n, torch.float16, None, shard_device='cpu', temp_device='cpu', cpu_pin_memory=True)
+    o = ea.Chunk(None, n, torch.float32, None, shard_device='cpu', temp_device='cpu', cpu_pin_memory=True)
+    t = torch.empty(n, dtype=torch.float32).normal_(0, 0.02)
+    p.append_tensor(t.half())
+    o.append_tensor(t)
+    p.close_chunk()
+    o.close_chunk()
+    p.init_pair(o)
+    block = torch.empty(n, dtype=torch.float16, device='cuda')
+
+    def timed(fn):
+        b, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        b.record()
+        fn()
+        e.record()
+        e.synchronize()
+        return b.elapsed_time(e) * 1e-3
+
+    def fused():
+        p.optim_sync_flag = False
+        p.replicate(block)
+
+    def staged():
+        block.copy_(o.shard.to('cuda', non_blocking=True))
+
+    fused_s = [timed(fused) for _ in range(4)][1:]
+    ok = torch.equal(block.cpu(), o.shard.half())
+    staged_s = [timed(staged) for _ in range(4)][1:]
+    return {
+        'what': 'gather source copy of one host-resident chunk, deferred refresh fused in',
+        'elements': n,
+        'fused_ms': float(np.mean(fused_s)) * 1e3,
+        'fused_host_link_gbps': 4 * n / float(np.mean(fused_s)) / 1e9,
+        'staged_ms': float(np.mean(staged_s)) * 1e3,
+        'staged_extra_device_bytes': 4 * n,
+        'matches_cast_of_master': bool(ok),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -193,6 +239,8 @@ def main():
     ap.add_argument('--landing-steps', type=int, default=5,
                     help='steps of the additional leg in which the gradients arrive through the fused landing '
                     'launch (0: skip the leg)')
+    ap.add_argument('--offload-gather', type=int, default=0, metavar='MI',
+                    help='only time the gather source copy of one host-resident chunk of MI Mi elements and exit')
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -202,6 +250,10 @@ def main():
     if not torch.cuda.is_available():
         print('bench.py needs a GPU: the optimizer step has no CPU path', file=sys.stderr)
         sys.exit(2)
+
+    if args.offload_gather > 0:
+        print(json.dumps(offload_gather_leg(args.offload_gather)))
+        return
 
     if args.calibrate_copy > 0:
         n = int(args.calibrate_copy * (1 << 30)) // 4

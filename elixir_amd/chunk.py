@@ -649,6 +649,54 @@ class Chunk:
         else:
             raise NotImplementedError
 
+    # ------------------------------------------------------------------ gather source / release
+
+    def _refresh_into(self, dst: torch.Tensor, master: torch.Tensor) -> None:
+        """dst (device, this chunk's dtype) = round-to-nearest-even(master); ``master`` is device
+        memory or pinned host memory, which the kernel reads in place over the host link."""
+        assert dst.is_cuda and dst.is_contiguous() and dst.numel() == master.numel() == self.shard_size
+        assert master.dtype == torch.float32 and master.is_contiguous()
+        assert master.is_cuda or master.is_pinned(), 'the kernel can only read device or pinned host memory'
+        row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+        row['lowp_out'] = dst.data_ptr()
+        row['master'] = row['m'] = row['v'] = master.data_ptr()
+        row['n_alloc'] = self.shard_size
+        row['n_valid'] = self.n_valid
+        code = dtype_code(self.chunk_dtype)
+        info = _abi.check_tables(row, None, 0, code, code)
+        table = DeviceTable(row, dst.device)
+        _abi.writeback_mt(table.ptr, 1, code, self.shard_size, info.aligned, torch.cuda.current_stream(dst.device).cuda_stream)
+        self._workspace['gather_table'] = table    # alive until the launch has consumed it
+
+    def replicate(self, payload: torch.Tensor) -> None:
+        """chunk.py:264-270 + 475-482 on one process: fills this shard's slice of a replicated block
+        (``chunk_size`` elements on the GPU) -- the source copy of the gather.  A shard that is in
+        sync with its optimizer chunk is copied (a transfer when it lives on the host).  One whose
+        refresh was deferred (``optim_sync_flag`` False: host-resident shards after an update) is
+        produced from the fp32 optimizer shard in ONE pass: the cast kernel reads pinned host memory
+        in place and writes the low-precision slice, without the fp32 staging copy on the GPU that
+        ``optim_chunk.shard.to(gpu)`` + ``copy_`` would make.  An unpinned host shard is staged."""
+        assert not self.is_init
+        assert payload.is_cuda and payload.numel() == self.chunk_size and payload.dtype == self.chunk_dtype
+        dst = payload[self.shard_begin:self.shard_end]
+        if self.optim_sync_flag:
+            dst.copy_(self.shard)
+            return
+        assert self.paired_chunk is not None, 'chunks should be paired before training'
+        master = self.paired_chunk.shard
+        if not (master.is_cuda or master.is_pinned()):
+            master = master.to(payload.device)
+        self._refresh_into(dst, master)
+
+    def scatter(self, payload: torch.Tensor) -> None:
+        """chunk.py:273-281 on one process: the block is released; a shard whose refresh was
+        deferred takes the refreshed values from the block and is in sync again."""
+        assert not self.is_init
+        assert payload.numel() == self.chunk_size and payload.dtype == self.chunk_dtype
+        if not self.optim_sync_flag:
+            self.shard.copy_(payload[self.shard_begin:self.shard_end])
+            self.optim_sync_flag = True
+
     # ------------------------------------------------------------------ misc
 
     def __hash__(self) -> int:

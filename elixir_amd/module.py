@@ -201,10 +201,20 @@ class ElixirModule(nn.Module):
         """Give every parameter of the wrapped module a private copy of its low-precision values
         (what a gather into the replicated cache would expose to the forward pass)."""
         assert not self.synthetic
+        blocks = {}
+        for chunk in self.param_chunks:
+            if not chunk.optim_sync_flag and torch.cuda.is_available():
+                # a host-resident shard whose refresh was deferred: gather source copy with the cast
+                # fused in, then the release brings the shard back in sync (chunk.py:264-281)
+                block = torch.empty(chunk.chunk_size, dtype=chunk.chunk_dtype, device=gpu_device())
+                chunk.replicate(block)
+                chunk.scatter(block)
+                blocks[chunk] = block
         for param in self.grad_state_dict.values():
             chunk = self.param_chunk_group.ten_to_chunk[param]
             info = chunk.tensors_info[param]
-            param.data = chunk.shard[info.offset:info.end].clone().view(info.fake_data.shape)
+            src = blocks.get(chunk, chunk.shard)
+            param.data = src[info.offset:info.end].clone().view(info.fake_data.shape)
 
     def forward(self, *args, **kwargs):
         assert not self.synthetic

@@ -1,0 +1,101 @@
+"""Host-resident shards: the deferred low-precision refresh fused into the source copy of the gather
+(elixir/chunk/core/chunk.py:264-281, 403-421, 475-499).  After an update of a host-resident
+optimizer chunk the parameter chunk is only marked out of sync; the next ``replicate`` produces the
+low-precision slice of the block straight from the fp32 shard (the cast kernel reads pinned host
+memory in place), and ``scatter`` brings the host shard back in sync.
+
+Bar: the block equals the oracle's cast of the fp32 shard bit for bit (= torch's ``.to()``)."""
+import numpy as np
+import pytest
+import torch
+
+import elixir_amd as ea
+from oracle import oracle as O
+
+from helpers import CODE, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def _pair(dtype, sizes, chunk_size, pinned):
+    p = ea.Chunk(None, chunk_size, dtype, None, shard_device='cpu', temp_device='cpu', cpu_pin_memory=pinned)
+    o = ea.Chunk(None, chunk_size, torch.float32, None, shard_device='cpu', temp_device='cpu', cpu_pin_memory=pinned)
+    g = torch.Generator().manual_seed(sum(sizes))
+    for n in sizes:
+        t = torch.randn(n, generator=g) * 0.05
+        p.append_tensor(t.to(dtype))
+        o.append_tensor(t.clone())
+    p.close_chunk()
+    o.close_chunk()
+    p.init_pair(o)
+    assert p.shard.is_pinned() is pinned and o.shard.is_pinned() is pinned
+    return p, o
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('pinned', [True, False])
+def test_deferred_refresh_rides_the_gather_source_copy(oracle, dtype, pinned):
+    sizes = [4097, 3, 15000, 1, 8191, 70001]
+    p, o = _pair(dtype, sizes, 1 << 17, pinned)
+    old = p.shard.clone()
+    # an update of the host-resident master (what a step or a state load leaves behind)
+    g = torch.Generator().manual_seed(1)
+    o.shard[:sum(sizes)] = torch.randn(sum(sizes), generator=g) * 0.3
+    o.shard[:6] = torch.tensor([0.0, -0.0, 65504.0, 65520.0, 1e-8, -3.0e38])
+    p.optim_update()
+    assert p.optim_sync_flag is False and torch.equal(p.shard, old)       # deferred: nothing moved yet
+
+    block = torch.full((p.chunk_size,), 9.0, dtype=dtype, device=DEV)
+    p.replicate(block)
+    want = oracle.writeback(o.shard.numpy().copy(), CODE[dtype])
+    assert np.array_equal(to_np(block), want)
+    assert torch.equal(block.cpu(), o.shard.to(dtype))
+    assert torch.equal(p.shard, old) and p.optim_sync_flag is False       # the host shard is refreshed on release
+
+    p.scatter(block)
+    assert p.optim_sync_flag is True
+    assert torch.equal(p.shard, o.shard.to(dtype))
+
+    # in sync again: the next gather is a plain transfer of the low-precision shard
+    o.shard.add_(1.0)                                                     # must NOT show up
+    block2 = torch.zeros(p.chunk_size, dtype=dtype, device=DEV)
+    p.replicate(block2)
+    assert torch.equal(block2, block)
+
+
+def test_device_resident_chunks_gather_by_copy(oracle):
+    named = [('w', (300, 40)), ('b', (40,))]
+    sr = ea.greedy_search([(n, int(np.prod(s))) for n, s in named], 16384, torch.float16)
+    module = ea.ElixirModule(dict(named), sr, dtype=torch.float16)
+    pc = module.param_chunks[0]
+    pc.paired_chunk.shard.normal_(0, 0.1)
+    pc.optim_update()
+    assert pc.optim_sync_flag is True
+    block = torch.zeros(pc.chunk_size, dtype=torch.float16, device=DEV)
+    pc.replicate(block)
+    assert torch.equal(block, pc.paired_chunk.shard.half())
+    pc.scatter(block)
+
+
+def test_load_state_dict_into_host_resident_chunks():
+    """module.py:294-344 with an offload placement: values go into the fp32 host shards, the refresh
+    is deferred, and the parameters the forward pass sees come from the fused gather copy."""
+    torch.manual_seed(0)
+    net = torch.nn.Sequential(torch.nn.Linear(24, 48), torch.nn.LayerNorm(48), torch.nn.Linear(48, 10))
+    named = [(n, p.numel()) for n, p in net.named_parameters()]
+    sr = ea.greedy_search(named, 2048, torch.float16, shard_device=torch.device('cpu'))
+    for plan in sr.param_chunk_plans:
+        plan.kwargs['cpu_pin_memory'] = True
+    module = ea.ElixirModule(net, sr, dtype=torch.float16)
+    assert all(pc.shard_device.type == 'cpu' and pc.shard.is_pinned() for pc in module.param_chunks)
+    new = {n: torch.randn_like(p, dtype=torch.float32) * 0.2 for n, p in net.named_parameters()}
+    module.load_state_dict(new)
+    assert all(pc.optim_sync_flag for pc in module.param_chunks)          # released after the gather
+    for n, p in net.named_parameters():
+        assert p.is_cuda and torch.equal(p.data.cpu(), new[n].half()), n
+    sd = module.state_dict()
+    for n in new:
+        assert torch.equal(sd[n], new[n])
+    for pc in module.param_chunks:
+        assert torch.equal(pc.shard, pc.paired_chunk.shard.half())
