@@ -33,7 +33,7 @@ BYTES_STATS = 2                 # per valid element: the compulsory second read 
 MEASURED_TRAFFIC_BYTES = {'c5': 188.775e9}
 
 
-def cpu_baseline(built, sample_elems: int, steps: int = 3):
+def cpu_baseline(built, sample_elems: int, steps: int = 8):
     """The same step as torch CPU ops (the oracle's torch harness) on a bounded sample: the first
     `sample_elems` elements of chunk 0.  Returns the cpu_baseline object of the JSON line."""
     from oracle import oracle as O
@@ -230,7 +230,7 @@ def main():
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--workload', default='c5', choices=['c2', 'c4', 'c5'])
-    ap.add_argument('--cpu-sample', type=int, default=32 << 20, help='elements of the CPU baseline sample; 0 skips it')
+    ap.add_argument('--cpu-sample', type=int, default=128 << 20, help='elements of the CPU baseline sample; 0 skips it')
     ap.add_argument('--blocks-per-cu', type=int, default=0,
                     help='cap on resident update workgroups per compute unit (0 = library default)')
     ap.add_argument('--calibrate-copy', type=float, default=0.0,

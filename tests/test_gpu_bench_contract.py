@@ -1,0 +1,34 @@
+"""bench.py prints one JSON line with the agreed fields (run on the small GPT-2 chunk set)."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_bench_json_line():
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--workload', 'c2', '--steps', '3',
+                           '--warmup', '1', '--cpu-sample', str(1 << 20), '--landing-steps', '2'],
+                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=280)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [l for l in proc.stdout.splitlines() if l.startswith('{')]
+    assert len(lines) == 1
+    out = json.loads(lines[0])
+    for key in ('metric', 'value', 'unit', 'n_gpus', 'steps', 'warmup', 'ms_per_step', 'higher_is_better', 'scaling',
+                'vs_baseline', 'dtype', 'data', 'config', 'roofline', 'cpu_baseline'):
+        assert key in out, key
+    assert out['n_gpus'] == 1 and out['steps'] == 3 and out['warmup'] == 1 and out['vs_baseline'] is None
+    assert out['config']['workload'].startswith('c2') and out['config']['valid_elements'] == 124_439_808
+    assert abs(out['value'] - out['config']['valid_elements'] / (out['ms_per_step'] * 1e-3)) <= 1e-6 * out['value']
+    r = out['roofline']
+    assert r['bound'] == 'hbm' and r['peak'] == 8000.0 and r['unit'] == 'GB/s'
+    assert abs(r['frac'] - r['achieved'] / r['peak']) < 1e-12 and 0 < r['frac'] < 1
+    assert abs(r['achieved'] - r['bytes_per_launch'] / (r['ms_per_launch'] * 1e-3) / 1e9) <= 1e-6 * r['achieved']
+    assert r['bytes_per_launch'] == 28 * out['config']['valid_elements']
+    c = out['cpu_baseline']
+    assert c['kind'] == 'port' and c['cores'] >= 1 and c['value'] > 0 and c['unit'] == 'elements/s'
+    assert out['fused_landing']['ms_per_step'] > 0
