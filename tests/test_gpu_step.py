@@ -487,3 +487,45 @@ def test_abi_rejects_bad_tables():
     bad = row.copy(); bad['seg_end'] = 2; expect(-5, chunk=bad, segs=two)
     bad = row.copy(); bad['tile_begin'] = 1; expect(-6, chunk=bad)
     bad = row.copy(); bad['n_alloc'] = 0; bad['n_valid'] = 0; expect(-7, chunk=bad, segs=None)
+
+
+# ------------------------------------------------------------------------------------------------
+# seeded random layouts: tensor counts, sizes, chunk sizes, dtypes, modes
+# ------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize('seed', list(range(16)))
+def test_random_layouts_match_oracle(oracle, seed):
+    """Whatever the packing looks like -- boundaries inside vectors, tensors of one element, chunks
+    that are not a multiple of the tile, a padded tail or none -- an unclipped step is bit-identical
+    to the oracle's, over two steps (the second with new gradients and warm state)."""
+    rng = np.random.default_rng(1000 + seed)
+    n_tensors = int(rng.integers(1, 24))
+    kinds = rng.integers(0, 4, n_tensors)
+    sizes = [int({0: rng.integers(1, 9), 1: rng.integers(9, 700), 2: rng.integers(700, 9000),
+                  3: rng.integers(9000, 60000)}[int(k)]) for k in kinds]
+    named = [(f't{i}.{"weight" if rng.random() < 0.7 else "bias"}', (n,)) for i, n in enumerate(sizes)]
+    chunk_size = int(max(sizes) + rng.integers(0, 40000))
+    dtype = [torch.float16, torch.bfloat16, torch.float32][seed % 3]
+    loss_scale = float(2.0**rng.integers(0, 12)) if dtype == torch.float16 else 1.0
+    adamw = bool(rng.random() < 0.6)
+    betas = (0.9, 0.999) if rng.random() < 0.7 else (0.45, 0.98)
+    kw = dict(initial_scale=loss_scale, hysteresis=1) if dtype == torch.float16 else {}
+    module, opt, ochunks = build_workload(named, chunk_size, dtype, seed=seed, loss_scale=loss_scale, lr=3e-3,
+                                          betas=betas, weight_decay=float(rng.choice([0.0, 0.05])), adamw_mode=adamw,
+                                          **kw)
+    scaler = (O.DynamicGradScalerOracle(initial_scale=loss_scale, min_scale=1, max_scale=2**24, hysteresis=1)
+              if dtype == torch.float16 else O.ConstantGradScalerOracle(1.0))
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(seed)
+    for step in range(2):
+        if step:
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (2e-3 * loss_scale)
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+                pc.invalidate_stats()
+            refresh_oracle_grads(module, ochunks)
+        info = _run_and_compare(module, opt, ochunks, dtype, scaler, adamw_mode=adamw, tag=f'seed {seed} step {step}')
+        assert info['found_inf'] is False
+        assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'seed {seed} step {step}') == 0
