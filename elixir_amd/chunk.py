@@ -207,11 +207,14 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
     stream = torch.cuda.current_stream(device).cuda_stream
     _abi.land_grads_mt(cached.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
                        arena.ptr(chunks[0]._stats_slot), aligned, stream, LAND_BLOCKS_PER_CU)
+    landed = torch.cuda.Event()
+    landed.record(torch.cuda.current_stream(device))
     for c in chunks:
         c._overflow = False
         c._l2_norm = None
         c._stats_fresh = False
         c._stats_pending = True
+        c._stats_event = landed
 
 
 def _land_block_elems(total: int, tile: int) -> int:
@@ -313,11 +316,14 @@ def land_tensors(chunks: List['Chunk'], grad_of, mul: float = 1.0) -> None:
     _abi.land_grads_mt(table.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
                        arena.ptr(chunks[0]._stats_slot), True, stream, LAND_BLOCKS_PER_CU,
                        d_slot_offsets=offsets.data_ptr(), n_slots=len(chunks))
+    landed = torch.cuda.Event()
+    landed.record(torch.cuda.current_stream(device))
     for c in chunks:
         c._overflow = False
         c._l2_norm = None
         c._stats_fresh = False
         c._stats_pending = True
+        c._stats_event = landed
 
 
 def resolve_pending_stats(chunks: List['Chunk']) -> None:
@@ -328,12 +334,16 @@ def resolve_pending_stats(chunks: List['Chunk']) -> None:
         if c._stats_pending:
             by_device.setdefault(c.shard_device, []).append(c)
     for device, pending in by_device.items():
+        # the landing may have been enqueued on another stream than the one the copy below uses
+        for event in {c._stats_event for c in pending if c._stats_event is not None}:
+            torch.cuda.current_stream(device).wait_event(event)
         lo = min(c._stats_slot for c in pending)
         hi = max(c._stats_slot for c in pending) + 1
         records = StatsArena.get(device).read(lo, hi)
         for c in pending:
             rec = records[c._stats_slot - lo]
             c._stats_pending = False
+            c._stats_event = None
             c._apply_stats(bool(rec['overflow']), float(rec['sumsq']))
 
 
@@ -414,6 +424,7 @@ class Chunk:
         self._stats_fresh = False
         self._stats_slot: Optional[int] = None    # this chunk's record in the device arena
         self._stats_pending = False               # a landing launch has written it, nobody has read it
+        self._stats_event = None                  # recorded behind that launch, on its stream
         self._workspace: Dict = {}
 
     # ------------------------------------------------------------------ properties
@@ -445,6 +456,7 @@ class Chunk:
     def invalidate_stats(self) -> None:
         """The shard was written behind the chunk's back: forget flags and outstanding records."""
         self._stats_pending = False
+        self._stats_event = None
         self._stats_fresh = False
         self._overflow = False
         self._l2_norm = None

@@ -411,3 +411,24 @@ def test_full_size_per_tensor_landing_c5():
     opt.kernel_events = {}
     opt.step()
     assert 'stats' not in opt.kernel_events and opt.last_step_info['found_inf'] is False
+
+
+def test_landing_on_a_side_stream_is_waited_for(oracle):
+    """A landing enqueued on another stream: reading the flags from the default stream waits for it."""
+    dtype = torch.float16
+    module, opt, _ = build_workload(_tiny(), 16384, dtype, seed=8, loss_scale=1.0)
+    pc = module.param_chunks[0]
+    big = _payload(1 << 26, torch.float32, 1)          # something for the side stream to chew on first
+    side = torch.cuda.Stream()
+    pl = _payload(pc.chunk_size, dtype, 50, scale=0.3)
+    pl[pc.utilized_size:] = 0
+    pl[3] = float('inf')
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(8):
+            big.mul_(1.0001)
+        pc.invalidate_stats()
+        pc.reduce_chunk(pl, sync=False)
+    assert pc.overflow is True
+    side.synchronize()
+    assert torch.equal(pc.shard.view(torch.int16), pl.view(torch.int16))
