@@ -180,3 +180,42 @@ def test_resume_from_checkpoint_is_bit_identical():
         sa['state'])
     assert sa['grad_scaler']['growth_step'] == sb['grad_scaler']['growth_step']
     assert sa['grad_scaler']['hysteresis_step'] == sb['grad_scaler']['hysteresis_step']
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_clipped_training_matches_torchs_clip_grad_norm(dtype):
+    """Global L2 clipping end to end: the combined scale of optimizer.py:166-183 against
+    ``torch.nn.utils.clip_grad_norm_`` (coefficient max_norm / (norm + 1e-6), applied only above the
+    threshold) followed by torch's AdamW on fp32 master weights.  max_norm is small enough that
+    every step clips."""
+    torch.manual_seed(1)
+    master = Net().to(DEV)
+    model = copy.deepcopy(master)
+    ropt = torch.optim.AdamW(groups_of(master, 0.1), lr=1e-2, weight_decay=0.1)
+    module, opt = wrap(model, dtype, max_norm=0.05)
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    for step in range(4):
+        x = batch(gen)
+        if dtype == torch.float32:
+            work = master
+            ropt.zero_grad()
+            work(x).backward()
+        else:
+            work = copy.deepcopy(master).to(dtype)
+            work(x).backward()
+            for p, w in zip(master.parameters(), work.parameters()):
+                p.grad = w.grad.float()
+        norm = torch.nn.utils.clip_grad_norm_(master.parameters(), 0.05)
+        assert float(norm) > 0.05
+        ropt.step()
+        opt.zero_grad()
+        opt.backward(module(x))
+        opt.step()
+        info = opt.last_step_info
+        assert info['found_inf'] is False
+        assert abs(info['total_norm'] - float(norm)) <= 2e-6 * float(norm)
+        assert info['combined_scale'] > 1.0
+        module.materialize_params()
+        sd = module.state_dict()
+        for name, want in master.state_dict().items():
+            torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
