@@ -224,6 +224,58 @@ def offload_gather_leg(mi_elements):
     }
 
 
+def offload_step_leg(mi_elements, steps=5):
+    """The optimizer step over ONE host-resident chunk pair (fp16 shard, fp32 master, moments, all in
+    pinned host memory): the same launches read and write host memory in place, so the step is
+    bound by the host link (16 B in, 14 B out per element).  Next to it, torch's CPU ops on the
+    same data on this box's cores -- what a CPU Adam for offloaded shards costs."""
+    import elixir_amd as ea
+    from oracle.torch_ref import TorchCpuStep
+    n = mi_elements << 20
+    sr = ea.greedy_search([('w.weight', n)], n, torch.float16, shard_device=torch.device('cpu'))
+    sr.param_chunk_plans[0].kwargs['cpu_pin_memory'] = True
+    module = ea.ElixirModule({'w.weight': (n,)}, sr, dtype=torch.float16)
+    inner = ea.HybridAdam(list(module.parameters()), lr=1e-3, weight_decay=0.1)
+    opt = ea.ElixirOptimizer(module, inner, initial_scale=1024.0, hysteresis=1, max_norm=1.0)
+    pc = module.param_chunks[0]
+    oc = pc.paired_chunk
+    m, v = opt._binding.moments(oc)
+    oc.shard.normal_(0, 0.02)
+    m.normal_(0, 1e-4)
+    v.uniform_(0, 1e-6)
+    g = (torch.empty(n).normal_(0, 1e-3 * 1024.0)).half()
+    ref = TorchCpuStep(oc.shard.clone(), torch.float16, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.1,
+                       adamw_mode=True, exp_avg=m.clone(), exp_avg_sq=v.clone())
+    cpu_s = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ref.step(g, loss_scale=1024.0, max_norm=1.0)
+        cpu_s.append(time.perf_counter() - t0)
+    out = {}
+    for bpc in (0, 32):
+        opt.optim.blocks_per_cu = bpc
+        ts = []
+        for i in range(steps + 1):
+            pc.shard.copy_(g)
+            pc.invalidate_stats()
+            opt.mark_gradients_scaled()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            opt.step()
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+            assert opt.last_step_info['found_inf'] is False
+        t = float(np.mean(ts[1:]))
+        out['blocks_per_cu_%d' % (bpc or 12)] = {'ms_per_step': t * 1e3, 'elements_per_sec': n / t,
+                                                  'host_link_gbps_30B': 30 * n / t / 1e9}
+    tc = float(np.median(cpu_s[1:]))
+    out.update({'what': 'optimizer step over one host-resident (pinned) chunk pair, in place over the host link',
+                'elements': n,
+                'torch_cpu_same_box': {'ms_per_step': tc * 1e3, 'elements_per_sec': n / tc,
+                                       'cores': torch.get_num_threads()}})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -239,6 +291,8 @@ def main():
     ap.add_argument('--landing-steps', type=int, default=5,
                     help='steps of the additional leg in which the gradients arrive through the fused landing '
                     'launch (0: skip the leg)')
+    ap.add_argument('--offload-step', type=int, default=0, metavar='MI',
+                    help='only time the step over one host-resident chunk pair of MI Mi elements and exit')
     ap.add_argument('--offload-gather', type=int, default=0, metavar='MI',
                     help='only time the gather source copy of one host-resident chunk of MI Mi elements and exit')
     args = ap.parse_args()
@@ -251,6 +305,9 @@ def main():
         print('bench.py needs a GPU: the optimizer step has no CPU path', file=sys.stderr)
         sys.exit(2)
 
+    if args.offload_step > 0:
+        print(json.dumps(offload_step_leg(args.offload_step)))
+        return
     if args.offload_gather > 0:
         print(json.dumps(offload_gather_leg(args.offload_gather)))
         return

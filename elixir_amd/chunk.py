@@ -48,6 +48,19 @@ def gpu_device() -> torch.device:
     return torch.device('cuda', torch.cuda.current_device())
 
 
+def kernel_device(tensors) -> torch.device:
+    """The GPU whose kernels will touch these buffers.  Each must be device memory or pinned host
+    memory (read and written in place over the host link); pageable host memory is refused."""
+    device = None
+    for t in tensors:
+        if t.is_cuda:
+            device = device or t.device
+        elif not (torch.cuda.is_available() and t.is_pinned()):
+            raise RuntimeError('the HIP kernels reach device memory and pinned host memory only: this shard lives in '
+                               'pageable host memory (allocate it with cpu_pin_memory=True) or there is no GPU')
+    return device or gpu_device()
+
+
 def dtype_code(dtype: torch.dtype) -> int:
     try:
         return {torch.float32: _abi.ELX_F32, torch.float16: _abi.ELX_F16, torch.bfloat16: _abi.ELX_BF16}[dtype]
@@ -587,9 +600,7 @@ class Chunk:
         self._compute_stats()
 
     def _compute_stats(self) -> None:
-        if self.shard_device.type != 'cuda':
-            raise RuntimeError('gradient flags are computed by the HIP kernels: the shard must be on the GPU')
-        stats = run_grad_stats(self._stats_row(), dtype_code(self.chunk_dtype), self.shard_device,
+        stats = run_grad_stats(self._stats_row(), dtype_code(self.chunk_dtype), kernel_device([self.shard]),
                                workspace=self._workspace)
         self._apply_stats(bool(stats['overflow'][0]), float(stats['sumsq'][0]))
 

@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from . import _abi
-from .chunk import Chunk, DeviceTable, dtype_code
+from .chunk import gpu_device, Chunk, DeviceTable, dtype_code
 from .launch_plan import FlatBuffer, LaunchPlan, build_plan
 
 
@@ -128,15 +128,33 @@ class ChunkBinding:
             assert c.paired_chunk.shard_device == c.shard_device
 
     def require_gpu(self) -> None:
+        """Every buffer of the launch must be reachable by the kernels: device memory, or pinned
+        host memory (which they read and write in place over the host link)."""
+        if not torch.cuda.is_available():
+            raise RuntimeError('HybridAdam runs on the GPU: no device is available')
         for c in self.chunks:
-            if c.shard_device.type != 'cuda':
-                raise RuntimeError('HybridAdam runs on the GPU: optimizer shards must live in device memory '
-                                   '(host-resident shards are not supported by this build)')
+            for shard in (c.shard, c.paired_chunk.shard):
+                if not (shard.is_cuda or shard.is_pinned()):
+                    raise RuntimeError('HybridAdam runs on the GPU: shards must live in device memory or in '
+                                       'pinned host memory (cpu_pin_memory=True); pageable host memory cannot be '
+                                       'reached by the kernels')
+
+    def launch_device(self) -> torch.device:
+        for c in self.chunks:
+            if c.shard.is_cuda:
+                return c.shard_device
+        return gpu_device()
 
     def moments(self, chunk: Chunk) -> Tuple[torch.Tensor, torch.Tensor]:
+        """The flat exp_avg / exp_avg_sq of an optimizer chunk, allocated beside its shard: in device
+        memory, or in pinned host memory for a host-resident shard."""
         if chunk not in self.flat_m:
-            self.flat_m[chunk] = torch.zeros(chunk.shard_size, dtype=torch.float32, device=chunk.shard_device)
-            self.flat_v[chunk] = torch.zeros(chunk.shard_size, dtype=torch.float32, device=chunk.shard_device)
+            if chunk.shard.is_cuda or not torch.cuda.is_available():
+                kw = dict(device=chunk.shard_device)
+            else:
+                kw = dict(pin_memory=True)
+            self.flat_m[chunk] = torch.zeros(chunk.shard_size, dtype=torch.float32, **kw)
+            self.flat_v[chunk] = torch.zeros(chunk.shard_size, dtype=torch.float32, **kw)
         return self.flat_m[chunk], self.flat_v[chunk]
 
 
@@ -378,7 +396,7 @@ class HybridAdam(torch.optim.Optimizer):
         lowp_dtype = b.chunks[0].paired_chunk.chunk_dtype
         grad_code = dtype_code(lowp_dtype)
         lowp_code = _abi.ELX_NONE if b.zero_grads else grad_code
-        device = b.chunks[0].shard_device
+        device = b.launch_device()
         shard_ptrs = tuple(c.paired_chunk.shard.data_ptr() for c in b.chunks)
         key = ('bound', b.zero_grads, tuple(idx_of), shard_ptrs, tuple(c.shard.data_ptr() for c in b.chunks))
 

@@ -29,7 +29,8 @@ import torch
 from torch.nn import Parameter
 
 from . import _abi
-from .chunk import Chunk, DeviceTable, dtype_code, launch_grad_stats, read_grad_stats, resolve_pending_stats
+from .chunk import (Chunk, DeviceTable, dtype_code, kernel_device, launch_grad_stats, read_grad_stats,
+                    resolve_pending_stats)
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
 from .hybrid_adam import HybridAdam
 
@@ -325,9 +326,7 @@ class ElixirOptimizer:
         pending = [c for c in self._param_chunk_list if not c._stats_fresh and not c._stats_pending]
         if not pending:
             return None
-        device = pending[0].shard_device
-        if device.type != 'cuda':
-            raise RuntimeError('gradient flags are computed by the HIP kernels: shards must be on the GPU')
+        device = kernel_device(c.shard for c in pending)
         ids = tuple(c.chunk_id for c in pending)
         if self._stats_table is None or self._stats_table[0] != ids:
             rows = np.zeros(len(pending), dtype=_abi.CHUNK_DTYPE)

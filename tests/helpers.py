@@ -48,12 +48,18 @@ def assert_close_f32(got: np.ndarray, want: np.ndarray, name: str, rtol: float =
 
 def build_workload(named_shapes, chunk_size, dtype, *, seed=0, grad_std=1e-3, loss_scale=1.0, lr=1e-3,
                    betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, adamw_mode=True, decay_exempt=True,
-                   warm_state=True, device='cuda', **opt_kwargs):
+                   warm_state=True, device='cuda', host_resident=False, **opt_kwargs):
     """A synthetic chunk set on the GPU with seeded contents, its ElixirOptimizer, and the oracle's
     copy of the same data.  Gradients (already multiplied by ``loss_scale``) sit in the
     low-precision shards, as they do after backward."""
     named_shapes = list(named_shapes)
-    sr = ea.greedy_search([(n, S.numel(s)) for n, s in named_shapes], chunk_size, dtype)
+    if host_resident:    # shards (and with them the moments) in pinned host memory
+        sr = ea.greedy_search([(n, S.numel(s)) for n, s in named_shapes], chunk_size, dtype,
+                              shard_device=torch.device('cpu'))
+        for plan in sr.param_chunk_plans:
+            plan.kwargs['cpu_pin_memory'] = True
+    else:
+        sr = ea.greedy_search([(n, S.numel(s)) for n, s in named_shapes], chunk_size, dtype)
     module = ea.ElixirModule(dict(named_shapes), sr, dtype=dtype)
     decay, exempt = [], []
     for (name, shape), p in zip(named_shapes, module.parameters()):

@@ -99,3 +99,77 @@ def test_load_state_dict_into_host_resident_chunks():
         assert torch.equal(sd[n], new[n])
     for pc in module.param_chunks:
         assert torch.equal(pc.shard, pc.paired_chunk.shard.half())
+
+
+# ------------------------------------------------------------------------------------------------
+# the step over host-resident shards: the same launches, reading and writing pinned host memory
+# ------------------------------------------------------------------------------------------------
+
+
+def _tiny_named():
+    return [('wte.weight', (500, 48)), ('h.ln.weight', (48,)), ('h.ln.bias', (48,)), ('h.fc.weight', (48, 192)),
+            ('h.fc.bias', (192,)), ('h.proj.weight', (192, 48)), ('odd', (4097,)), ('lnf.weight', (48,))]
+
+
+@pytest.mark.parametrize('dtype,loss_scale,max_norm', [(torch.float16, 128.0, 0.0), (torch.bfloat16, 1.0, 1.0)])
+def test_step_over_pinned_host_shards_matches_oracle(oracle, dtype, loss_scale, max_norm):
+    import math
+    from helpers import build_workload, compare_state, refresh_oracle_grads
+    kw = dict(initial_scale=loss_scale, hysteresis=1) if dtype == torch.float16 else {}
+    module, opt, ochunks = build_workload(_tiny_named(), 1 << 15, dtype, seed=31, loss_scale=loss_scale,
+                                          grad_std=2e-2 if max_norm else 1e-3, weight_decay=0.1, max_norm=max_norm,
+                                          host_resident=True, **kw)
+    assert len(module.param_chunks) >= 2
+    for pc in module.param_chunks:
+        assert pc.shard.is_pinned() and pc.paired_chunk.shard.is_pinned()
+        assert all(t.is_pinned() for t in opt._binding.moments(pc.paired_chunk))
+    scaler = (O.DynamicGradScalerOracle(initial_scale=loss_scale, min_scale=1, max_scale=2**24, hysteresis=1)
+              if dtype == torch.float16 else O.ConstantGradScalerOracle(1.0))
+    g = torch.Generator().manual_seed(5)
+    for step in range(2):
+        if step:
+            for pc in module.param_chunks:
+                grads = torch.randn(pc.shard_size, generator=g) * (1e-3 * loss_scale)
+                grads[pc.utilized_size:] = 0
+                pc.shard.copy_(grads.to(dtype))
+                pc.invalidate_stats()
+            refresh_oracle_grads(module, ochunks)
+        opt.mark_gradients_scaled()
+        opt.step()
+        torch.cuda.synchronize()
+        info = O.reference_step(ochunks, CODE[dtype], scaler, max_norm=max_norm, adamw_mode=True)
+        assert opt.last_step_info['found_inf'] is False and info['found_inf'] is False
+        if max_norm:
+            assert math.isclose(opt.last_step_info['combined_scale'], info['combined_scale'], rel_tol=1e-6)
+            compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-11, atol_v=1e-14)
+        else:
+            assert opt.last_step_info['combined_scale'] == info['combined_scale']
+            assert compare_state(module, opt, ochunks, dtype, exact=True) == 0
+        assert all(pc.optim_sync_flag for pc in module.param_chunks)
+
+    # an overflow: skipped, master and moments untouched, the refresh of the host shard deferred
+    module.param_chunks[0].shard[3] = float('inf')
+    module.param_chunks[0].invalidate_stats()
+    before = [pc.paired_chunk.shard.clone() for pc in module.param_chunks]
+    opt.mark_gradients_scaled()
+    opt.step()
+    torch.cuda.synchronize()
+    assert opt.last_step_info['found_inf'] is True
+    for pc, p0 in zip(module.param_chunks, before):
+        assert torch.equal(pc.paired_chunk.shard, p0)
+        assert pc.optim_sync_flag is False                                  # chunk.py:416-419
+        block = torch.empty(pc.chunk_size, dtype=dtype, device=DEV)
+        pc.replicate(block)
+        pc.scatter(block)
+        assert torch.equal(pc.shard, p0.to(dtype)) and pc.optim_sync_flag is True
+
+
+def test_pageable_host_shards_are_refused():
+    named = [('w', (64, 64))]
+    sr = ea.greedy_search([('w', 4096)], 8192, torch.float16, shard_device=torch.device('cpu'))
+    module = ea.ElixirModule(dict(named), sr, dtype=torch.float16)
+    inner = ea.HybridAdam(list(module.parameters()), lr=1e-3)
+    opt = ea.ElixirOptimizer(module, inner, initial_scale=2.0)
+    opt.mark_gradients_scaled()
+    with pytest.raises(RuntimeError, match='pinned'):
+        opt.step()
