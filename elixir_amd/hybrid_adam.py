@@ -12,7 +12,9 @@ Two ways in:
 
 Either way one step is one launch over every tensor of every parameter group.  The arithmetic
 follows ``torch.optim.Adam`` / ``AdamW`` (float64 host scalars narrowed to fp32, same op order);
-there is no CPU path.
+there is no CPU path.  "Hybrid" in the reference means GPU kernels for device-resident shards and
+a CPU Adam for host-resident ones; here shards in pinned host memory go into the same launch and
+are read and written in place over the host link, shards in pageable host memory are refused.
 """
 import math
 from typing import Dict, List, Optional, Tuple
