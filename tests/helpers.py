@@ -53,7 +53,11 @@ def build_workload(named_shapes, chunk_size, dtype, *, seed=0, grad_std=1e-3, lo
     copy of the same data.  Gradients (already multiplied by ``loss_scale``) sit in the
     low-precision shards, as they do after backward."""
     named_shapes = list(named_shapes)
-    if host_resident:    # shards (and with them the moments) in pinned host memory
+    if host_resident == 'mixed':    # every other chunk in pinned host memory, the rest on the GPU
+        sr = ea.greedy_search([(n, S.numel(s)) for n, s in named_shapes], chunk_size, dtype)
+        for plan in sr.param_chunk_plans[::2]:
+            plan.kwargs.update(shard_device=torch.device('cpu'), cpu_pin_memory=True)
+    elif host_resident:    # shards (and with them the moments) in pinned host memory
         sr = ea.greedy_search([(n, S.numel(s)) for n, s in named_shapes], chunk_size, dtype,
                               shard_device=torch.device('cpu'))
         for plan in sr.param_chunk_plans:

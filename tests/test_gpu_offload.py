@@ -173,3 +173,21 @@ def test_pageable_host_shards_are_refused():
     opt.mark_gradients_scaled()
     with pytest.raises(RuntimeError, match='pinned'):
         opt.step()
+
+
+def test_mixed_placement_steps_in_one_launch(oracle):
+    """Every other chunk pair in pinned host memory, the others in device memory: one stats launch and
+    one update launch cover both, and the result is the oracle's bit for bit."""
+    from helpers import build_workload, compare_state
+    dtype = torch.float16
+    module, opt, ochunks = build_workload(_tiny_named(), 1 << 15, dtype, seed=33, loss_scale=64.0, weight_decay=0.1,
+                                          host_resident='mixed', initial_scale=64.0, hysteresis=1)
+    where = [pc.shard_device.type for pc in module.param_chunks]
+    assert 'cpu' in where and 'cuda' in where
+    opt.mark_gradients_scaled()
+    opt.step()
+    torch.cuda.synchronize()
+    scaler = O.DynamicGradScalerOracle(initial_scale=64.0, min_scale=1, max_scale=2**24, hysteresis=1)
+    info = O.reference_step(ochunks, CODE[dtype], scaler, max_norm=0.0, adamw_mode=True)
+    assert opt.last_step_info['found_inf'] is False and opt.last_step_info['combined_scale'] == info['combined_scale']
+    assert compare_state(module, opt, ochunks, dtype, exact=True) == 0
