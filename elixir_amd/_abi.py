@@ -13,6 +13,7 @@ import numpy as np
 ELX_ABI_VERSION = 1
 ELX_F32, ELX_F16, ELX_BF16, ELX_NONE = 0, 1, 2, -1
 ELX_FLAG_SCALAR_ONLY = 1
+ELX_E_NULL, ELX_E_DTYPE, ELX_E_ALIGN, ELX_E_RANGE, ELX_E_ORDER, ELX_E_TILES, ELX_E_SIZE = -1, -2, -3, -4, -5, -6, -7
 ELX_HYPER_L2 = 1
 ELX_HYPER_LERP_FROM_G = 2
 
@@ -30,7 +31,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg',
            'elx_sizeof_hyper', 'elx_sizeof_stats', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
-           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_land_grads_mt', 'elx_land_max_blocks', 'elx_land_tile_elems', 'elx_land_fold_blocks')
+           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems', 'elx_land_fold_blocks')
 
 
 class ElxError(RuntimeError):
@@ -74,6 +75,8 @@ def load() -> ctypes.CDLL:
     L.elx_writeback_mt.argtypes = [vp, u32, cint, u32, u32, vp]
     L.elx_land_tile_elems.restype = u32
     L.elx_land_tile_elems.argtypes = [cint]
+    L.elx_check_land_rows.restype = cint
+    L.elx_check_land_rows.argtypes = [vp, u32, vp, u32, cint, cint, ctypes.POINTER(u32)]
     L.elx_land_grads_mt.restype = cint
     L.elx_land_grads_mt.argtypes = [vp, u32, vp, u32, cint, cint, flt, u32, vp, vp, u32, vp]
 
@@ -193,3 +196,17 @@ def land_grads_mt(d_rows: int, n_rows: int, src_dtype: int, dst_dtype: int, mul:
     check('elx_land_grads_mt',
           load().elx_land_grads_mt(d_rows, n_rows, d_slot_offsets or None, n_slots, src_dtype, dst_dtype, mul,
                                    blocks_per_row, d_partials, d_stats, flags, stream))
+
+
+def check_land_rows(rows: np.ndarray, slot_offsets: Optional[np.ndarray], src_dtype: int, dst_dtype: int) -> int:
+    """Validate a host landing table; returns the one-tile-per-workgroup grid width."""
+    assert rows.dtype == CHUNK_DTYPE
+    n_slots = 0
+    if slot_offsets is not None:
+        assert slot_offsets.dtype == np.uint32
+        n_slots = len(slot_offsets) - 1
+    bpr = ctypes.c_uint32(0)
+    check('elx_check_land_rows',
+          load().elx_check_land_rows(_np_ptr(rows), len(rows), _np_ptr(slot_offsets), n_slots, src_dtype, dst_dtype,
+                                     ctypes.byref(bpr)))
+    return int(bpr.value)

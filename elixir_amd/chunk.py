@@ -131,12 +131,6 @@ def l2_norm_from_sumsq(sumsq: float) -> float:
     return float(np.float32(math.sqrt(sumsq)))**2
 
 
-def land_launch_blocks(n_alloc_max: int, src_dtype: int) -> int:
-    """Workgroups per row of the landing launch: one per tile."""
-    tile = _abi.land_tile_elems(src_dtype)
-    return int(max(1, min(_abi.land_max_blocks(), (n_alloc_max + tile - 1) // tile)))
-
-
 LAND_BLOCKS_PER_CU = 0    # 0: the library default
 
 
@@ -208,7 +202,7 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
         rows[i]['n_alloc'] = c.shard_size
         rows[i]['n_valid'] = c.n_valid
     aligned = bool(np.all(rows['grad'] % 16 == 0) and np.all(rows['lowp_out'] % 16 == 0))
-    bpr = land_launch_blocks(int(rows['n_alloc'].max()), src_code)
+    bpr = _abi.check_land_rows(rows, None, src_code, dst_code)
     ws = chunks[0]._workspace
     need = _abi.land_workspace_records(len(rows), bpr) * arena.itemsize
     buf = ws.get('land')
@@ -317,7 +311,7 @@ def land_tensors(chunks: List['Chunk'], grad_of, mul: float = 1.0) -> None:
         first = arena.new_slots(len(chunks))
         for i, c in enumerate(chunks):
             c._stats_slot = first + i
-    bpr = max(1, (int(rows['n_alloc'].max()) + tile - 1) // tile)
+    bpr = _abi.check_land_rows(rows, slot_offsets, src_code, dst_code)
     ws = chunks[0]._workspace
     need = _abi.land_workspace_records(len(rows), bpr, len(chunks)) * arena.itemsize
     buf = ws.get('land')

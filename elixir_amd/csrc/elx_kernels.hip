@@ -872,6 +872,35 @@ int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *
     return 0;
 }
 
+int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t *h_slot_offsets, uint32_t n_slots,
+                        int src_dtype, int dst_dtype, uint32_t *blocks_per_row) {
+    if (!h_rows || !blocks_per_row) return ELX_E_NULL;
+    if (!is_lowp_or_f32(src_dtype) || !is_lowp_or_f32(dst_dtype)) return ELX_E_DTYPE;
+    if (src_dtype != dst_dtype && src_dtype != ELX_F32) return ELX_E_DTYPE;
+    if (n_rows == 0 || n_rows > 65535u) return ELX_E_SIZE;
+    const uintptr_t smask = elem_size(src_dtype) - 1, dmask = elem_size(dst_dtype) - 1;
+    const uint64_t tile = kWave * (16u / elem_size(src_dtype)) * kLandUnroll;
+    uint64_t max_tiles = 1;
+    for (uint32_t i = 0; i < n_rows; ++i) {
+        const ElxChunk &r = h_rows[i];
+        if (!r.lowp_out) return ELX_E_NULL;
+        if (r.n_alloc == 0) return ELX_E_SIZE;
+        if (r.n_valid > r.n_alloc) return ELX_E_RANGE;
+        if (((uintptr_t)r.grad & smask) || ((uintptr_t)r.lowp_out & dmask)) return ELX_E_ALIGN;
+        const uint64_t t = (r.n_alloc + tile - 1) / tile;
+        if (t > max_tiles) max_tiles = t;
+    }
+    if (max_tiles > kMaxLandBlocks) return ELX_E_SIZE;
+    if (h_slot_offsets) {
+        if (n_slots == 0 || n_slots > n_rows) return ELX_E_SIZE;
+        if (h_slot_offsets[0] != 0 || h_slot_offsets[n_slots] != n_rows) return ELX_E_RANGE;
+        for (uint32_t s = 0; s < n_slots; ++s)
+            if (h_slot_offsets[s] > h_slot_offsets[s + 1]) return ELX_E_ORDER;
+    }
+    *blocks_per_row = (uint32_t)max_tiles;
+    return 0;
+}
+
 int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
                       ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream) {
     if (!d_chunks || !d_partials || !d_stats) return ELX_E_NULL;

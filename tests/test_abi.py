@@ -127,3 +127,37 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_NONE, 4, 0, None) == -2
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_F16, 0, 0, None) == -7
     assert lib.elx_refresh_piece_elems() == 4096
+
+
+def test_check_land_rows_accepts_and_rejects():
+    tile = _abi.land_tile_elems(_abi.ELX_F16)
+    assert tile == 2048 and _abi.land_tile_elems(_abi.ELX_F32) == 1024
+    rows = np.zeros(3, dtype=_abi.CHUNK_DTYPE)
+    rows['grad'] = [0x10000000, 0, 0x30000000]
+    rows['lowp_out'] = [0x40000000, 0x50000000, 0x60000002]
+    rows['n_alloc'] = [5 * tile, 7, 3 * tile + 1]
+    rows['n_valid'] = [5 * tile, 0, 3 * tile + 1]
+    assert _abi.check_land_rows(rows, None, _abi.ELX_F16, _abi.ELX_F16) == 5
+    assert _abi.check_land_rows(rows, np.array([0, 2, 3], dtype=np.uint32), _abi.ELX_F16, _abi.ELX_F16) == 5
+    assert _abi.check_land_rows(rows, None, _abi.ELX_F32, _abi.ELX_F16) == 10
+
+    def expect(code, r=rows, offsets=None, sd=_abi.ELX_F16, dd=_abi.ELX_F16):
+        with pytest.raises(_abi.ElxError) as e:
+            _abi.check_land_rows(r, offsets, sd, dd)
+        assert e.value.code == code, e.value
+
+    expect(_abi.ELX_E_DTYPE, sd=_abi.ELX_F16, dd=_abi.ELX_F32)
+    expect(_abi.ELX_E_DTYPE, sd=_abi.ELX_BF16, dd=_abi.ELX_F16)
+    bad = rows.copy(); bad['lowp_out'][1] = 0
+    expect(_abi.ELX_E_NULL, bad)
+    bad = rows.copy(); bad['n_alloc'][0] = 0; bad['n_valid'][0] = 0
+    expect(_abi.ELX_E_SIZE, bad)
+    bad = rows.copy(); bad['n_valid'][1] = 8
+    expect(_abi.ELX_E_RANGE, bad)
+    bad = rows.copy(); bad['grad'][0] += 1
+    expect(_abi.ELX_E_ALIGN, bad)
+    expect(_abi.ELX_E_ALIGN, sd=_abi.ELX_F32, dd=_abi.ELX_F32)            # 0x60000002 is not 4-byte aligned
+    expect(_abi.ELX_E_RANGE, offsets=np.array([1, 2, 3], dtype=np.uint32))
+    expect(_abi.ELX_E_RANGE, offsets=np.array([0, 2, 2], dtype=np.uint32))
+    expect(_abi.ELX_E_ORDER, offsets=np.array([0, 3, 2, 3], dtype=np.uint32))
+    expect(_abi.ELX_E_SIZE, offsets=np.array([0, 1, 2, 3, 3], dtype=np.uint32))
