@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the optimizer step (ElixirOptimizer.step over chunk-packed parameters) on one GPU.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c2|c1]
 
 A step is one full pass of the hot path over one set of synthetic gradients that already sit in
 the low-precision chunk shards: stats launch (overflow flag + sum of squares) -> 16 B/chunk
@@ -276,12 +276,69 @@ def offload_step_leg(mi_elements, steps=5):
     return out
 
 
+def config1_line(args):
+    """Configuration 1: plain fp32 Adam on one flat buffer of 16,777,216 elements (p ~ N(0, 0.02),
+    g ~ N(0, 1e-2), m = v = 0 at the start, lr 1e-3, betas (0.9, 0.999), eps 1e-8, no weight decay,
+    no loss scale, no stats pass, no low-precision copy) -- the case torch.optim.Adam runs on the
+    CPU.  28 B per element: read p, g, m, v, write p, m, v.  The whole state (268 MB) is about the
+    size of the last-level cache, so this line says little about HBM; it is the latency case."""
+    import elixir_amd as ea
+    n = 1 << 24
+    gen = torch.Generator(device='cuda')
+    gen.manual_seed(1234 + 1)
+    p = torch.nn.Parameter(torch.randn(n, device='cuda', generator=gen) * 0.02)
+    g = torch.randn(n, device='cuda', generator=gen) * 1e-2
+    opt = ea.HybridAdam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
+    p.grad = g
+    step_s, adam_ms = [], []
+    for i in range(args.warmup + args.steps):
+        opt.kernel_events = {}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if i >= args.warmup:
+            step_s.append(dt)
+            ev = opt.kernel_events['adam_step']
+            adam_ms.append(ev[0].elapsed_time(ev[1]))
+    opt.kernel_events = None
+    t_step, t_upd = float(np.mean(step_s)), float(np.mean(adam_ms)) * 1e-3
+    out = {
+        'metric': 'adam_elements_per_sec', 'value': n / t_step, 'unit': 'elements/s', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': t_step * 1e3, 'higher_is_better': True, 'scaling': 'weak',
+        'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'c1: plain fp32 Adam, one flat buffer of 16Mi elements, no loss scale, no low-precision '
+                               'copy', 'valid_elements': n},
+        'step': {'ms_min': float(np.min(step_s)) * 1e3, 'gbps_28B': BYTES_UPDATE * n / t_step / 1e9,
+                 'frac_28B': BYTES_UPDATE * n / t_step / 1e9 / HBM_PEAK_GBPS},
+        'roofline': {'kernel': 'adam_step_kernel', 'bound': 'hbm', 'achieved': BYTES_UPDATE * n / t_upd / 1e9,
+                     'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': BYTES_UPDATE * n / t_upd / 1e9 / HBM_PEAK_GBPS,
+                     'traffic': None, 'bytes_per_launch': BYTES_UPDATE * n, 'ms_per_launch': t_upd * 1e3},
+    }
+    if args.cpu_sample > 0:
+        # the reference's own path for this configuration: torch.optim.Adam on CPU tensors, full size
+        cp = torch.nn.Parameter(p.detach().cpu())
+        copt = torch.optim.Adam([cp], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
+        cp.grad = g.cpu()
+        ts = []
+        for _ in range(6):
+            t0 = time.perf_counter()
+            copt.step()
+            ts.append(time.perf_counter() - t0)
+        t = float(np.median(ts[1:]))
+        out['cpu_baseline'] = {'value': n / t, 'unit': 'elements/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+                               'sample': 'the whole configuration: torch.optim.Adam on CPU fp32 tensors, median of 5 '
+                                         'steps after 1 warm-up', 'ms_per_step_sample': t * 1e3}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=3)
-    ap.add_argument('--workload', default='c5', choices=['c2', 'c4', 'c5'])
+    ap.add_argument('--workload', default='c5', choices=['c1', 'c2', 'c4', 'c5'])
     ap.add_argument('--cpu-sample', type=int, default=128 << 20, help='elements of the CPU baseline sample; 0 skips it')
     ap.add_argument('--blocks-per-cu', type=int, default=0,
                     help='cap on resident update workgroups per compute unit (0 = library default)')
@@ -326,6 +383,9 @@ def main():
     _abi.load()
     device = torch.device('cuda', 0)
     torch.cuda.set_device(device)
+    if args.workload == 'c1':
+        config1_line(args)
+        return
 
     t_build = time.perf_counter()
     built = workloads.build(args.workload, device)
