@@ -8,10 +8,14 @@ gradient buffer at step time, and an fp32 chunk that holds the master weights
 ``shard_begin == 0``.
 
 What is kept: the layout fields and rules (``append_tensor``, ``close_chunk``, ``valid_end``,
-``tensors_info``, ``init_pair``), the reduction flags (``overflow``, ``l2_norm``,
-``update_extra_reduce_info``) and ``optim_update``.  The flags and the low-precision refresh run on
-the HIP kernels.  What is not here: the replicated-cache blocks, gather / scatter / reduce-scatter
-and the tensor state machine of the forward/backward pass.
+``tensors_info``, ``init_pair``), the landing of reduced gradients in the shard (``reduce_chunk``;
+``land_chunks`` / ``land_tensors`` for many chunks in one launch) with the reduction flags
+(``overflow``, ``l2_norm``, ``update_extra_reduce_info``) taken in the same pass, ``optim_update``,
+the source copy of the gather and the release (``replicate`` / ``scatter`` on a caller-provided
+block) including the deferred refresh of host-resident shards, and ``get_cpu_copy`` /
+``load_tensors``.  Everything that touches chunk contents on the GPU runs on the HIP kernels.  What is
+not here: the replicated-cache block pool, the collectives and the tensor state machine of the
+forward/backward pass.
 """
 import math
 from dataclasses import dataclass

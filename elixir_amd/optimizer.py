@@ -3,10 +3,11 @@ constructor, methods and control flow, driving the HIP kernels.
 
 One step is:
 
-  1. one stats launch over every parameter chunk that has no fresh flags (overflow flag and sum of
-     squares of the still-scaled gradients) and ONE device-to-host copy of 16 bytes per chunk
-     (the reference pays two ``.item()`` per chunk at gradient-landing time, plus one for the loss
-     scale, plus one for the norm);
+  1. one stats launch over every parameter chunk that has no flags yet (overflow flag and sum of
+     squares of the still-scaled gradients) -- none at all when the gradients arrived through the
+     fused landing, which leaves the flags on the device -- and ONE device-to-host copy of 16 bytes
+     per chunk (the reference pays two ``.item()`` per chunk at gradient-landing time, plus one for
+     the loss scale, plus one for the norm);
   2. the host decisions of optimizer.py:192-209 in Python floats: overflow -> skip and back off,
      otherwise combined scale = loss scale (x clip coefficient);
   3. one fused launch: unscale + Adam/AdamW on master/m/v + low-precision writeback
@@ -17,7 +18,10 @@ Differences from the reference, all on purpose:
     reference never sets the flag and trips its own assertion, optimizer.py:152);
   * bfloat16 parameter chunks are accepted (``use_amp`` stays tied to float16, so bf16 trains
     with a constant scale of 1 and the overflow check still runs);
-  * exp_avg / exp_avg_sq live in flat per-chunk buffers (``state[p]['exp_avg']`` are views).
+  * exp_avg / exp_avg_sq live in flat per-chunk buffers (``state[p]['exp_avg']`` are views);
+  * ``state_dict`` / ``load_state_dict`` also carry the loss scaler, and loading copies into the
+    flat buffers in place;
+  * shards in pinned host memory are stepped by the same launches, in place over the host link.
 """
 import math
 from collections import defaultdict
