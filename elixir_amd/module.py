@@ -122,6 +122,13 @@ class ElixirModule(nn.Module):
         self.param_to_optim: Dict[nn.Parameter, torch.Tensor] = dict()
         self.__init_chunk_group(search_result, module)
         self.fetcher = _Fetcher(self.param_chunk_group)
+        # landing during backward: chunks whose gradients are complete land from a hook
+        self._landing_in_backward = False
+        self._ready: Dict[Chunk, set] = {}
+        self._landed: set = set()
+        if not self.synthetic:
+            for param in self.grad_state_dict.values():
+                param.register_post_accumulate_grad_hook(self._gradient_handler)
 
     def __init_chunk_group(self, sr: SearchResult, module):
         device = gpu_device() if torch.cuda.is_available() else torch.device('cpu')
@@ -223,12 +230,38 @@ class ElixirModule(nn.Module):
             outputs = outputs.float()
         return outputs
 
+    def _gradient_handler(self, param: nn.Parameter) -> None:
+        """module.py:177-190 as a post-accumulate hook: when the last gradient of a chunk has been
+        produced, the chunk lands at once (one launch, flags included) and its gradients are freed,
+        so that at most one chunk's worth of gradients outlives its producer, as in the reference,
+        where a chunk is reduced as soon as all its tensors are ready."""
+        if not self._landing_in_backward:
+            return
+        chunk = self.param_chunk_group.ten_to_chunk[param]
+        if chunk.shard_device.type != 'cuda':
+            return    # host-resident: lands after backward, through a payload and a transfer
+        ready = self._ready.setdefault(chunk, set())
+        ready.add(param)
+        if len(ready) == chunk.num_tensors:
+            land_tensors([chunk], lambda t: t.grad.data.contiguous())
+            for t in chunk.tensors_info:
+                t.grad = None
+            self._landed.add(chunk)
+            ready.clear()
+
     def backward(self, loss: torch.Tensor):
-        loss.backward()
-        self.land_gradients()
+        self._landed.clear()
+        self._ready.clear()
+        self._landing_in_backward = True
+        try:
+            loss.backward()
+        finally:
+            self._landing_in_backward = False
+        self.land_gradients(skip=self._landed)
+        self._landed = set()
         self.module.zero_grad(set_to_none=True)
 
-    def land_gradients(self, sync: bool = False) -> None:
+    def land_gradients(self, sync: bool = False, skip=()) -> None:
         """module.py:177-190 + chunk.py:358-393 for one process: every parameter's gradient goes
         into its slice of the chunk's shard, what no parameter covers becomes zero (as the
         replicated block of the reference is after a gather of zero padding), and the flags of every
@@ -237,7 +270,7 @@ class ElixirModule(nn.Module):
         ``sync`` the flags are fetched here, otherwise when somebody reads them (the optimizer step
         does, for all chunks at once)."""
         assert not self.synthetic
-        on_gpu = [c for c in self.param_chunks if c.shard_device.type == 'cuda']
+        on_gpu = [c for c in self.param_chunks if c.shard_device.type == 'cuda' and c not in skip]
         if on_gpu:
 
             def grad_of(param):
@@ -249,7 +282,7 @@ class ElixirModule(nn.Module):
                 for chunk in on_gpu:
                     chunk.update_extra_reduce_info()
         for chunk in self.param_chunks:
-            if chunk.shard_device.type == 'cuda':
+            if chunk.shard_device.type == 'cuda' or chunk in skip:
                 continue
             payload = torch.zeros(chunk.chunk_size, dtype=chunk.chunk_dtype, device=chunk.shard_device)
             for param, info in chunk.tensors_info.items():

@@ -219,3 +219,56 @@ def test_clipped_training_matches_torchs_clip_grad_norm(dtype):
         sd = module.state_dict()
         for name, want in master.state_dict().items():
             torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
+
+
+def test_chunks_land_from_hooks_during_backward(monkeypatch):
+    """module.py:177-190: a chunk lands as soon as its last gradient exists -- one launch per chunk,
+    issued from inside backward, gradients freed right away -- and the shards hold exactly what a
+    landing after backward would have put there."""
+    import elixir_amd.module as M
+    torch.manual_seed(5)
+    model = Net().to(DEV)
+    module, opt = wrap(model, torch.float16, initial_scale=256.0)
+    n_chunks = len(module.param_chunks)
+    assert n_chunks >= 4
+    calls = []
+    inside = {'flag': False}
+    real = M.land_tensors
+
+    def spy(chunks, grad_of, mul=1.0):
+        calls.append((len(chunks), inside['flag'], sum(p.grad is not None for p in model.parameters())))
+        return real(chunks, grad_of, mul)
+
+    monkeypatch.setattr(M, 'land_tensors', spy)
+    real_backward = torch.Tensor.backward
+
+    def marked_backward(self, *a, **k):
+        inside['flag'] = True
+        try:
+            return real_backward(self, *a, **k)
+        finally:
+            inside['flag'] = False
+
+    monkeypatch.setattr(torch.Tensor, 'backward', marked_backward)
+    gen = torch.Generator(device=DEV).manual_seed(6)
+    x = batch(gen)
+    opt.zero_grad()
+    opt.backward(module(x))
+    assert len(calls) == n_chunks and all(n == 1 and was_inside for n, was_inside, _ in calls)
+    n_params = sum(1 for _ in model.parameters())
+    assert max(alive for _, _, alive in calls) < n_params        # earlier chunks had already freed theirs
+    assert all(p.grad is None for p in model.parameters())
+    assert all(pc._stats_pending for pc in module.param_chunks)
+    landed = [pc.shard.clone() for pc in module.param_chunks]
+
+    # the same gradients, landed after a plain backward
+    monkeypatch.setattr(torch.Tensor, 'backward', real_backward)
+    (module(x) * opt.loss_scale).backward()
+    for pc in module.param_chunks:
+        pc.invalidate_stats()
+    module.land_gradients()
+    for pc, want in zip(module.param_chunks, landed):
+        assert torch.equal(pc.shard.view(torch.int16), want.view(torch.int16))
+    module.module.zero_grad(set_to_none=True)
+    opt.step()
+    assert opt.last_step_info['found_inf'] is False
