@@ -362,9 +362,9 @@ def test_land_rows_tile_every_piece_exactly():
             k += 1
     assert k == len(rows)
     # block choice: a power of two of at least 16 tiles that keeps a 7.2 G element set below 32 Ki rows
-    assert _land_block_elems(1000, 2048) == 16 * 2048
-    b = _land_block_elems(7_247_757_312, 2048)
-    assert b & (b - 1) == 0 and 7_247_757_312 // b < 16384 <= 7_247_757_312 // (b // 2)
+    assert _land_block_elems(1000, 2048) == 2048 * 2048 == _land_block_elems(7_247_757_312, 2048)
+    b = _land_block_elems(1 << 40, 2048)
+    assert b & (b - 1) == 0 and (1 << 40) // b <= 32768 < (1 << 40) // (b // 2)
 
 
 # ------------------------------------------------------------------------------------------------
