@@ -81,6 +81,7 @@ class _HyperUploader:
 
     def __init__(self):
         self.staging: List[torch.Tensor] = []
+        self.copied: List[Optional[torch.cuda.Event]] = [None, None]
         self.dev: Optional[torch.Tensor] = None
         self.turn = 0
 
@@ -90,10 +91,16 @@ class _HyperUploader:
             cap = max(4096, nbytes)
             self.dev = torch.empty(cap, dtype=torch.uint8, device=device)
             self.staging = [torch.empty(cap, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
-        stage = self.staging[self.turn]
+            self.copied = [None, None]
+        turn = self.turn
+        stage = self.staging[turn]
         self.turn ^= 1
+        if self.copied[turn] is not None:
+            self.copied[turn].synchronize()    # normally long past: the copy out of this buffer has run
         stage[:nbytes].numpy()[:] = host.view(np.uint8).reshape(-1)
         self.dev[:nbytes].copy_(stage[:nbytes], non_blocking=True)
+        self.copied[turn] = torch.cuda.Event()
+        self.copied[turn].record(torch.cuda.current_stream(device))
         return self.dev.data_ptr()
 
 
@@ -170,6 +177,7 @@ class _Prepared:
         self.grad_code, self.lowp_code, self.device = grad_code, lowp_code, device
         self.states: List[Dict] = states      # per-parameter state dicts whose 'step' advances on commit
         self.d_hypers: int = 0
+        self.sig = None
 
 
 class HybridAdam(torch.optim.Optimizer):
@@ -252,6 +260,9 @@ class HybridAdam(torch.optim.Optimizer):
         can overlap this host work with device work whose result decides whether the step happens
         (``ElixirOptimizer`` calls it between launching and reading the gradient flags).  The next
         ``step()`` consumes what was prepared; ``discard_prepared()`` drops it."""
+        sig = self._prepare_signature()
+        if self._prepared is not None and sig is not None and self._prepared.sig == sig:
+            return    # prepared ahead of time (ElixirOptimizer.backward does) and still valid
         hypers: Dict = {}
         if self._binding is not None:
             self._prepared = self._prepare_bound(hypers)
@@ -259,7 +270,18 @@ class HybridAdam(torch.optim.Optimizer):
             self._prepared = self._prepare_standalone(hypers)
         prep = self._prepared
         if prep is not None:
+            prep.sig = sig
             prep.d_hypers = self._hyper_uploader.upload(prep.hyper_host, prep.device)
+
+    def _prepare_signature(self):
+        """Everything a prepared step of bound chunks depends on besides the step counts (which only
+        change when a prepared step is consumed or a state is loaded, and both drop it): the group
+        hyper-parameters, the group sizes and the kind of step.  None for standalone parameters,
+        whose gradient buffers change from step to step."""
+        if self._binding is None:
+            return None
+        return (self._binding.zero_grads,
+                tuple((len(g['params']), ) + self._group_key(g, 0) for g in self.param_groups))
 
     def discard_prepared(self) -> None:
         self._prepared = None

@@ -455,6 +455,14 @@ class ElixirOptimizer:
         loss = self.loss_scale * loss
         self.optim_state = OptimState.SCALED
         self.module.backward(loss)
+        self.prepare_ahead()
+
+    def prepare_ahead(self) -> None:
+        """Builds and uploads the tables of the coming step now, while the device is still busy with
+        backward and the landing of the gradients; ``step()`` then finds them ready (and rebuilds them
+        if a hyper-parameter has changed in between)."""
+        if self._binding is not None:
+            self.optim.prepare_step()
 
     def backward_by_grad(self, tensor: torch.Tensor, grad: torch.Tensor):
         self.optim_state = OptimState.SCALED

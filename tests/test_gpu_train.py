@@ -272,3 +272,33 @@ def test_chunks_land_from_hooks_during_backward(monkeypatch):
     module.module.zero_grad(set_to_none=True)
     opt.step()
     assert opt.last_step_info['found_inf'] is False
+
+
+def test_tables_prepared_at_backward_follow_late_hyperparameter_changes():
+    """``backward`` prepares the tables of the coming step ahead of time; a learning rate changed
+    between backward and step must still be the one the step uses."""
+    torch.manual_seed(2)
+    ref = Net().to(DEV)
+    model = copy.deepcopy(ref)
+    ropt = torch.optim.AdamW(groups_of(ref, 0.1), lr=1e-2, weight_decay=0.1)
+    module, opt = wrap(model, torch.float32)
+    gen = torch.Generator(device=DEV).manual_seed(8)
+    for step in range(4):
+        x = batch(gen)
+        ropt.zero_grad()
+        ref(x).backward()
+        opt.zero_grad()
+        opt.backward(module(x))
+        assert opt.optim._prepared is not None                 # built ahead of the step
+        ahead = opt.optim._prepared
+        if step % 2 == 1:                                      # a scheduler that fires late
+            for g in list(ropt.param_groups) + list(opt.param_groups):
+                g['lr'] = g['lr'] * 0.5
+        ropt.step()
+        opt.step()
+        assert opt.optim._prepared is None                     # consumed
+        module.materialize_params()
+        sd = module.state_dict()
+        for name, want in ref.state_dict().items():
+            torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
+        del ahead
