@@ -614,7 +614,13 @@ __device__ __forceinline__ typename Elem<DD>::scalar land_elem(typename Elem<SD>
         return x;
     } else {
         float v = Elem<SD>::to_f32(x);
-        if constexpr (MUL) v = Elem<SD>::to_f32(Elem<SD>::from_f32(v * mul));
+        if constexpr (MUL) {
+            v = v * mul;
+            // keep the product a plain fp32 multiply: folded into a mixed-precision fma with a +0
+            // addend it would turn -0 * mul into +0
+            asm volatile("" : "+v"(v));
+            v = Elem<SD>::to_f32(Elem<SD>::from_f32(v));
+        }
         const typename Elem<DD>::scalar d = Elem<DD>::from_f32(v);
         as_f32 = Elem<DD>::to_f32(d);
         return d;

@@ -127,6 +127,29 @@ def main():
         out[f'scaler/{label}/found'] = np.array(seq, dtype=np.int32)
         out[f'scaler/{label}/scale'] = np.array(traj, dtype=np.float64)
 
+    # gradient landing with torch's CPU ops: the payload divided in place by a power-of-two group
+    # size (chunk.py:299; for a power of two the division is the multiplication by the reciprocal
+    # that the device kernel performs), copied into a shard of the chunk's type (chunk.py:314), and
+    # the flags of what then sits in the shard (chunk.py:214-221)
+    lgen = torch.Generator().manual_seed(777)
+    lowps = {'f16': torch.float16, 'bf16': torch.bfloat16}
+    for dt, tdt in (('f16', torch.float16), ('bf16', torch.bfloat16), ('f32', torch.float32)):
+        for label, spread in (('tame', 1.0), ('wild', 6.0)):
+            x = (torch.randn(3000, generator=lgen) * torch.exp(torch.randn(3000, generator=lgen) * spread)).to(tdt)
+            out[f'land/{dt}/{label}/x'] = bits(x)
+            for pg in (1, 4):
+                y = x.clone()
+                if pg > 1:
+                    y /= pg
+                targets = {dt: y} if tdt != torch.float32 else {'f32': y, **{k: y.to(v) for k, v in lowps.items()}}
+                for tname, shard in targets.items():
+                    key = f'land/{dt}/{label}/pg{pg}/{tname}'
+                    out[key] = bits(shard)
+                    bad = bool(torch.isinf(shard).any() | torch.isnan(shard).any())
+                    out[key + '/flag'] = np.array(bad)
+                    if not bad:
+                        out[key + '/l2'] = np.array(shard.float().norm(2).item()**2, dtype=np.float64)
+
     np.savez_compressed(OUT, **out)
     print(f'wrote {OUT}: {len(out)} arrays, {os.path.getsize(OUT)} bytes')
 

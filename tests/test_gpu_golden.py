@@ -97,3 +97,39 @@ def test_scaler_trajectories(golden):
             sc.update(bool(f))
             got.append(sc.scale_value)
         assert got == list(golden[f'scaler/{label}/scale'])
+
+
+def test_landing_vectors(golden):
+    """The landing launch against the committed torch-CPU vectors: shard bits, flag, squared norm."""
+    from elixir_amd.chunk import DeviceTable
+    n_checked = 0
+    for key in golden.files:
+        parts = key.split('/')
+        if parts[0] != 'land' or len(parts) != 5:
+            continue
+        _, sd, label, pg, dd = parts
+        src = _to_dev(golden[f'land/{sd}/{label}/x'], sd)
+        want = golden[key]
+        dst = torch.zeros(src.numel(), dtype=TORCH[dd], device=DEV)
+        row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+        row['grad'], row['lowp_out'], row['n_alloc'], row['n_valid'] = src.data_ptr(), dst.data_ptr(), src.numel(), src.numel()
+        bpr = _abi.check_land_rows(row, None, CODE[sd], CODE[dd])
+        rec = _abi.STATS_DTYPE.itemsize
+        ws = torch.empty((_abi.land_workspace_records(1, bpr) + 1) * rec, dtype=torch.uint8, device=DEV)
+        table = DeviceTable(row, dst.device)
+        _abi.land_grads_mt(table.ptr, 1, CODE[sd], CODE[dd], float(np.float32(1.0 / int(pg[2:]))), bpr,
+                           ws.data_ptr(), ws.data_ptr() + ws.numel() - rec, True, torch.cuda.current_stream().cuda_stream)
+        stats = ws[-rec:].cpu().numpy().view(_abi.STATS_DTYPE)
+        got = to_np(dst)
+        if dd == 'f32':
+            nan = np.isnan(want)
+            assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan]), key
+        else:
+            nan = np.isnan(to_np(_to_dev(want, dd).float()))
+            assert np.array_equal(got[~nan], want[~nan]), key
+        assert bool(stats['overflow'][0]) == bool(golden[key + '/flag']), key
+        if key + '/l2' in golden.files:
+            l2 = float(np.float32(np.sqrt(stats['sumsq'][0])))**2
+            assert abs(l2 - float(golden[key + '/l2'])) <= 2e-6 * float(golden[key + '/l2']), key
+        n_checked += 1
+    assert n_checked == 20

@@ -435,3 +435,18 @@ def test_landing_on_a_side_stream_is_waited_for(oracle):
     assert pc.overflow is True
     side.synchronize()
     assert torch.equal(pc.shard.view(torch.int16), pl.view(torch.int16))
+
+
+@pytest.mark.parametrize('sd,dd', PAIRS)
+def test_scaled_landing_keeps_the_sign_of_zero(oracle, sd, dd):
+    """-0 * mul is -0, in the vector body and in the element-by-element tail alike (a mixed-precision
+    fma with a +0 addend, which compilers like to make of such a product, would lose the sign)."""
+    n = 5000                                             # one full tile and a tail
+    src = _payload(n, sd, 9)
+    src[::3] = -0.0
+    src[1::3] = 0.0
+    dst = torch.ones(n, dtype=dd, device=DEV)
+    _land(src, dst, n, mul=0.25)
+    want = oracle.land(to_np(src), CODE[sd], CODE[dd], mul=0.25)
+    assert np.array_equal(to_np(dst).view(np.uint8), want.view(np.uint8))
+    assert bool(torch.all(torch.signbit(dst[::3]))) and not bool(torch.any(torch.signbit(dst[1::3])))

@@ -529,3 +529,34 @@ def test_random_layouts_match_oracle(oracle, seed):
         info = _run_and_compare(module, opt, ochunks, dtype, scaler, adamw_mode=adamw, tag=f'seed {seed} step {step}')
         assert info['found_inf'] is False
         assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'seed {seed} step {step}') == 0
+
+
+@pytest.mark.parametrize('div_scale', [-1.0, 64.0, 48.0])
+@pytest.mark.parametrize('gdtype', [torch.float32, torch.float16, torch.bfloat16])
+def test_signed_zeros_go_through_the_update_like_ieee(oracle, gdtype, div_scale):
+    """Zeros of both signs in gradient, master and moments: every combination must come out with the
+    bits the scalar C oracle produces (a multiply folded into a fused op with a +0 addend would not)."""
+    vals = torch.tensor([0.0, -0.0, 1e-3, -2e-3])
+    grid = torch.cartesian_prod(vals, vals, vals)                # (g, p, m) combinations
+    reps = 70                                                    # several tiles, and a ragged tail
+    g0 = grid[:, 0].repeat(reps)
+    n = g0.numel()
+    p0, m0 = grid[:, 1].repeat(reps), grid[:, 2].repeat(reps)
+    v0 = torch.where(torch.arange(n) % 2 == 0, torch.zeros(n), torch.full((n,), 1e-6))
+    for adamw, wd in ((True, 0.1), (False, 0.1), (True, 0.0)):
+        p = torch.nn.Parameter(p0.clone().to(DEV))
+        opt = ea.HybridAdam([p], lr=1e-3, weight_decay=wd, adamw_mode=adamw)
+        p.grad_dtype = None
+        p.grad = g0.to(gdtype).to(DEV)
+        opt.step()                                               # creates the state (zeros)
+        st = opt.state[p]
+        p.data.copy_(p0)
+        st['exp_avg'].copy_(m0)
+        st['exp_avg_sq'].copy_(v0)
+        p.grad = g0.to(gdtype).to(DEV)
+        opt.step(div_scale=div_scale)
+        pn, mn, vn = p0.numpy().copy(), m0.numpy().copy(), v0.numpy().copy()
+        oracle.adam(to_np(g0.to(gdtype)), CODE[gdtype], pn, mn, vn, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8,
+                    weight_decay=wd, step=2, adamw_mode=adamw, div_scale=div_scale)
+        for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
+            assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32)), (name, adamw, wd)

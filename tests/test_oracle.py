@@ -418,3 +418,29 @@ def test_landing_rounds_twice_not_once(oracle):
     want = (x.astype(np.float32) * third).astype(np.float16)
     got = oracle.land(x.view(np.uint16), O.F16, O.F16, mul=float(third))
     assert np.array_equal(got, want.view(np.uint16))
+
+
+def test_golden_landing(oracle, golden):
+    """Committed vectors from torch's CPU ops: payload / group size, the copy into the shard, flags."""
+    n_checked = 0
+    for key in golden.files:
+        parts = key.split('/')
+        if parts[0] != 'land' or len(parts) != 5:
+            continue
+        _, sd, label, pg, dd = parts
+        x = golden[f'land/{sd}/{label}/x']
+        want = golden[key]
+        got = oracle.land(x, CODE[sd], CODE[dd], mul=1.0 / int(pg[2:]))
+        if dd == 'f32':
+            nan = np.isnan(want)
+            assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan]), key
+            assert np.all(np.isnan(got[nan])), key
+        else:
+            nan = np.isnan(oracle.lowp_to_f32(want, CODE[dd]))
+            assert np.array_equal(got[~nan], want[~nan]), key
+            assert np.all(np.isnan(oracle.lowp_to_f32(got[nan], CODE[dd]))), key
+        assert oracle.overflow(got, CODE[dd]) == bool(golden[key + '/flag']), key
+        if key + '/l2' in golden.files:
+            assert math.isclose(oracle.l2norm_sq_ref(got, CODE[dd]), float(golden[key + '/l2']), rel_tol=2e-6), key
+        n_checked += 1
+    assert n_checked == 20
