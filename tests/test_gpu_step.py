@@ -560,3 +560,47 @@ def test_signed_zeros_go_through_the_update_like_ieee(oracle, gdtype, div_scale)
                     weight_decay=wd, step=2, adamw_mode=adamw, div_scale=div_scale)
         for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
             assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32)), (name, adamw, wd)
+
+
+@pytest.mark.parametrize('gdtype,div_scale', [(torch.float32, -1.0), (torch.float16, 1024.0), (torch.bfloat16, 3.0)])
+def test_full_range_values_match_the_oracle(oracle, gdtype, div_scale):
+    """Magnitudes over the whole fp32 range -- subnormals, values whose square overflows or
+    underflows, infinities and NaNs in every operand: the same bits as the scalar C oracle, NaNs in
+    the same places."""
+    n = 1 << 16
+    gen = torch.Generator().manual_seed(17)
+
+    def wild(positive=False):
+        mag = torch.exp2(torch.rand(n, generator=gen) * 276.0 - 149.0)          # 2^-149 .. 2^127
+        x = mag if positive else mag * torch.where(torch.rand(n, generator=gen) < 0.5, -1.0, 1.0)
+        x[torch.rand(n, generator=gen) < 0.01] = 0.0
+        return x
+
+    g0, p0, m0, v0 = wild(), wild(), wild(), wild(positive=True)
+    for t, k in ((g0, 0), (p0, 1), (m0, 2), (v0, 3)):
+        t[100 + k] = float('inf')
+        t[200 + k] = float('nan')
+        if k != 3:
+            t[300 + k] = float('-inf')
+    g_low = g0.to(gdtype)
+    for adamw in (True, False):
+        p = torch.nn.Parameter(torch.zeros(n, device=DEV))
+        opt = ea.HybridAdam([p], lr=1e-2, weight_decay=0.1, adamw_mode=adamw)
+        p.grad_dtype = None
+        p.grad = torch.zeros(n, dtype=gdtype, device=DEV)
+        opt.step()
+        st = opt.state[p]
+        p.data.copy_(p0)
+        st['exp_avg'].copy_(m0)
+        st['exp_avg_sq'].copy_(v0)
+        p.grad = g_low.to(DEV)
+        opt.step(div_scale=div_scale)
+        pn, mn, vn = p0.numpy().copy(), m0.numpy().copy(), v0.numpy().copy()
+        oracle.adam(to_np(g_low), CODE[gdtype], pn, mn, vn, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.1,
+                    step=2, adamw_mode=adamw, div_scale=div_scale)
+        for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
+            got = to_np(got)
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(got), nan), (name, adamw)
+            bad = got.view(np.uint32)[~nan] != want.view(np.uint32)[~nan]
+            assert not bad.any(), (name, adamw, int(bad.sum()), got[~nan][bad][:4], want[~nan][bad][:4])
