@@ -33,6 +33,8 @@ def test_config1_flat_fp32_adam_16mi(oracle):
     opt = ea.HybridAdam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
     tp = torch.nn.Parameter(p0.clone())
     topt = torch.optim.Adam([tp], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
+    dp = torch.nn.Parameter(p0.clone().to(DEV))                       # torch's own Adam on the device
+    dopt = torch.optim.Adam([dp], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, foreach=False)
     pn, mn, vn = p0.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
     for step in (1, 2):
         g = torch.randn(n, generator=gen) * 1e-2
@@ -40,6 +42,8 @@ def test_config1_flat_fp32_adam_16mi(oracle):
         opt.step()                      # div_scale = -1: no unscale
         tp.grad = g.clone()
         topt.step()
+        dp.grad = g.to(DEV)
+        dopt.step()
         oracle.adam(g.numpy().copy(), O.F32, pn, mn, vn, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8,
                     weight_decay=0.0, step=step, adamw_mode=True)
         st = opt.state[p]
@@ -55,6 +59,13 @@ def test_config1_flat_fp32_adam_16mi(oracle):
         # p: 1e-6 relative, with the step size lr as the scale of the cancelling operands
         assert_close_f32(got['p'], tp.data.numpy(), f'step {step} p vs torch', rtol=1e-6, atol=1e-6 * 1e-3)
         assert_close_f32(got['m'], tst['exp_avg'].numpy(), f'step {step} m', rtol=1e-6, atol=1e-6 * gmax)
+        # and torch's Adam on the device (its kernels contract differently): the same 1e-6 bar
+        dst = dopt.state[dp]
+        assert_close_f32(got['p'], to_np(dp.data), f'step {step} p vs torch on the device', rtol=1e-6, atol=1e-6 * 1e-3)
+        assert_close_f32(got['m'], to_np(dst['exp_avg']), f'step {step} m vs torch on the device', rtol=1e-6,
+                         atol=1e-6 * gmax)
+        assert_close_f32(got['v'], to_np(dst['exp_avg_sq']), f'step {step} v vs torch on the device', rtol=1e-6,
+                         atol=1e-6 * gmax * gmax)
 
 
 def _poison_per_million(built, seed):
