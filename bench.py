@@ -340,7 +340,7 @@ def main():
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--workload', default='c5', choices=['c1', 'c2', 'c4', 'c5'])
-    ap.add_argument('--cpu-sample', type=int, default=128 << 20, help='elements of the CPU baseline sample; 0 skips it')
+    ap.add_argument('--cpu-sample', type=int, default=256 << 20, help='elements of the CPU baseline sample; 0 skips it')
     ap.add_argument('--blocks-per-cu', type=int, default=0,
                     help='cap on resident update workgroups per compute unit (0 = library default)')
     ap.add_argument('--calibrate-copy', type=float, default=0.0,
