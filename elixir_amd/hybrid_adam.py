@@ -304,14 +304,13 @@ class HybridAdam(torch.optim.Optimizer):
         if prep is None:
             return loss
 
-        for state in prep.states:    # commit: this step happens
-            state['step'] += 1
         plan = prep.dplan.plan
         stream = torch.cuda.current_stream(prep.device).cuda_stream
         events = self.kernel_events
         if prep.dplan.rows is not None:
             if events is not None:
-                events['adam_step'] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                if 'adam_step' not in events:    # created once, recorded again every step
+                    events['adam_step'] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
                 events['adam_step'][0].record()
             _abi.adam_step_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs), prep.d_hypers,
                               len(prep.hyper_host), plan.info, float(div_scale), prep.grad_code, prep.lowp_code,
@@ -319,11 +318,17 @@ class HybridAdam(torch.optim.Optimizer):
             if events is not None:
                 events['adam_step'][1].record()
         if prep.dplan.refresh is not None:
+            if events is not None:
+                if 'refresh' not in events:
+                    events['refresh'] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                events['refresh'][0].record()
             _abi.writeback_mt(prep.dplan.refresh.ptr, len(plan.refresh_rows), prep.lowp_code, plan.refresh_max_elems,
                               prep.dplan.refresh_aligned, stream)
             if events is not None:
-                events['refresh'] = (events['adam_step'][1], torch.cuda.Event(enable_timing=True))
                 events['refresh'][1].record()
+        # commit: this step happens (after the launches, so that the device is not kept waiting)
+        for state in prep.states:
+            state['step'] += 1
         if self._binding is not None and prep.lowp_code != _abi.ELX_NONE:
             self._binding.fused_writeback = True
         return loss

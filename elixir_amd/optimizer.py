@@ -66,15 +66,16 @@ class _EventPair:
 
     def __enter__(self):
         if self.sink is not None:
-            self.begin = torch.cuda.Event(enable_timing=True)
-            self.end = torch.cuda.Event(enable_timing=True)
+            pair = self.sink.get(self.key)
+            if pair is None:    # created once, recorded again every step: creating events is the costly part
+                pair = self.sink[self.key] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            self.begin, self.end = pair
             self.begin.record()
         return self
 
     def __exit__(self, *exc):
         if self.sink is not None:
             self.end.record()
-            self.sink[self.key] = (self.begin, self.end)
         return False
 
 
@@ -417,7 +418,7 @@ class ElixirOptimizer:
         self._set_grad_ptr()
         found_inf = self._check_overflow()
         self.last_step_info = dict(found_inf=found_inf, combined_scale=None, total_norm=None,
-                                   chunk_overflow=[bool(c.overflow) for c in self._param_chunk_list])
+                                   chunk_overflow=[c._overflow for c in self._param_chunk_list])
 
         if found_inf:
             if self._binding is not None:
@@ -432,10 +433,8 @@ class ElixirOptimizer:
         # get combined scale. combined scale = loss scale * clipping norm
         # so that gradient = gradient / combined scale
         combined_scale = self._get_combined_scale()
-        self.last_step_info['combined_scale'] = combined_scale
-        self.grad_scaler.update(found_inf)
-        self._clear_optim_states()
 
+        # the launch goes out first; the bookkeeping that does not feed it follows while it runs
         if not self.scaled_optimizer:
             assert combined_scale == -1, 'You should use an optimizer in the available list:\n' \
             f'{_AVAIL_OPTIM_LIST}'
@@ -444,6 +443,9 @@ class ElixirOptimizer:
             with self._timed('update'):
                 ret = self.optim.step(div_scale=combined_scale, *args, **kwargs)
 
+        self.last_step_info['combined_scale'] = combined_scale
+        self.grad_scaler.update(found_inf)
+        self._clear_optim_states()
         self.zero_grad()
         self._update_fp16_params()
         return ret
