@@ -318,7 +318,8 @@ __device__ __forceinline__ ElxChunk load_chunk_row(const ElxChunk *__restrict__ 
 }
 static_assert(sizeof(ElxChunk) == 72, "load_chunk_row reads nine 64-bit words");
 
-extern __shared__ char elx_occupancy_reservation[];    // never touched: it only caps residency
+// The update and landing launches pass a dynamic LDS size that no kernel ever touches: it only caps how
+// many workgroups share a compute unit (occupancy_reservation below).
 
 template <int GD, int LD>
 __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks, uint32_t n_chunks,
