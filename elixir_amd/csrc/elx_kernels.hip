@@ -7,6 +7,11 @@
 //                       fp64 accumulator; wave shuffle -> LDS -> one partial per workgroup;
 //                       a second tiny launch folds the partials in a fixed order)
 //   adam_step_kernel    unscale + Adam/AdamW on master/m/v + low-precision writeback, tile by tile
+//   refresh_kernel      the low-precision refresh alone (padding runs, skipped steps, state loading,
+//                       the gather source copy of a host-resident shard)
+//   land_grads_kernel   payload or per-tensor gradients -> shard (copy / cast), with the overflow
+//                       flag and sum of squares of what lands riding the copy; stats_fold_kernel and
+//                       stats_finish_kernel fold its per-workgroup partials
 //
 // Shape of the update launch, as measured on MI355X.  The update moves 14 B in and 14 B out per
 // element over four in-place regions.  HBM serves such a read/write mix best when the set of
