@@ -31,7 +31,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg',
            'elx_sizeof_hyper', 'elx_sizeof_stats', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
-           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems', 'elx_land_fold_blocks')
+           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_writeback', 'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems', 'elx_land_fold_blocks')
 
 
 class ElxError(RuntimeError):
@@ -75,6 +75,10 @@ def load() -> ctypes.CDLL:
     L.elx_writeback_mt.argtypes = [vp, u32, cint, u32, u32, vp]
     L.elx_land_tile_elems.restype = u32
     L.elx_land_tile_elems.argtypes = [cint]
+    L.elx_writeback.restype = cint
+    L.elx_writeback.argtypes = [vp, vp, cint, u64, vp]
+    L.elx_grad_stats.restype = cint
+    L.elx_grad_stats.argtypes = [vp, cint, u64, u32, vp, vp, vp]
     L.elx_check_land_rows.restype = cint
     L.elx_check_land_rows.argtypes = [vp, u32, vp, u32, cint, cint, ctypes.POINTER(u32)]
     L.elx_land_grads_mt.restype = cint
@@ -210,3 +214,13 @@ def check_land_rows(rows: np.ndarray, slot_offsets: Optional[np.ndarray], src_dt
           load().elx_check_land_rows(_np_ptr(rows), len(rows), _np_ptr(slot_offsets), n_slots, src_dtype, dst_dtype,
                                      ctypes.byref(bpr)))
     return int(bpr.value)
+
+
+def writeback(master: int, lowp: int, lowp_dtype: int, n: int, stream: int) -> None:
+    """One buffer: lowp[0, n) = cast(master[0, n))."""
+    check('elx_writeback', load().elx_writeback(master, lowp, lowp_dtype, n, stream))
+
+
+def grad_stats(grad: int, grad_dtype: int, n: int, blocks: int, d_partials: int, d_stats: int, stream: int) -> None:
+    """One buffer: overflow flag and sum of squares of grad[0, n)."""
+    check('elx_grad_stats', load().elx_grad_stats(grad, grad_dtype, n, blocks, d_partials, d_stats, stream))

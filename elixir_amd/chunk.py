@@ -581,13 +581,6 @@ class Chunk:
 
     # ------------------------------------------------------------------ gradient landing and flags
 
-    def _stats_row(self) -> np.ndarray:
-        row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
-        row['grad'] = self.shard.data_ptr()
-        row['n_alloc'] = self.shard_size
-        row['n_valid'] = self.n_valid
-        return row
-
     def set_overflow_flag(self, valid_tensor: Optional[torch.Tensor] = None) -> None:
         """chunk.py:214-216; here both flags come from one pass over ``shard[:valid_end]``."""
         assert not self._stats_pending and not self._overflow
@@ -598,8 +591,15 @@ class Chunk:
         self._compute_stats()
 
     def _compute_stats(self) -> None:
-        stats = run_grad_stats(self._stats_row(), dtype_code(self.chunk_dtype), kernel_device([self.shard]),
-                               workspace=self._workspace)
+        device = kernel_device([self.shard])
+        blocks = stats_launch_blocks(self.n_valid)
+        rec = _abi.STATS_DTYPE.itemsize
+        buf = self._workspace.get('stats_one')
+        if buf is None or buf.numel() < (blocks + 1) * rec or buf.device != device:
+            buf = self._workspace['stats_one'] = torch.empty((blocks + 1) * rec, dtype=torch.uint8, device=device)
+        _abi.grad_stats(self.shard.data_ptr(), dtype_code(self.chunk_dtype), self.n_valid, blocks, buf.data_ptr(),
+                        buf.data_ptr() + blocks * rec, torch.cuda.current_stream(device).cuda_stream)
+        stats = read_grad_stats(buf[blocks * rec:(blocks + 1) * rec])
         self._apply_stats(bool(stats['overflow'][0]), float(stats['sumsq'][0]))
 
     def _apply_stats(self, overflow: bool, sumsq: float) -> None:
@@ -648,21 +648,8 @@ class Chunk:
         assert self.shard_device.type == friend_chunk.shard_device.type
 
         if self.shard_device.type == 'cuda':
-            row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
-            row['lowp_out'] = self.shard.data_ptr()
-            row['master'] = friend_chunk.shard.data_ptr()
-            # m and v are not touched by the refresh; the table check wants non-NULL pointers
-            row['m'] = friend_chunk.shard.data_ptr()
-            row['v'] = friend_chunk.shard.data_ptr()
-            row['n_alloc'] = self.shard_size
-            row['n_valid'] = self.n_valid
-            code = dtype_code(self.chunk_dtype)
-            info = _abi.check_tables(row, None, 0, code, code)
-            table = DeviceTable(row, self.shard_device)
-            stream = torch.cuda.current_stream(self.shard_device).cuda_stream
-            _abi.writeback_mt(table.ptr, 1, code, self.shard_size, info.aligned, stream)
-            # keep the table alive until the launch has consumed it
-            self._workspace['wb_table'] = table
+            _abi.writeback(friend_chunk.shard.data_ptr(), self.shard.data_ptr(), dtype_code(self.chunk_dtype),
+                           self.shard_size, torch.cuda.current_stream(self.shard_device).cuda_stream)
             self.optim_sync_flag = True
         elif self.shard_device.type == 'cpu':
             # the refresh is deferred to the next gather of this chunk
@@ -678,16 +665,8 @@ class Chunk:
         assert dst.is_cuda and dst.is_contiguous() and dst.numel() == master.numel() == self.shard_size
         assert master.dtype == torch.float32 and master.is_contiguous()
         assert master.is_cuda or master.is_pinned(), 'the kernel can only read device or pinned host memory'
-        row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
-        row['lowp_out'] = dst.data_ptr()
-        row['master'] = row['m'] = row['v'] = master.data_ptr()
-        row['n_alloc'] = self.shard_size
-        row['n_valid'] = self.n_valid
-        code = dtype_code(self.chunk_dtype)
-        info = _abi.check_tables(row, None, 0, code, code)
-        table = DeviceTable(row, dst.device)
-        _abi.writeback_mt(table.ptr, 1, code, self.shard_size, info.aligned, torch.cuda.current_stream(dst.device).cuda_stream)
-        self._workspace['gather_table'] = table    # alive until the launch has consumed it
+        _abi.writeback(master.data_ptr(), dst.data_ptr(), dtype_code(self.chunk_dtype), self.shard_size,
+                       torch.cuda.current_stream(dst.device).cuda_stream)
 
     def replicate(self, payload: torch.Tensor) -> None:
         """chunk.py:264-270 + 475-482 on one process: fills this shard's slice of a replicated block

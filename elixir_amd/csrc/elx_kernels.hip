@@ -452,11 +452,9 @@ constexpr int kRefreshUnroll = 4;
 constexpr uint32_t kRefreshPiece = kRefreshThreads * kVec * kRefreshUnroll;
 
 template <int LD>
-__global__ __launch_bounds__(kRefreshThreads) void refresh_kernel(const ElxChunk *__restrict__ chunks,
-                                                                  uint32_t scalar_only) {
+__device__ __forceinline__ void refresh_body(const ElxChunk &c, uint32_t scalar_only) {
     typedef typename Elem<LD>::vec4 lvec;
     typedef typename Elem<LD>::scalar lscalar;
-    const ElxChunk c = chunks[blockIdx.y];
     if (!c.lowp_out) return;
     lscalar *out = reinterpret_cast<lscalar *>(c.lowp_out);
     const uint64_t n = c.n_alloc;
@@ -482,6 +480,19 @@ __global__ __launch_bounds__(kRefreshThreads) void refresh_kernel(const ElxChunk
             for (uint32_t i = threadIdx.x; i < cnt; i += kRefreshThreads) out[base + i] = Elem<LD>::from_f32(c.master[base + i]);
         }
     }
+}
+
+template <int LD>
+__global__ __launch_bounds__(kRefreshThreads) void refresh_kernel(const ElxChunk *__restrict__ chunks,
+                                                                  uint32_t scalar_only) {
+    const ElxChunk c = chunks[blockIdx.y];
+    refresh_body<LD>(c, scalar_only);
+}
+
+// One buffer, described in the kernel arguments: no table in device memory is needed.
+template <int LD>
+__global__ __launch_bounds__(kRefreshThreads) void refresh_one_kernel(ElxChunk c, uint32_t scalar_only) {
+    refresh_body<LD>(c, scalar_only);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -525,16 +536,14 @@ __device__ __forceinline__ void stats_elem(float x, float &acc, float &poison) {
 }
 
 template <int GD>
-__global__ __launch_bounds__(kStatsThreads) void grad_stats_kernel(const ElxChunk *__restrict__ chunks, uint32_t bpc,
-                                                                   ElxStats *__restrict__ partials,
-                                                                   uint32_t scalar_only) {
+__device__ __forceinline__ void grad_stats_body(const ElxChunk &c, uint32_t bpc, ElxStats *__restrict__ partials,
+                                                uint32_t scalar_only) {
     typedef typename Elem<GD>::scalar gscalar;
     constexpr uint32_t kEpl = 16 / sizeof(gscalar);    // elements per lane per 128-bit load
     constexpr uint32_t kSSpan = kStatsThreads * kEpl;
     constexpr uint32_t kSTile = kSSpan * kStatsUnroll;
     typedef gscalar gvec __attribute__((ext_vector_type(kEpl)));
 
-    const ElxChunk c = chunks[blockIdx.y];
     const gscalar *g = reinterpret_cast<const gscalar *>(c.grad);
     const uint64_t n = g ? c.n_valid : 0;
     const uint64_t n_tiles = (n + kSTile - 1) / kSTile;
@@ -570,6 +579,22 @@ __global__ __launch_bounds__(kStatsThreads) void grad_stats_kernel(const ElxChun
         r.reserved = 0;
         partials[(uint64_t)blockIdx.y * bpc + blockIdx.x] = r;
     }
+}
+
+template <int GD>
+__global__ __launch_bounds__(kStatsThreads) void grad_stats_kernel(const ElxChunk *__restrict__ chunks, uint32_t bpc,
+                                                                   ElxStats *__restrict__ partials,
+                                                                   uint32_t scalar_only) {
+    const ElxChunk c = chunks[blockIdx.y];
+    grad_stats_body<GD>(c, bpc, partials, scalar_only);
+}
+
+// One buffer, described in the kernel arguments.
+template <int GD>
+__global__ __launch_bounds__(kStatsThreads) void grad_stats_one_kernel(ElxChunk c, uint32_t bpc,
+                                                                       ElxStats *__restrict__ partials,
+                                                                       uint32_t scalar_only) {
+    grad_stats_body<GD>(c, bpc, partials, scalar_only);
 }
 
 __global__ __launch_bounds__(kStatsThreads) void stats_finish_kernel(const ElxStats *__restrict__ partials,
@@ -984,6 +1009,51 @@ int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype
 }
 
 uint32_t elx_refresh_piece_elems(void) { return kRefreshPiece; }
+
+int elx_writeback(const float *master, void *lowp, int lowp_dtype, uint64_t n, void *stream) {
+    if (!master || !lowp) return ELX_E_NULL;
+    if (!is_lowp_or_f32(lowp_dtype)) return ELX_E_DTYPE;
+    if (n == 0) return ELX_E_SIZE;
+    if (((uintptr_t)master & 3u) || ((uintptr_t)lowp & (elem_size(lowp_dtype) - 1))) return ELX_E_ALIGN;
+    ElxChunk c = {};
+    c.lowp_out = lowp;
+    c.master = const_cast<float *>(master);
+    c.n_alloc = n;
+    const uint32_t so = (((uintptr_t)master | (uintptr_t)lowp) & 15u) ? 1u : 0u;
+    const uint64_t pieces = (n + kRefreshPiece - 1) / kRefreshPiece;
+    const dim3 grid((uint32_t)(pieces < 4096 ? pieces : 4096));
+    hipStream_t st = (hipStream_t)stream;
+    switch (lowp_dtype) {
+        case ELX_F32: hipLaunchKernelGGL((refresh_one_kernel<ELX_F32>), grid, dim3(kRefreshThreads), 0, st, c, so); break;
+        case ELX_F16: hipLaunchKernelGGL((refresh_one_kernel<ELX_F16>), grid, dim3(kRefreshThreads), 0, st, c, so); break;
+        default: hipLaunchKernelGGL((refresh_one_kernel<ELX_BF16>), grid, dim3(kRefreshThreads), 0, st, c, so); break;
+    }
+    return (int)hipGetLastError();
+}
+
+int elx_grad_stats(const void *grad, int grad_dtype, uint64_t n, uint32_t blocks, ElxStats *d_partials,
+                   ElxStats *d_stats, void *stream) {
+    if (!d_partials || !d_stats || (!grad && n)) return ELX_E_NULL;
+    if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
+    if (blocks == 0 || blocks > kMaxStatsBlocks) return ELX_E_SIZE;
+    if ((uintptr_t)grad & (elem_size(grad_dtype) - 1)) return ELX_E_ALIGN;
+    ElxChunk c = {};
+    c.grad = grad;
+    c.n_alloc = n;
+    c.n_valid = n;
+    const uint32_t so = ((uintptr_t)grad & 15u) ? 1u : 0u;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid(blocks);
+    switch (grad_dtype) {
+        case ELX_F32: hipLaunchKernelGGL((grad_stats_one_kernel<ELX_F32>), grid, dim3(kStatsThreads), 0, st, c, blocks, d_partials, so); break;
+        case ELX_F16: hipLaunchKernelGGL((grad_stats_one_kernel<ELX_F16>), grid, dim3(kStatsThreads), 0, st, c, blocks, d_partials, so); break;
+        default: hipLaunchKernelGGL((grad_stats_one_kernel<ELX_BF16>), grid, dim3(kStatsThreads), 0, st, c, blocks, d_partials, so); break;
+    }
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    hipLaunchKernelGGL(stats_finish_kernel, dim3(1), dim3(kStatsThreads), 0, st, d_partials, blocks, d_stats);
+    return (int)hipGetLastError();
+}
 
 int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d_slot_offsets, uint32_t n_slots,
                       int src_dtype, int dst_dtype, float mul, uint32_t blocks_per_row, ElxStats *d_partials,

@@ -197,6 +197,19 @@ int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype
 uint32_t elx_refresh_piece_elems(void);
 
 /*
+ * The same two passes for ONE buffer described in the arguments: no table in device memory.
+ *   elx_writeback   lowp[0, n) = round-to-nearest-even(master[0, n)): Chunk.optim_update for one chunk
+ *                   (chunk.py:403-414) and the source copy of a gather whose refresh was deferred
+ *                   (chunk.py:264-270, 475-482); `master` may be pinned host memory
+ *   elx_grad_stats  flags of grad[0, n): Chunk.set_overflow_flag / set_l2_norm for one chunk
+ *                   (chunk.py:214-221); blocks = 1..1024 workgroups, d_partials holds `blocks`
+ *                   records, *d_stats receives the result
+ */
+int elx_writeback(const float *master, void *lowp, int lowp_dtype, uint64_t n, void *stream);
+int elx_grad_stats(const void *grad, int grad_dtype, uint64_t n, uint32_t blocks, ElxStats *d_partials,
+                   ElxStats *d_stats, void *stream);
+
+/*
  * Gradient landing with the stats riding the copy: for every row
  *   lowp_out[i] = cast_dst(grad[i])                          for i in [0, n_alloc)
  * and d_stats[row] = overflow flag and sum of squares of lowp_out[0, n_valid) as stored.  Replaces the

@@ -604,3 +604,40 @@ def test_full_range_values_match_the_oracle(oracle, gdtype, div_scale):
             assert np.array_equal(np.isnan(got), nan), (name, adamw)
             bad = got.view(np.uint32)[~nan] != want.view(np.uint32)[~nan]
             assert not bad.any(), (name, adamw, int(bad.sum()), got[~nan][bad][:4], want[~nan][bad][:4])
+
+
+# ------------------------------------------------------------------------------------------------
+# the single-buffer entry points
+# ------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('n,offset', [(1, 0), (4097, 0), ((1 << 20) + 5, 0), (70001, 1)])
+def test_single_buffer_stats_and_writeback(oracle, dtype, n, offset):
+    """elx_grad_stats / elx_writeback take one buffer in their arguments (no table in device memory):
+    the same results as the oracle, aligned or not."""
+    gen = torch.Generator(device=DEV).manual_seed(n)
+    g = (torch.randn(n + offset, generator=gen, device=DEV) * 2.0).to(dtype)[offset:]
+    rec = _abi.STATS_DTYPE.itemsize
+    stream = torch.cuda.current_stream().cuda_stream
+    for blocks in (1, 7, 1024):
+        ws = torch.empty((blocks + 1) * rec, dtype=torch.uint8, device=DEV)
+        _abi.grad_stats(g.data_ptr(), CODE[dtype], n, blocks, ws.data_ptr(), ws.data_ptr() + blocks * rec, stream)
+        out = ws[blocks * rec:].cpu().numpy().view(_abi.STATS_DTYPE)
+        want = oracle.sumsq(to_np(g), CODE[dtype])
+        assert out['overflow'][0] == 0 and abs(out['sumsq'][0] - want) <= 1e-6 * want
+    g2 = g.clone()
+    g2[n // 2] = float('inf')
+    ws = torch.empty(5 * rec, dtype=torch.uint8, device=DEV)
+    _abi.grad_stats(g2.data_ptr(), CODE[dtype], n, 4, ws.data_ptr(), ws.data_ptr() + 4 * rec, stream)
+    assert ws[4 * rec:].cpu().numpy().view(_abi.STATS_DTYPE)['overflow'][0] == 1
+
+    master = torch.randn(n + offset, generator=gen, device=DEV)[offset:] * 100.0
+    lowp = torch.zeros(n + offset, dtype=dtype, device=DEV)[offset:]
+    _abi.writeback(master.data_ptr(), lowp.data_ptr(), CODE[dtype], n, stream)
+    want = oracle.writeback(to_np(master), CODE[dtype])
+    assert np.array_equal(to_np(lowp).view(np.uint8), want.view(np.uint8))
+    with pytest.raises(_abi.ElxError):
+        _abi.writeback(0, lowp.data_ptr(), CODE[dtype], n, stream)
+    with pytest.raises(_abi.ElxError):
+        _abi.grad_stats(g.data_ptr(), CODE[dtype], n, 2000, ws.data_ptr(), ws.data_ptr(), stream)
