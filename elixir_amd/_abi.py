@@ -23,15 +23,19 @@ CHUNK_DTYPE = np.dtype([('grad', '<u8'), ('lowp_out', '<u8'), ('master', '<u8'),
 SEG_DTYPE = np.dtype([('begin', '<u8'), ('end', '<u8'), ('hyper', '<u4'), ('reserved', '<u4')])
 HYPER_DTYPE = np.dtype([('decay_mul', '<f4'), ('l2_wd', '<f4'), ('lerp_w', '<f4'), ('beta2', '<f4'), ('omb2', '<f4'),
                         ('bc2_sqrt', '<f4'), ('eps', '<f4'), ('neg_step', '<f4'), ('flags', '<u4'),
-                        ('reserved', '<u4', (3,))])
+                        ('gate_div_scale', '<f4'), ('gate_inv_scale', '<f4'), ('gate', '<u4')])
 STATS_DTYPE = np.dtype([('sumsq', '<f8'), ('overflow', '<u4'), ('reserved', '<u4')])
+DECISION_DTYPE = np.dtype([('div_scale', '<f4'), ('inv_scale', '<f4'), ('mode', '<u4'), ('skip', '<u4'),
+                           ('total_norm', '<f8'), ('combined_scale', '<f8')])
 
 LIB_NAME = 'libelx_hip.so'
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
-EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg',
-           'elx_sizeof_hyper', 'elx_sizeof_stats', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
-           'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_writeback', 'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems', 'elx_land_fold_blocks')
+EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper',
+           'elx_sizeof_stats', 'elx_sizeof_decision', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
+           'elx_decide', 'elx_adam_step_gated_mt', 'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_writeback',
+           'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems',
+           'elx_land_fold_blocks')
 
 
 class ElxError(RuntimeError):
@@ -61,6 +65,7 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
+                 'elx_sizeof_decision', 'elx_sizeof_decision', 'elx_decide', 'elx_adam_step_gated_mt',
                  'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
@@ -71,6 +76,10 @@ def load() -> ctypes.CDLL:
     L.elx_grad_stats_mt.argtypes = [vp, u32, cint, u32, vp, vp, cint, vp]
     L.elx_adam_step_mt.restype = cint
     L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
+    L.elx_decide.restype = cint
+    L.elx_decide.argtypes = [vp, u32, ctypes.c_double, ctypes.c_double, cint, vp, u32, vp, vp]
+    L.elx_adam_step_gated_mt.restype = cint
+    L.elx_adam_step_gated_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, cint, cint, u32, u32, vp]
     L.elx_writeback_mt.restype = cint
     L.elx_writeback_mt.argtypes = [vp, u32, cint, u32, u32, vp]
     L.elx_land_tile_elems.restype = u32
@@ -162,6 +171,21 @@ def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hyper
     check('elx_adam_step_mt',
           load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles, grid_tiles,
                                   div_scale, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
+
+
+def decide(d_stats: int, n_chunks: int, loss_scale: float, max_norm: float, clipping: bool, d_hypers: int,
+           n_hypers: int, d_decision: int, stream: int) -> None:
+    check('elx_decide',
+          load().elx_decide(d_stats, n_chunks, loss_scale, max_norm, int(clipping), d_hypers, n_hypers, d_decision, stream))
+
+
+def adam_step_gated_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int,
+                       info: TableInfo, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int, stream: int) -> None:
+    """``adam_step_mt`` with the unscale parameters and the skip flag read from the hyper records."""
+    grid_tiles = 0 if n_chunks > 65535 else info.max_tiles
+    check('elx_adam_step_gated_mt',
+          load().elx_adam_step_gated_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles,
+                                        grid_tiles, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
 
 
 def refresh_piece_elems() -> int:

@@ -144,10 +144,22 @@ struct TileIo<u16x4> {
 struct Hyper {
     float decay_mul, l2_wd, lerp_w, beta2, omb2, bc2_sqrt, eps, neg_step;
     uint32_t flags;
+    float gate_div, gate_inv;    // only loaded by the gated launch
+    uint32_t gate;               // mode | skip << 8
 };
 
+template <bool GATED = false>
 __device__ __forceinline__ Hyper load_hyper(const ElxHyper *__restrict__ h) {
     Hyper r;
+    if constexpr (GATED) {
+        r.gate_div = h->gate_div_scale;
+        r.gate_inv = h->gate_inv_scale;
+        r.gate = h->gate;
+    } else {
+        r.gate_div = -1.0f;
+        r.gate_inv = 1.0f;
+        r.gate = 0;
+    }
     r.decay_mul = h->decay_mul;
     r.l2_wd = h->l2_wd;
     r.lerp_w = h->lerp_w;
@@ -273,10 +285,10 @@ __device__ __forceinline__ void tile_refresh_vec(const ElxChunk &c, uint64_t bas
 // Any tile: element by element, each element looking up the segment that covers it.  Used for
 // tiles that straddle a segment boundary, the partial tile at the end of a chunk, and buffers
 // whose base pointers are not 16-byte aligned.  `s` is the first segment whose end is > base.
-template <int GD, int LD>
+template <int GD, int LD, bool GATED>
 __device__ __forceinline__ void tile_scalar(const ElxChunk &c, uint64_t base, uint32_t tile_n, uint32_t s,
                                             const ElxSeg *__restrict__ segs, const ElxHyper *__restrict__ hypers,
-                                            const Unscale &us, bool refresh_only) {
+                                            const Unscale &us_arg, bool refresh_only) {
     typedef typename Elem<GD>::scalar gscalar;
     const gscalar *grad = reinterpret_cast<const gscalar *>(c.grad);
     for (uint32_t i = threadIdx.x; i < tile_n; i += kWave) {
@@ -286,13 +298,23 @@ __device__ __forceinline__ void tile_scalar(const ElxChunk &c, uint64_t base, ui
             uint32_t cs = s;
             while (cs < c.seg_end && segs[cs].end <= e) ++cs;
             if (cs < c.seg_end && segs[cs].begin <= e) {
-                const Hyper h = load_hyper(hypers + segs[cs].hyper);
-                float g = grad ? Elem<GD>::to_f32(grad[e]) : 0.0f;
-                float m = c.m[e], v = c.v[e];
-                adam_elem(g, p, m, v, h, us);
-                c.master[e] = p;
-                c.m[e] = m;
-                c.v[e] = v;
+                const Hyper h = load_hyper<GATED>(hypers + segs[cs].hyper);
+                Unscale us = us_arg;
+                bool skip = false;
+                if constexpr (GATED) {
+                    us.div_scale = h.gate_div;
+                    us.inv_scale = h.gate_inv;
+                    us.mode = (int)(h.gate & 0xFFu);
+                    skip = (h.gate >> 8) != 0;
+                }
+                if (!skip) {
+                    float g = grad ? Elem<GD>::to_f32(grad[e]) : 0.0f;
+                    float m = c.m[e], v = c.v[e];
+                    adam_elem(g, p, m, v, h, us);
+                    c.master[e] = p;
+                    c.m[e] = m;
+                    c.v[e] = v;
+                }
             }
         }
         if constexpr (LD != ELX_NONE) {
@@ -326,7 +348,11 @@ static_assert(sizeof(ElxChunk) == 72, "load_chunk_row reads nine 64-bit words");
 // The update and landing launches pass a dynamic LDS size that no kernel ever touches: it only caps how
 // many workgroups share a compute unit (occupancy_reservation below).
 
-template <int GD, int LD>
+// GATED: the unscale parameters and the skip flag are read from the hyper records (where elx_decide
+// has put them earlier on the same stream) instead of the kernel arguments, so that the launch can be
+// enqueued before the host knows whether the step happens.  They arrive with the hyper record the
+// tile loads anyway; on a skip the tile only refreshes its low-precision copy.
+template <int GD, int LD, bool GATED>
 __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks, uint32_t n_chunks,
                                                           const ElxSeg *__restrict__ segs,
                                                           const ElxHyper *__restrict__ hypers,
@@ -395,7 +421,16 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
         const uint64_t sb = has ? segs[s].begin : ~0ull;
         const uint64_t se = has ? segs[s].end : 0ull;
         if (has && sb <= base && se >= base + kTile) {
-            const Hyper h = load_hyper(hypers + segs[s].hyper);
+            const Hyper h = load_hyper<GATED>(hypers + segs[s].hyper);
+            if constexpr (GATED) {
+                us.div_scale = h.gate_div;
+                us.inv_scale = h.gate_inv;
+                us.mode = (int)(h.gate & 0xFFu);
+                if (h.gate >> 8) {    // the step is skipped: refresh the low-precision copy only
+                    store_lowp_vec<LD>(c, base, P);
+                    return;
+                }
+            }
             if (us.mode == kDivMulInv)
                 tile_math_flags<GD, kDivMulInv>(G, P, M, V, h, us);
             else if (us.mode == kDivTrue)
@@ -426,7 +461,7 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
         if (tile_n == kTile && !scalar_only)
             tile_refresh_vec<LD>(c, base);
         else
-            tile_scalar<GD, LD>(c, base, tile_n, 0, segs, hypers, us, true);
+            tile_scalar<GD, LD, GATED>(c, base, tile_n, 0, segs, hypers, us, true);
         return;
     }
     uint32_t s = c.seg_begin, s_hi = c.seg_end;
@@ -437,7 +472,7 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
         else
             s = mid + 1;
     }
-    tile_scalar<GD, LD>(c, base, tile_n, s, segs, hypers, us, false);
+    tile_scalar<GD, LD, GATED>(c, base, tile_n, s, segs, hypers, us, false);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -790,6 +825,62 @@ __global__ __launch_bounds__(kStatsThreads) void stats_fold_kernel(const ElxStat
 }
 
 // ---------------------------------------------------------------------------------------------
+// the decisions of the step, on the device
+// ---------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ bool exact_reciprocal_dev(float s) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, s);
+    const uint32_t exp = (u >> 23) & 0xFFu, man = u & 0x7FFFFFu;
+    return (u >> 31) == 0 && man == 0 && exp >= 1 && exp <= 252;
+}
+
+// elixir/wrapper/optimizer.py:137-183 in the float64 arithmetic the host uses, one thread: any
+// overflow -> skip; otherwise the combined scale = loss scale (x clip coefficient when the global
+// norm exceeds max_norm).  Per chunk the squared norm passes through an fp32 norm
+// (chunk.py:218-221), the sum over chunks through an fp32 buffer (optimizer.py:158-162).  The
+// result goes into *out and into the gate words of every hyper record.
+__global__ void decide_kernel(const ElxStats *__restrict__ stats, uint32_t n, double loss_scale, double max_norm,
+                              int clipping, ElxHyper *__restrict__ hypers, uint32_t n_hypers,
+                              ElxDecision *__restrict__ out) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    uint32_t found = 0;
+    double norm_sqr = 0.0;
+    for (uint32_t i = 0; i < n; ++i) {
+        found |= stats[i].overflow;
+        const float nrm = (float)sqrt(stats[i].sumsq);
+        norm_sqr += (double)nrm * (double)nrm;
+    }
+    ElxDecision d;
+    d.skip = found ? 1u : 0u;
+    d.total_norm = 0.0;
+    double combined = loss_scale;
+    if (clipping) {
+        d.total_norm = sqrt((double)(float)norm_sqr);
+        const double clip = ((d.total_norm / loss_scale) + 1e-6) / max_norm;
+        if (clip > 1.0) combined = clip * loss_scale;
+    }
+    if (combined == 1.0) combined = -1.0;
+    d.combined_scale = combined;
+    d.div_scale = (float)combined;
+    d.inv_scale = 1.0f;
+    d.mode = kDivNone;
+    if (d.div_scale > 0.0f) {
+        if (exact_reciprocal_dev(d.div_scale)) {
+            d.mode = kDivMulInv;
+            d.inv_scale = 1.0f / d.div_scale;
+        } else {
+            d.mode = kDivTrue;
+        }
+    }
+    *out = d;
+    for (uint32_t i = 0; i < n_hypers; ++i) {
+        hypers[i].gate_div_scale = d.div_scale;
+        hypers[i].gate_inv_scale = d.inv_scale;
+        hypers[i].gate = d.mode | (d.skip << 8);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side of the ABI
 // ---------------------------------------------------------------------------------------------
 
@@ -815,19 +906,24 @@ int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes) {
 
 template <int GD, int LD>
 int launch_step(uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
-                const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, uint32_t scalar_only) {
+                const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated,
+                uint32_t scalar_only) {
     const dim3 grid = grid_tiles ? dim3(grid_tiles, n_chunks) : dim3(tiles);
-    hipLaunchKernelGGL((adam_step_kernel<GD, LD>), grid, dim3(kWave), lds, st, chunks, n_chunks, segs, hypers,
-                       grid_tiles, us, scalar_only);
+    if (gated)
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true>), grid, dim3(kWave), lds, st, chunks, n_chunks, segs, hypers,
+                           grid_tiles, us, scalar_only);
+    else
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false>), grid, dim3(kWave), lds, st, chunks, n_chunks, segs, hypers,
+                           grid_tiles, us, scalar_only);
     return (int)hipGetLastError();
 }
 
 int dispatch_step(int gd, int ld, uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks,
                   uint32_t n_chunks, const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us,
-                  uint32_t scalar_only) {
+                  bool gated, uint32_t scalar_only) {
 #define ELX_CASE(G, L)                                                                                         \
     if (gd == G && ld == L)                                                                                    \
-        return launch_step<G, L>(tiles, lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, scalar_only);
+        return launch_step<G, L>(tiles, lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -849,6 +945,7 @@ uint32_t elx_sizeof_chunk(void) { return (uint32_t)sizeof(ElxChunk); }
 uint32_t elx_sizeof_seg(void) { return (uint32_t)sizeof(ElxSeg); }
 uint32_t elx_sizeof_hyper(void) { return (uint32_t)sizeof(ElxHyper); }
 uint32_t elx_sizeof_stats(void) { return (uint32_t)sizeof(ElxStats); }
+uint32_t elx_sizeof_decision(void) { return (uint32_t)sizeof(ElxDecision); }
 
 const char *elx_strerror(int code) {
     switch (code) {
@@ -989,7 +1086,37 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
         }
     }
     return dispatch_step(grad_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
-                         d_segs, d_hypers, grid_tiles_per_chunk, us, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+                         d_segs, d_hypers, grid_tiles_per_chunk, us, false, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+}
+
+int elx_decide(const ElxStats *d_stats, uint32_t n_chunks, double loss_scale, double max_norm, int clipping,
+               ElxHyper *d_hypers, uint32_t n_hypers, ElxDecision *d_decision, void *stream) {
+    if (!d_stats || !d_decision || (n_hypers && !d_hypers)) return ELX_E_NULL;
+    if (n_chunks == 0) return ELX_E_SIZE;
+    if (!(loss_scale > 0.0) || (clipping && !(max_norm > 0.0))) return ELX_E_RANGE;
+    hipLaunchKernelGGL(decide_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, d_stats, n_chunks, loss_scale, max_norm,
+                       clipping, d_hypers, n_hypers, d_decision);
+    return (int)hipGetLastError();
+}
+
+int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
+                           const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,
+                           uint32_t grid_tiles_per_chunk, int grad_dtype, int lowp_dtype, uint32_t flags,
+                           uint32_t blocks_per_cu, void *stream) {
+    if (!d_chunks || (n_segs && (!d_segs || !d_hypers))) return ELX_E_NULL;
+    if (n_chunks == 0 || n_chunks > 65535u || total_tiles == 0 || total_tiles > 0x7FFFFFFFull || (n_segs && n_hypers == 0))
+        return ELX_E_SIZE;
+    if (grid_tiles_per_chunk && (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
+    if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
+    if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    uint32_t lds = 0;
+    if (int rc = occupancy_reservation(blocks_per_cu, &lds)) return rc;
+    Unscale us;
+    us.div_scale = -1.0f;
+    us.inv_scale = 1.0f;
+    us.mode = kDivNone;
+    return dispatch_step(grad_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
+                         d_segs, d_hypers, grid_tiles_per_chunk, us, true, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
 int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype, uint32_t blocks_per_chunk,

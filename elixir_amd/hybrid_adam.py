@@ -213,6 +213,7 @@ class HybridAdam(torch.optim.Optimizer):
         self._plans: Dict = {}                      # plan key -> _DevicePlan
         self._hyper_uploader = _HyperUploader()
         self._prepared: Optional[_Prepared] = None
+        self._launched: Optional[_Prepared] = None   # launched with defer_commit, not yet committed or aborted
         self._bound_entries = None                  # cached walk over the bound fake parameters
         # when set to a dict, step() records (begin, end) torch.cuda.Event pairs under 'adam_step' and 'refresh'
         self.kernel_events = None
@@ -293,7 +294,11 @@ class HybridAdam(torch.optim.Optimizer):
         ])
 
     @torch.no_grad()
-    def step(self, closure=None, div_scale: float = -1):
+    def step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
+        """``gated``: the unscale parameters and the skip flag are read on the device from the gate
+        words of the prepared hyper table, where ``elx_decide`` has put them (``div_scale`` is then
+        ignored).  ``defer_commit``: launch only; the caller finishes with ``commit_step()`` once it
+        knows that the step happened, or ``abort_step()`` when the device decided to skip."""
         loss = None
         if closure is not None:
             with torch.enable_grad():
@@ -312,9 +317,14 @@ class HybridAdam(torch.optim.Optimizer):
                 if 'adam_step' not in events:    # created once, recorded again every step
                     events['adam_step'] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
                 events['adam_step'][0].record()
-            _abi.adam_step_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs), prep.d_hypers,
-                              len(prep.hyper_host), plan.info, float(div_scale), prep.grad_code, prep.lowp_code,
-                              self.blocks_per_cu, stream)
+            if gated:
+                _abi.adam_step_gated_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs),
+                                        prep.d_hypers, len(prep.hyper_host), plan.info, prep.grad_code,
+                                        prep.lowp_code, self.blocks_per_cu, stream)
+            else:
+                _abi.adam_step_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs),
+                                  prep.d_hypers, len(prep.hyper_host), plan.info, float(div_scale), prep.grad_code,
+                                  prep.lowp_code, self.blocks_per_cu, stream)
             if events is not None:
                 events['adam_step'][1].record()
         if prep.dplan.refresh is not None:
@@ -326,12 +336,28 @@ class HybridAdam(torch.optim.Optimizer):
                               prep.dplan.refresh_aligned, stream)
             if events is not None:
                 events['refresh'][1].record()
-        # commit: this step happens (after the launches, so that the device is not kept waiting)
+        self._launched = prep
+        if not defer_commit:
+            self.commit_step()
+        return loss
+
+    def commit_step(self) -> None:
+        """The launched step happened: step counts advance (after the launches, so that the device is
+        not kept waiting for host bookkeeping)."""
+        prep, self._launched = self._launched, None
+        if prep is None:
+            return
         for state in prep.states:
             state['step'] += 1
         if self._binding is not None and prep.lowp_code != _abi.ELX_NONE:
             self._binding.fused_writeback = True
-        return loss
+
+    def abort_step(self) -> None:
+        """The launched step found the skip flag set on the device: nothing was updated and no step
+        count advances; the launches refreshed every low-precision element they cover."""
+        prep, self._launched = self._launched, None
+        if prep is not None and self._binding is not None and prep.lowp_code != _abi.ELX_NONE:
+            self._binding.fused_writeback = True
 
     # ---- bound to chunk storage
 

@@ -33,7 +33,7 @@ import torch
 from torch.nn import Parameter
 
 from . import _abi
-from .chunk import (Chunk, DeviceTable, dtype_code, kernel_device, launch_grad_stats, read_grad_stats,
+from .chunk import (Chunk, DeviceTable, StatsArena, dtype_code, kernel_device, launch_grad_stats, read_grad_stats,
                     resolve_pending_stats)
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
 from .hybrid_adam import HybridAdam
@@ -154,6 +154,10 @@ class ElixirOptimizer:
                 self._binding = self.optim.bind_chunks(ranges)
         self._stats_table = None
         self._stats_workspace: Dict = {}
+        # the step decided on the device (no wait between the flags and the update); False: the host
+        # fetches the flags, decides and only then launches
+        self.gated_step = True
+        self._gate = None
         self._wb_table = None
         self.last_step_info: Dict = {}
         # when set to a dict, step() records (begin, end) torch.cuda.Event pairs on the launch
@@ -377,7 +381,7 @@ class ElixirOptimizer:
         """optimizer.py:149-164 on one process: the per-group sum passes through a one-element fp32
         buffer before the square root."""
         group_to_norm = defaultdict(float)
-        for param_chunk in self.param_chunk_set:
+        for param_chunk in self._param_chunk_list:    # a fixed order: float64 sums depend on it
             assert param_chunk.l2_norm is not None
             assert not param_chunk.is_replica
             group_to_norm[param_chunk.torch_pg] += param_chunk.l2_norm
@@ -409,8 +413,106 @@ class ElixirOptimizer:
 
     # ------------------------------------------------------------------ the step
 
+    # ------------------------------------------------------------------ the step, decided on the device
+
+    def _gate_buffers(self, device: torch.device, n_chunks: int):
+        g = self._gate
+        if g is None or g['device'] != device or g['host'].numel() < n_chunks * _abi.STATS_DTYPE.itemsize + 32:
+            g = self._gate = dict(device=device, decision=torch.zeros(32, dtype=torch.uint8, device=device),
+                                  host=torch.zeros(n_chunks * _abi.STATS_DTYPE.itemsize + 32, dtype=torch.uint8,
+                                                   pin_memory=True),
+                                  side=torch.cuda.Stream(device), copied=torch.cuda.Event())
+        return g
+
+    def _records_of_all_chunks(self, launched):
+        """The address of ONE run of ElxStats records that covers every parameter chunk in list order,
+        or None: either this step's stats launch covered them all, or fused landings left them all
+        in consecutive arena slots."""
+        chunks = self._param_chunk_list
+        if launched is not None:
+            pending, records = launched
+            return records if len(pending) == len(chunks) else None
+        if not chunks or not all(c._stats_pending for c in chunks):
+            return None
+        first = chunks[0]._stats_slot
+        if any(c._stats_slot != first + i for i, c in enumerate(chunks)):
+            return None
+        device = kernel_device(c.shard for c in chunks)
+        main = torch.cuda.current_stream(device)
+        for event in {c._stats_event for c in chunks if c._stats_event is not None}:
+            main.wait_event(event)    # the landings may have run on another stream
+        arena = StatsArena.get(chunks[0].shard_device)
+        rec = arena.itemsize
+        return arena.buf[first * rec:(first + len(chunks)) * rec]
+
+    def _step_gated(self, launched, records) -> bool:
+        """The step without a wait between the flags and the update: the decisions of
+        optimizer.py:137-183 are taken by a one-thread kernel that leaves them in the hyper table of
+        the update launch; the update is enqueued at once and reads them there (on a skip it only
+        refreshes the low-precision copies).  The flags and the decision travel to the host on a side
+        stream meanwhile, for the host's bookkeeping (scaler, step counts, chunk flags).  Returns False
+        when nothing was prepared to launch."""
+        inner = self.optim
+        prep = inner._prepared
+        if prep is None or prep.dplan.rows is None:
+            return False
+        chunks = self._param_chunk_list
+        n, rec = len(chunks), _abi.STATS_DTYPE.itemsize
+        g = self._gate_buffers(prep.device, n)
+        main = torch.cuda.current_stream(prep.device)
+        _abi.decide(records.data_ptr(), n, float(self.loss_scale), float(self.max_norm), self.clipping_flag,
+                    prep.d_hypers, len(prep.hyper_host), g['decision'].data_ptr(), main.cuda_stream)
+        decided = torch.cuda.Event()
+        decided.record(main)
+        with self._timed('update'):
+            inner.step(gated=True, defer_commit=True)
+
+        side = g['side']
+        side.wait_event(decided)
+        with torch.cuda.stream(side):
+            g['host'][:n * rec].copy_(records, non_blocking=True)
+            g['host'][n * rec:n * rec + 32].copy_(g['decision'], non_blocking=True)
+            g['copied'].record(side)
+        g['copied'].synchronize()
+        host = g['host'].numpy()
+        stats = host[:n * rec].view(_abi.STATS_DTYPE)
+        device_says = host[n * rec:n * rec + 32].view(_abi.DECISION_DTYPE)[0]
+        for c, r in zip(chunks, stats):
+            c._stats_pending = False
+            c._stats_event = None
+            c._apply_stats(bool(r['overflow']), float(r['sumsq']))
+
+        # what the device decided is what happened: the host records it
+        found_inf = bool(device_says['skip'])
+        assert found_inf == self._check_overflow()
+        self.last_step_info = dict(found_inf=found_inf, combined_scale=None, total_norm=None,
+                                   chunk_overflow=[c._overflow for c in chunks])
+        assert self.optim_state == OptimState.SCALED or found_inf
+        self.optim_state = OptimState.UNSCALED
+        if found_inf:
+            inner.abort_step()
+        else:
+            inner.commit_step()
+            combined_scale = float(device_says['combined_scale'])
+            self.last_step_info['combined_scale'] = -1 if combined_scale == -1.0 else combined_scale
+            if self.clipping_flag:
+                self.last_step_info['total_norm'] = float(device_says['total_norm'])
+        self.grad_scaler.update(found_inf)
+        self._clear_optim_states()
+        self.zero_grad()
+        self._update_fp16_params()
+        return True
+
     def step(self, *args, **kwargs):
         launched = self._launch_chunk_stats()
+        if (self.gated_step and self._binding is not None and self.scaled_optimizer and not args and not kwargs
+                and not self._binding.zero_grads):
+            records = self._records_of_all_chunks(launched)
+            if records is not None:
+                self.optim.prepare_step()
+                self._set_grad_ptr()
+                if self._step_gated(launched, records):
+                    return None
         if self._binding is not None and not args and not kwargs:
             # host work of the update launch, done while the flags pass runs on the device
             self.optim.prepare_step()

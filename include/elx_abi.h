@@ -107,7 +107,11 @@ typedef struct ElxHyper {
     float eps;       /* (float)eps */
     float neg_step;  /* (float)(-(lr/bc1)) */
     uint32_t flags;
-    uint32_t reserved[3];
+    /* the gate: read only by elx_adam_step_gated_mt, written by elx_decide (whatever the caller puts
+       here is overwritten) */
+    float gate_div_scale; /* the step's div_scale, -1 when no unscale is needed */
+    float gate_inv_scale; /* 1 / div_scale when that is exact */
+    uint32_t gate;        /* unscale mode (0 none, 1 multiply by the reciprocal, 2 divide) | skip << 8 */
 } ElxHyper;
 
 /* Result of the stats pass for one chunk; also the element type of its partials workspace. */
@@ -116,6 +120,19 @@ typedef struct ElxStats {
     uint32_t overflow; /* 1 if any valid element is +inf, -inf or NaN */
     uint32_t reserved;
 } ElxStats;
+
+/*
+ * The decisions of one step as elx_decide leaves them in device memory for elx_adam_step_gated_mt, and
+ * for the host to read back: elixir/wrapper/optimizer.py:137-183.
+ */
+typedef struct ElxDecision {
+    float div_scale;       /* (float)combined_scale, -1 when no unscale is needed */
+    float inv_scale;       /* 1 / div_scale when that is exact (div_scale a power of two), else 1 */
+    uint32_t mode;         /* 0 no unscale, 1 multiply by inv_scale, 2 divide by div_scale */
+    uint32_t skip;         /* 1: some chunk overflowed, the step must not update anything */
+    double total_norm;     /* global L2 norm of the scaled gradients (0 when clipping is off) */
+    double combined_scale; /* loss scale x clip coefficient as a float64, -1 when it equals 1 */
+} ElxDecision;
 
 /* ABI version of the loaded library (ELX_ABI_VERSION). */
 int elx_version(void);
@@ -131,6 +148,7 @@ uint32_t elx_sizeof_chunk(void);
 uint32_t elx_sizeof_seg(void);
 uint32_t elx_sizeof_hyper(void);
 uint32_t elx_sizeof_stats(void);
+uint32_t elx_sizeof_decision(void);
 
 /*
  * Host-side validation of HOST copies of the tables, to be called once before they are uploaded:
@@ -181,6 +199,31 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
                      const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,
                      uint32_t grid_tiles_per_chunk, float div_scale, int grad_dtype, int lowp_dtype,
                      uint32_t flags, uint32_t blocks_per_cu, void *stream);
+
+/*
+ * The host decisions of optimizer.py:137-183 taken on the device, so that the update can be enqueued
+ * without waiting for the flags to reach the host: one thread reads the n_chunks records of a stats or
+ * landing launch (in the order given), ORs the overflow flags and, with `clipping`, forms the global
+ * norm and the clip coefficient in the float64 arithmetic the reference's Python uses
+ *   l2_i = (double)(float)sqrt(sumsq_i) squared;  norm = sqrt((double)(float)sum_i l2_i);
+ *   clip = ((norm / loss_scale) + 1e-6) / max_norm;  combined = clip > 1 ? clip * loss_scale : loss_scale
+ * and writes *d_decision and the gate words of the n_hypers records at d_hypers (the table of the
+ * update launch that follows).  loss_scale > 0; max_norm > 0 when clipping.
+ */
+int elx_decide(const ElxStats *d_stats, uint32_t n_chunks, double loss_scale, double max_norm, int clipping,
+               ElxHyper *d_hypers, uint32_t n_hypers, ElxDecision *d_decision, void *stream);
+
+/*
+ * elx_adam_step_mt with the unscale parameters and the skip flag read from the gate words of the hyper
+ * records when the kernel runs (elx_decide on the same d_hypers must precede it on the same stream);
+ * they arrive with the record a tile loads anyway.  With skip set nothing is updated and every element
+ * of every record only has its low-precision copy refreshed -- what the skip branch of
+ * optimizer.py:196-203 does through Chunk.optim_update.
+ */
+int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
+                           const ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,
+                           uint32_t grid_tiles_per_chunk, int grad_dtype, int lowp_dtype, uint32_t flags,
+                           uint32_t blocks_per_cu, void *stream);
 
 /*
  * Low-precision refresh alone: lowp_out[0, n_alloc) = round-to-nearest-even(master) for every

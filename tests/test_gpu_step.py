@@ -641,3 +641,91 @@ def test_single_buffer_stats_and_writeback(oracle, dtype, n, offset):
         _abi.writeback(0, lowp.data_ptr(), CODE[dtype], n, stream)
     with pytest.raises(_abi.ElxError):
         _abi.grad_stats(g.data_ptr(), CODE[dtype], n, 2000, ws.data_ptr(), ws.data_ptr(), stream)
+
+
+# ------------------------------------------------------------------------------------------------
+# the decisions of the step taken on the device
+# ------------------------------------------------------------------------------------------------
+
+
+def test_decide_kernel_matches_host_arithmetic(oracle):
+    """elx_decide against the float64 arithmetic of optimizer.py:137-183 as the host (and the oracle)
+    performs it: skip flag, global norm, combined scale, and the fp32 unscale parameters derived from
+    it, over many random sets of per-chunk records -- identical bits."""
+    rng = np.random.default_rng(7)
+    stream = torch.cuda.current_stream().cuda_stream
+    dec = torch.zeros(32, dtype=torch.uint8, device=DEV)
+    hyp_host = np.zeros(3, dtype=_abi.HYPER_DTYPE)
+    cases = 0
+    for trial in range(300):
+        n = int(rng.integers(1, 40))
+        recs = np.zeros(n, dtype=_abi.STATS_DTYPE)
+        recs['sumsq'] = 10.0**rng.uniform(-12, 14, n) * rng.choice([0.0, 1.0], n, p=[0.05, 0.95])
+        overflow = trial % 7 == 3
+        if overflow:
+            recs['overflow'][int(rng.integers(0, n))] = 1
+        loss_scale = float(rng.choice([1.0, 2.0, 64.0, 65536.0, 3.0, 1024.0, 2.0**24]))
+        max_norm = float(rng.choice([0.0, 0.5, 1.0, 2.5]))
+        clipping = max_norm > 0
+        d_recs = torch.from_numpy(recs.view(np.uint8).copy()).to(DEV)
+        hyp = torch.from_numpy(hyp_host.view(np.uint8).copy()).to(DEV)
+        _abi.decide(d_recs.data_ptr(), n, loss_scale, max_norm, clipping, hyp.data_ptr(), 3, dec.data_ptr(), stream)
+        got = dec.cpu().numpy().view(_abi.DECISION_DTYPE)[0]
+        gates = hyp.cpu().numpy().view(_abi.HYPER_DTYPE)
+        assert bool(got['skip']) == overflow
+        for g in gates:
+            assert g['gate'] == int(got['mode']) | (int(got['skip']) << 8)
+            assert g['gate_div_scale'] == got['div_scale'] and g['gate_inv_scale'] == got['inv_scale']
+        if overflow:
+            continue
+        l2 = [float(np.float32(np.sqrt(x)))**2 for x in recs['sumsq']]          # chunk.py:218-221
+        norm = O.global_norm(l2) if clipping else None
+        want = ea.calc_combined_scale(loss_scale, norm, max_norm, clipping)
+        assert float(got['combined_scale']) == float(want), (trial, got['combined_scale'], want)
+        if clipping:
+            assert float(got['total_norm']) == norm
+        div = np.float32(want)
+        assert got['div_scale'] == div
+        if div > 0:
+            m, e = np.frexp(div)
+            pow2 = m == 0.5 and -125 <= e <= 126
+            assert got['mode'] == (1 if pow2 else 2)
+            assert got['inv_scale'] == (np.float32(1.0) / div if pow2 else np.float32(1.0))
+        else:
+            assert got['mode'] == 0
+        cases += 1
+    assert cases > 200
+
+
+def test_device_decided_and_host_decided_steps_agree(oracle):
+    """The same three steps (clean, overflow, clean) with the decisions on the device and on the host:
+    identical state, scale and reports."""
+    dtype = torch.float16
+    outs = []
+    for gated in (True, False):
+        module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=13, grad_std=3e-2, loss_scale=256.0,
+                                              weight_decay=0.1, max_norm=1.0, initial_scale=256.0, hysteresis=1)
+        opt.gated_step = gated
+        gen = torch.Generator(device=DEV).manual_seed(3)
+        infos = []
+        for step in range(3):
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (3e-2 * opt.loss_scale)
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+                pc.invalidate_stats()
+            if step == 1:
+                module.param_chunks[-1].shard[11] = float('nan')
+            opt.mark_gradients_scaled()
+            opt.step()
+            infos.append(dict(opt.last_step_info))
+        outs.append((infos, opt.loss_scale, [st['step'] for st in opt.state.values()],
+                     [(pc.paired_chunk.shard.clone(), pc.shard.clone(), *[t.clone() for t in
+                                                                          opt._binding.moments(pc.paired_chunk)])
+                      for pc in module.param_chunks]))
+    (ia, sa, ka, ta), (ib, sb, kb, tb) = outs
+    assert [i['found_inf'] for i in ia] == [False, True, False] == [i['found_inf'] for i in ib]
+    assert ia == ib and sa == sb == 128.0 and ka == kb and set(ka) == {2}
+    for a, b in zip(ta, tb):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
