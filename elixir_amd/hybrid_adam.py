@@ -328,10 +328,12 @@ class HybridAdam(torch.optim.Optimizer):
             if events is not None:
                 events['adam_step'][1].record()
         if prep.dplan.refresh is not None:
-            if events is not None:
-                if 'refresh' not in events:
-                    events['refresh'] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-                events['refresh'][0].record()
+            if events is not None and 'refresh' not in events:
+                # the refresh is bracketed by the end of the update launch and its own end event
+                begin = events['adam_step'][1] if 'adam_step' in events else torch.cuda.Event(enable_timing=True)
+                events['refresh'] = (begin, torch.cuda.Event(enable_timing=True))
+                if 'adam_step' not in events:
+                    begin.record()
             _abi.writeback_mt(prep.dplan.refresh.ptr, len(plan.refresh_rows), prep.lowp_code, plan.refresh_max_elems,
                               prep.dplan.refresh_aligned, stream)
             if events is not None:
