@@ -299,6 +299,11 @@ class HybridAdam(torch.optim.Optimizer):
         words of the prepared hyper table, where ``elx_decide`` has put them (``div_scale`` is then
         ignored).  ``defer_commit``: launch only; the caller finishes with ``commit_step()`` once it
         knows that the step happened, or ``abort_step()`` when the device decided to skip."""
+        return self.launch_step(closure, div_scale, gated=gated, defer_commit=defer_commit)
+
+    def launch_step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
+        """``step`` without the profiler scope and hook dispatch torch wraps around every optimizer's
+        ``step`` (tens of microseconds that the device would wait for)."""
         loss = None
         if closure is not None:
             with torch.enable_grad():
@@ -449,7 +454,14 @@ class HybridAdam(torch.optim.Optimizer):
             return None
         groups = self.param_groups
         # hyper record per entry: the (group, step + 1) pair it will be updated with
-        idx_of = [self._hyper_index(hypers, groups[gi], state['step'] + 1) for state, gi, _, _, _ in entries]
+        seen: Dict = {}    # (group, step) -> hyper index: nearly always one step count per group
+        idx_of = []
+        for state, gi, _, _, _ in entries:
+            k = (gi, state['step'])
+            h = seen.get(k)
+            if h is None:
+                h = seen[k] = self._hyper_index(hypers, groups[gi], k[1] + 1)
+            idx_of.append(h)
         lowp_dtype = b.chunks[0].paired_chunk.chunk_dtype
         grad_code = dtype_code(lowp_dtype)
         lowp_code = _abi.ELX_NONE if b.zero_grads else grad_code

@@ -465,7 +465,7 @@ class ElixirOptimizer:
         decided = torch.cuda.Event()
         decided.record(main)
         with self._timed('update'):
-            inner.step(gated=True, defer_commit=True)
+            inner.launch_step(gated=True, defer_commit=True)
 
         side = g['side']
         side.wait_event(decided)
