@@ -109,7 +109,6 @@ def fused_landing_leg(built, steps):
         for pc in chunks:
             pc.invalidate_stats()
         t_land = timed(lambda: built.land_gradients(fused=True))
-        opt.prepare_ahead()    # as ElixirOptimizer.backward does once the landing launches are queued
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         opt.step()

@@ -566,7 +566,10 @@ class ElixirOptimizer:
         backward and the landing of the gradients; ``step()`` then finds them ready (and rebuilds them
         if a hyper-parameter has changed in between)."""
         if self._binding is not None:
-            self.optim.prepare_step()
+            try:
+                self.optim.prepare_step()
+            except RuntimeError:
+                self.optim.discard_prepared()    # nothing to prepare for: step() is where the refusal belongs
 
     def backward_by_grad(self, tensor: torch.Tensor, grad: torch.Tensor):
         self.optim_state = OptimState.SCALED
@@ -574,5 +577,7 @@ class ElixirOptimizer:
 
     def mark_gradients_scaled(self) -> None:
         """For callers that land gradients in the chunk shards themselves (no ``backward`` through
-        this wrapper): declares that the shards now hold gradients scaled by ``loss_scale``."""
+        this wrapper): declares that the shards now hold gradients scaled by ``loss_scale`` and, as
+        ``backward`` does at this point, prepares the tables of the coming step."""
         self.optim_state = OptimState.SCALED
+        self.prepare_ahead()
