@@ -487,7 +487,6 @@ class ElixirOptimizer:
         assert found_inf == self._check_overflow()
         self.last_step_info = dict(found_inf=found_inf, combined_scale=None, total_norm=None,
                                    chunk_overflow=[c._overflow for c in chunks])
-        assert self.optim_state == OptimState.SCALED or found_inf
         self.optim_state = OptimState.UNSCALED
         if found_inf:
             inner.abort_step()
@@ -506,7 +505,7 @@ class ElixirOptimizer:
     def step(self, *args, **kwargs):
         launched = self._launch_chunk_stats()
         if (self.gated_step and self._binding is not None and self.scaled_optimizer and not args and not kwargs
-                and not self._binding.zero_grads):
+                and not self._binding.zero_grads and self.optim_state == OptimState.SCALED):
             records = self._records_of_all_chunks(launched)
             if records is not None:
                 self.optim.prepare_step()

@@ -729,3 +729,17 @@ def test_device_decided_and_host_decided_steps_agree(oracle):
     for a, b in zip(ta, tb):
         for x, y in zip(a, b):
             assert torch.equal(x, y)
+
+
+def test_step_without_scaled_gradients_is_refused(oracle):
+    """optimizer.py:169: a step needs gradients that backward has scaled; a second step() in a row
+    must not run an update on whatever sits in the shards."""
+    module, opt, ochunks = build_workload(tiny_gpt2(n_layer=1), 1 << 16, torch.float16, seed=3, loss_scale=64.0,
+                                          initial_scale=64.0)
+    opt.mark_gradients_scaled()
+    opt.step()
+    before = [pc.paired_chunk.shard.clone() for pc in module.param_chunks]
+    with pytest.raises(AssertionError):
+        opt.step()
+    for pc, p0 in zip(module.param_chunks, before):
+        assert torch.equal(pc.paired_chunk.shard, p0)
