@@ -411,8 +411,6 @@ class ElixirOptimizer:
             return None    # bound fake parameters never carry a .grad: nothing to drop
         return self.optim.zero_grad(set_to_none=True)
 
-    # ------------------------------------------------------------------ the step
-
     # ------------------------------------------------------------------ the step, decided on the device
 
     def _gate_buffers(self, device: torch.device, n_chunks: int):
@@ -501,6 +499,8 @@ class ElixirOptimizer:
         self.zero_grad()
         self._update_fp16_params()
         return True
+
+    # ------------------------------------------------------------------ the step
 
     def step(self, *args, **kwargs):
         launched = self._launch_chunk_stats()
