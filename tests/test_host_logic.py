@@ -442,3 +442,73 @@ def test_chunk_cpu_copy_and_load_tensors():
     chunk.load_tensors([None, new_b])
     assert torch.equal(chunk.shard[:15], ca.flatten()) and torch.equal(chunk.shard[15:22], new_b)
     assert torch.count_nonzero(chunk.shard[22:]) == 0
+
+
+def test_launch_plan_properties_random():
+    """Whatever the buffers and segments: update rows + refresh rows tile every buffer exactly once,
+    every segment element appears in exactly one row segment with its hyper index, and the tables
+    pass the library's own validation."""
+    from hypothesis import given, settings, strategies as st
+    from elixir_amd.launch_plan import FlatBuffer, build_plan
+    import elixir_amd.launch_plan as LP
+
+    @st.composite
+    def buffers(draw):
+        out = []
+        for k in range(draw(st.integers(1, 4))):
+            n_alloc = draw(st.integers(1, 300_000))
+            n_valid = draw(st.integers(0, n_alloc))
+            cuts = sorted(set(draw(st.lists(st.integers(0, n_valid), max_size=8)) + [0, n_valid]))
+            segs = []
+            for a, b in zip(cuts, cuts[1:]):
+                if b > a and draw(st.booleans()):
+                    lo = draw(st.integers(a, b - 1))
+                    segs.append((lo, b, draw(st.integers(0, 2))))
+            base = (k + 1) << 36
+            lowp = draw(st.booleans())
+            out.append(FlatBuffer(grad=base, lowp_out=base if lowp else 0, master=base + (1 << 32), m=base + (2 << 32),
+                                  v=base + (3 << 32), n_alloc=n_alloc, n_valid=n_valid, segs=segs))
+        if any(b.lowp_out for b in out):    # one launch has one low-precision type: all or none
+            for b in out:
+                b.lowp_out = b.grad
+        return out
+
+    @settings(max_examples=60, deadline=None)
+    @given(buffers(), st.sampled_from([16, 64, 2048]))
+    def check(bufs, block_tiles):
+        LP.BLOCK_TILES = block_tiles
+        try:
+            lowp = _abi.ELX_F16 if bufs[0].lowp_out else _abi.ELX_NONE
+            plan = build_plan(bufs, 2, 2, 3, _abi.ELX_F16, lowp)
+        finally:
+            LP.BLOCK_TILES = 2048
+        B = plan.block_elems
+        for buf in bufs:
+            rows = [r for r in plan.rows if buf.master <= r['master'] < buf.master + 4 * buf.n_alloc]
+            rows.sort(key=lambda r: r['master'])
+            pos = 0
+            seen = {}
+            for r in rows:
+                b = (int(r['master']) - buf.master) // 4
+                assert b == pos and b % B == 0 and 0 < r['n_alloc'] <= B
+                assert r['n_valid'] == max(0, min(int(r['n_alloc']), buf.n_valid - b))
+                prev = 0
+                for sg in plan.segs[r['seg_begin']:r['seg_end']]:
+                    assert prev <= sg['begin'] < sg['end'] <= r['n_valid']
+                    prev = int(sg['end'])
+                    for e in (int(sg['begin']), int(sg['end']) - 1):
+                        seen[b + e] = int(sg['hyper'])
+                pos += int(r['n_alloc'])
+            up_end = pos
+            assert up_end >= buf.n_valid and (up_end == buf.n_alloc or up_end % B == 0)
+            if plan.refresh_rows is not None and buf.lowp_out:
+                tail = [r for r in plan.refresh_rows if r['master'] == buf.master + 4 * up_end]
+                assert (len(tail) == 1 and tail[0]['n_alloc'] == buf.n_alloc - up_end) or up_end == buf.n_alloc
+            else:
+                assert up_end == buf.n_alloc or not buf.lowp_out
+            for sb, se, h in buf.segs:    # the ends of every segment are covered with the right hyper index
+                assert seen.get(sb) == h and seen.get(se - 1) == h
+        covered = sum(int(s['end'] - s['begin']) for s in plan.segs)
+        assert covered == sum(se - sb for buf in bufs for sb, se, _ in buf.segs)
+
+    check()
