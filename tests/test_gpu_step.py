@@ -743,3 +743,50 @@ def test_step_without_scaled_gradients_is_refused(oracle):
         opt.step()
     for pc, p0 in zip(module.param_chunks, before):
         assert torch.equal(pc.paired_chunk.shard, p0)
+
+
+def test_tensors_the_optimizer_does_not_own_are_left_alone(oracle):
+    """Tensors of a chunk that are in no parameter group (the optimizer was given a subset): their
+    master / exp_avg / exp_avg_sq stay untouched, their low-precision copy is still refreshed with the
+    rest of the shard (chunk.py:414 copies the whole shard)."""
+    dtype = torch.float16
+    named = [('a.weight', (4096, 3)), ('b.weight', (5000,)), ('c.weight', (300, 64)), ('d.weight', (7,)),
+             ('e.weight', (9000,)), ('f.weight', (256, 33))]
+    sr = ea.greedy_search([(n, S.numel(s)) for n, s in named], 1 << 15, dtype)
+    module = ea.ElixirModule(dict(named), sr, dtype=dtype)
+    params = list(module.parameters())
+    owned = [params[0], params[2], params[5]]                       # b, d, e are not the optimizer's
+    inner = ea.HybridAdam(owned, lr=1e-2, weight_decay=0.1)
+    opt = ea.ElixirOptimizer(module, inner, initial_scale=32.0, hysteresis=1)
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    state0 = []
+    for pc in module.param_chunks:
+        oc = pc.paired_chunk
+        oc.shard[:pc.utilized_size] = torch.randn(pc.utilized_size, generator=gen, device=DEV) * 0.05
+        m, v = opt._binding.moments(oc)
+        m[:pc.utilized_size] = torch.randn(pc.utilized_size, generator=gen, device=DEV) * 1e-3
+        v[:pc.utilized_size] = torch.rand(pc.utilized_size, generator=gen, device=DEV) * 1e-5
+        g = torch.randn(pc.shard_size, generator=gen, device=DEV) * 0.3
+        g[pc.utilized_size:] = 0
+        pc.shard.copy_(g.to(dtype))
+        pc.invalidate_stats()
+        state0.append((oc.shard.clone(), m.clone(), v.clone(), pc.shard.clone()))
+    opt.mark_gradients_scaled()
+    opt.step()
+    assert opt.last_step_info['found_inf'] is False and opt.last_step_info['combined_scale'] == 32.0
+    owned_set = set(owned)
+    for pc, (p0, m0, v0, g0) in zip(module.param_chunks, state0):
+        oc = pc.paired_chunk
+        m, v = opt._binding.moments(oc)
+        for t, info in pc.tensors_info.items():
+            sl = slice(info.offset, info.end)
+            if t in owned_set:
+                pn, mn, vn = to_np(p0[sl]), to_np(m0[sl]), to_np(v0[sl])
+                oracle.adam(to_np(g0[sl]), O.F16, pn, mn, vn, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.1,
+                            step=1, adamw_mode=True, div_scale=32.0)
+                assert np.array_equal(to_np(oc.shard[sl]).view(np.uint32), pn.view(np.uint32))
+                assert np.array_equal(to_np(m[sl]).view(np.uint32), mn.view(np.uint32))
+                assert np.array_equal(to_np(v[sl]).view(np.uint32), vn.view(np.uint32))
+            else:
+                assert torch.equal(oc.shard[sl], p0[sl]) and torch.equal(m[sl], m0[sl]) and torch.equal(v[sl], v0[sl])
+        assert torch.equal(pc.shard, oc.shard.to(dtype))            # the whole shard, owned or not
