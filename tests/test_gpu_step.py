@@ -790,3 +790,42 @@ def test_tensors_the_optimizer_does_not_own_are_left_alone(oracle):
             else:
                 assert torch.equal(oc.shard[sl], p0[sl]) and torch.equal(m[sl], m0[sl]) and torch.equal(v[sl], v0[sl])
         assert torch.equal(pc.shard, oc.shard.to(dtype))            # the whole shard, owned or not
+
+
+def test_per_tensor_step_counts_and_changing_learning_rates(oracle):
+    """Every tensor is updated with ITS step count (bias corrections differ per tensor after a state
+    load) and with the learning rate its group has at that step."""
+    dtype = torch.bfloat16
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=23, loss_scale=1.0, weight_decay=0.05)
+    sd = opt.state_dict()
+    for i, st in sd['state'].items():
+        st['step'] = 3 * i % 11                                       # anything from 0 to 10
+    opt.load_state_dict(sd)
+    steps = {}
+    k = 0
+    for group in opt.param_groups:
+        for fake in group['params']:
+            steps[(id(opt.param_to_optim_chunk[fake]), opt.param_to_range[fake][0])] = sd['state'][k]['step']
+            k += 1
+    for pc, oc in zip(module.param_chunks, ochunks):
+        for seg in oc.segments:
+            seg.step = steps[(id(pc.paired_chunk), seg.begin)]
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    for step in range(3):
+        lr = 1e-3 * (0.5**step)
+        for g in opt.param_groups:
+            g['lr'] = lr
+        for oc in ochunks:
+            for seg in oc.segments:
+                seg.lr = lr
+        if step:
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * 1e-3
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+                pc.invalidate_stats()
+            refresh_oracle_grads(module, ochunks)
+        _run_and_compare(module, opt, ochunks, dtype, O.ConstantGradScalerOracle(1.0), tag=f'step {step}')
+        assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'step {step}') == 0
+    want = sorted(s + 3 for s in steps.values())
+    assert sorted(st['step'] for st in opt.state.values()) == want
