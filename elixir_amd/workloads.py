@@ -13,7 +13,7 @@ import torch
 from . import shapes as S
 from .chunk import land_chunks
 from .hybrid_adam import HybridAdam
-from .module import ElixirModule, greedy_search
+from .module import ElixirModule, greedy_search, reserve_device_pool
 from .optimizer import ElixirOptimizer
 
 
@@ -73,13 +73,17 @@ class BuiltWorkload:
 
 
 def build(name: str, device: Optional[torch.device] = None, seed: int = 1234, shapes: Optional[List[S.NamedShape]] = None,
-          chunk_size: Optional[int] = None, hysteresis: Optional[int] = None) -> BuiltWorkload:
+          chunk_size: Optional[int] = None, hysteresis: Optional[int] = None, reserve_memory: bool = True) -> BuiltWorkload:
     spec = WORKLOADS[name]
     device = device or torch.device('cuda', torch.cuda.current_device())
     named = list(shapes if shapes is not None else spec.shapes())
     csize = chunk_size or spec.chunk_size
     sr = greedy_search([(n, S.numel(s)) for n, s in named], csize, spec.dtype, shard_device=device)
-    module = ElixirModule(dict(named), sr, dtype=spec.dtype)
+    if reserve_memory:
+        # everything this workload keeps on the device, the saved gradients included, in one allocation
+        esize = torch.empty(0, dtype=spec.dtype).element_size()
+        reserve_device_pool(sum(p.chunk_size for p in sr.param_chunk_plans) * (2 * esize + 12), device)
+    module = ElixirModule(dict(named), sr, dtype=spec.dtype, reserve_memory=reserve_memory)
 
     decay, exempt = [], []
     for (pname, shape), p in zip(named, module.parameters()):
