@@ -161,3 +161,22 @@ def test_check_land_rows_accepts_and_rejects():
     expect(_abi.ELX_E_RANGE, offsets=np.array([0, 2, 2], dtype=np.uint32))
     expect(_abi.ELX_E_ORDER, offsets=np.array([0, 3, 2, 3], dtype=np.uint32))
     expect(_abi.ELX_E_SIZE, offsets=np.array([0, 1, 2, 3, 3], dtype=np.uint32))
+
+
+def test_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 on its own, and the record sizes a C
+    compiler sees must be the ones the library and the binding use."""
+    import subprocess
+    src = tmp_path / 'probe.c'
+    src.write_text('#include "elx_abi.h"\n#include <stdio.h>\n'
+                   'int main(void) { printf("%zu %zu %zu %zu %zu\\n", sizeof(ElxChunk), sizeof(ElxSeg), sizeof(ElxHyper), '
+                   'sizeof(ElxStats), sizeof(ElxDecision)); return 0; }\n')
+    exe = tmp_path / 'probe'
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), 'include')
+    subprocess.run(['gcc', '-std=c99', '-Wall', '-Wextra', '-pedantic', '-Werror', '-I', inc, str(src), '-o', str(exe)],
+                   check=True)
+    sizes = [int(x) for x in subprocess.run([str(exe)], check=True, stdout=subprocess.PIPE, text=True).stdout.split()]
+    lib = _abi.load()
+    assert sizes == [lib.elx_sizeof_chunk(), lib.elx_sizeof_seg(), lib.elx_sizeof_hyper(), lib.elx_sizeof_stats(),
+                     lib.elx_sizeof_decision()] == [72, 24, 48, 16, 32]
+    assert _abi.DECISION_DTYPE.itemsize == 32
