@@ -333,12 +333,62 @@ def config1_line(args):
     print(json.dumps(out))
 
 
+def velocity_line(args):
+    """The reference's own optimizer micro-benchmark, profile/profile_optimizer.py:34-60, on one GPU:
+    a flat fp32 parameter of 10**9 elements (zeros), a fresh fp32 gradient of ones before every
+    step, HybridAdam(lr=1e-5), each ``optimizer.step()`` timed by the wall clock between two device
+    synchronisations; velocity = steps * 1 (10**9 elements) / summed time.  elixir/search/
+    simulator.py:128-129 hard-codes 50 (x10**9 elements/s per GPU, hardware not stated) as the result
+    the reference's planner assumes.  28 B per element: read p, g, m, v, write p, m, v."""
+    import elixir_amd as ea
+    n = 10**9
+    weight = torch.nn.Parameter(torch.zeros(n, device='cuda'))
+    opt = ea.HybridAdam([weight], lr=1e-5)
+    opt.kernel_events = {}
+    step_s, adam_ms = [], []
+    for i in range(args.warmup + args.steps):
+        opt.zero_grad()
+        weight.grad = torch.ones(n, dtype=torch.float, device='cuda')
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if i >= args.warmup:
+            step_s.append(dt)
+            ev = opt.kernel_events['adam_step']
+            adam_ms.append(ev[0].elapsed_time(ev[1]))
+    opt.kernel_events = None
+    # closed form after k steps from p = 0 with g = 1: m_hat = v_hat = 1, so every step moves p by -lr / (1 + eps)
+    k = args.warmup + args.steps
+    expect = -k * 1e-5 / (1.0 + 1e-8)
+    got = weight.detach()[::max(1, n // 4096)].double().cpu().numpy()
+    assert np.allclose(got, expect, rtol=1e-5, atol=0), (float(got[0]), expect)
+    velocity = len(step_s) * (n / 1e9) / float(np.sum(step_s))
+    t_step, t_upd = float(np.mean(step_s)), float(np.mean(adam_ms)) * 1e-3
+    published = 50.0
+    out = {
+        'metric': 'adam_velocity', 'value': velocity, 'unit': '1e9 elements/s', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': t_step * 1e3, 'higher_is_better': True, 'scaling': 'weak',
+        'vs_baseline': velocity / published, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'velocity: flat fp32 parameter of 1e9 elements, fp32 gradient of ones, HybridAdam lr 1e-5 '
+                               '(the reference\'s profile/profile_optimizer.py)', 'valid_elements': n,
+                   'published_velocity': published, 'published_hardware': 'not stated by the reference'},
+        'step': {'ms_min': float(np.min(step_s)) * 1e3, 'gbps_28B': BYTES_UPDATE * n / t_step / 1e9,
+                 'frac_28B': BYTES_UPDATE * n / t_step / 1e9 / HBM_PEAK_GBPS},
+        'roofline': {'kernel': 'adam_step_kernel', 'bound': 'hbm', 'achieved': BYTES_UPDATE * n / t_upd / 1e9,
+                     'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': BYTES_UPDATE * n / t_upd / 1e9 / HBM_PEAK_GBPS,
+                     'traffic': None, 'bytes_per_launch': BYTES_UPDATE * n, 'ms_per_launch': t_upd * 1e3},
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=3)
-    ap.add_argument('--workload', default='c5', choices=['c1', 'c2', 'c4', 'c5'])
+    ap.add_argument('--workload', default='c5', choices=['c1', 'c2', 'c4', 'c5', 'velocity'])
     ap.add_argument('--cpu-sample', type=int, default=256 << 20, help='elements of the CPU baseline sample; 0 skips it')
     ap.add_argument('--blocks-per-cu', type=int, default=0,
                     help='cap on resident update workgroups per compute unit (0 = library default)')
@@ -385,6 +435,9 @@ def main():
     torch.cuda.set_device(device)
     if args.workload == 'c1':
         config1_line(args)
+        return
+    if args.workload == 'velocity':
+        velocity_line(args)
         return
 
     t_build = time.perf_counter()

@@ -95,11 +95,12 @@ class _HyperUploader:
         turn = self.turn
         stage = self.staging[turn]
         self.turn ^= 1
-        if self.copied[turn] is not None:
+        if self.copied[turn] is None:
+            self.copied[turn] = torch.cuda.Event()    # created once per buffer, recorded again at every use
+        else:
             self.copied[turn].synchronize()    # normally long past: the copy out of this buffer has run
         stage[:nbytes].numpy()[:] = host.view(np.uint8).reshape(-1)
         self.dev[:nbytes].copy_(stage[:nbytes], non_blocking=True)
-        self.copied[turn] = torch.cuda.Event()
         self.copied[turn].record(torch.cuda.current_stream(device))
         return self.dev.data_ptr()
 

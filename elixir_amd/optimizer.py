@@ -419,7 +419,7 @@ class ElixirOptimizer:
             g = self._gate = dict(device=device, decision=torch.zeros(32, dtype=torch.uint8, device=device),
                                   host=torch.zeros(n_chunks * _abi.STATS_DTYPE.itemsize + 32, dtype=torch.uint8,
                                                    pin_memory=True),
-                                  side=torch.cuda.Stream(device), copied=torch.cuda.Event())
+                                  side=torch.cuda.Stream(device), decided=torch.cuda.Event(), copied=torch.cuda.Event())
         return g
 
     def _records_of_all_chunks(self, launched):
@@ -460,7 +460,7 @@ class ElixirOptimizer:
         main = torch.cuda.current_stream(prep.device)
         _abi.decide(records.data_ptr(), n, float(self.loss_scale), float(self.max_norm), self.clipping_flag,
                     prep.d_hypers, len(prep.hyper_host), g['decision'].data_ptr(), main.cuda_stream)
-        decided = torch.cuda.Event()
+        decided = g['decided']    # reused: the wait on 'copied' below ends before the next step records it again
         decided.record(main)
         with self._timed('update'):
             inner.launch_step(gated=True, defer_commit=True)
@@ -573,6 +573,7 @@ class ElixirOptimizer:
     def backward_by_grad(self, tensor: torch.Tensor, grad: torch.Tensor):
         self.optim_state = OptimState.SCALED
         self.module.backward_by_grad(tensor, grad)
+        self.prepare_ahead()
 
     def mark_gradients_scaled(self) -> None:
         """For callers that land gradients in the chunk shards themselves (no ``backward`` through

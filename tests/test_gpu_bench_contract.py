@@ -32,3 +32,16 @@ def test_bench_json_line():
     c = out['cpu_baseline']
     assert c['kind'] == 'port' and c['cores'] >= 1 and c['value'] > 0 and c['unit'] == 'elements/s'
     assert out['fused_landing']['ms_per_step'] > 0
+
+
+def test_velocity_line():
+    """The reference's flat-parameter micro-benchmark (profile/profile_optimizer.py:34-60) as a bench workload:
+    10**9 fp32 elements, result checked against the closed form inside the run."""
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--workload', 'velocity', '--steps', '3',
+                           '--warmup', '1'], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=280)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = json.loads([l for l in proc.stdout.splitlines() if l.startswith('{')][0])
+    assert out['metric'] == 'adam_velocity' and out['config']['valid_elements'] == 10**9
+    assert abs(out['vs_baseline'] - out['value'] / 50.0) < 1e-9
+    assert abs(out['value'] - 1.0 / (out['ms_per_step'] * 1e-3)) <= 1e-6 * out['value']
+    assert out['roofline']['bytes_per_launch'] == 28 * 10**9 and 0 < out['roofline']['frac'] < 1
