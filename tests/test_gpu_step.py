@@ -199,6 +199,42 @@ def test_flat_fp16_grads_fp32_params(oracle):
     assert np.array_equal(to_np(p.data).view(np.uint32), pn.view(np.uint32))
 
 
+@pytest.mark.parametrize('seed', range(12))
+def test_flat_random_hypers_match_oracle(oracle, seed):
+    """Hyper-parameters, gradient type and divisor drawn at random, the edges included (beta1 of 0 and
+    of exactly 0.5, beta2 of 0, no bias correction, a divisor that is not a power of two, two groups
+    in one launch): identical bits to the oracle over four steps."""
+    rng = np.random.default_rng(9100 + seed)
+    gdtype = [torch.float32, torch.float16, torch.bfloat16][seed % 3]
+    adamw = bool(rng.integers(2))
+    groups = []
+    for _ in range(2):
+        groups.append(dict(lr=float(rng.choice([1e-5, 1e-3, 3e-2, 1.0])), betas=(float(rng.choice([0.0, 0.3, 0.5, 0.9, 0.99])),
+                                                                                 float(rng.choice([0.0, 0.5, 0.95, 0.999]))),
+                           eps=float(rng.choice([1e-12, 1e-8, 1e-3])), weight_decay=float(rng.choice([0.0, 1e-4, 0.1])),
+                           bias_correction=bool(rng.integers(4) > 0)))
+    sizes = [int(rng.integers(1, 70_000)), int(rng.integers(1, 5_000))]
+    torch.manual_seed(seed)
+    params = [torch.nn.Parameter((torch.randn(n) * 0.02).to(DEV)) for n in sizes]
+    host = [(to_np(p.data).copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)) for p, n in zip(params, sizes)]
+    opt = ea.HybridAdam([dict(params=[p], **g) for p, g in zip(params, groups)], adamw_mode=adamw)
+    for step in range(1, 5):
+        div = float(rng.choice([-1.0, 1.0, 64.0, 3.7, 1000.0]))
+        grads = [(torch.randn(n) * float(rng.choice([1e-4, 1e-2, 1.0])) * max(div, 1.0)).to(gdtype) for n in sizes]
+        for p, g in zip(params, grads):
+            p.grad_dtype = None
+            p.grad = g.to(DEV)
+        opt.step(div_scale=div)
+        for p, g, grp, (pn, mn, vn) in zip(params, grads, groups, host):
+            oracle.adam(to_np(g), CODE[gdtype], pn, mn, vn, lr=grp['lr'], beta1=grp['betas'][0], beta2=grp['betas'][1],
+                        eps=grp['eps'], weight_decay=grp['weight_decay'], step=step, adamw_mode=adamw,
+                        bias_correction=grp['bias_correction'], div_scale=div)
+            st = opt.state[p]
+            for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
+                assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32)), \
+                    f'seed {seed} step {step} {name} {gdtype} adamw {adamw} group {grp} div {div}'
+
+
 def test_first_step_is_sign_descent():
     """Closed form: with m = v = 0 and step 1, p moves by -lr * g / (|g| + eps) ~ -lr * sign(g)."""
     n = 10000

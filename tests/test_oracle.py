@@ -163,6 +163,41 @@ def test_adam_against_live_torch_cpu(oracle, adamw, wd, betas):
         p[:], m[:], v[:] = want_p, st['exp_avg'].numpy(), st['exp_avg_sq'].numpy()
 
 
+@pytest.mark.parametrize('seed', range(12))
+def test_adam_against_live_torch_cpu_random_hypers(oracle, seed):
+    """Hyper-parameters drawn at random, the edges included (beta1 of 0 and exactly 0.5, where torch's
+    lerp changes formula; beta2 of 0; a large eps; no decay): every step compared on its own."""
+    rng = np.random.default_rng(4200 + seed)
+    n = 20_011
+    adamw = bool(rng.integers(2))
+    lr = float(rng.choice([1e-5, 1e-3, 3e-2, 1.0]))
+    beta1 = float(rng.choice([0.0, 0.3, 0.5, 0.9, 0.99]))
+    beta2 = float(rng.choice([0.0, 0.5, 0.95, 0.999]))
+    eps = float(rng.choice([1e-12, 1e-8, 1e-3]))
+    wd = float(rng.choice([0.0, 1e-4, 0.1]))
+    torch.manual_seed(seed)
+    p0 = torch.randn(n) * 0.02
+    tp = torch.nn.Parameter(p0.clone())
+    topt = (torch.optim.AdamW if adamw else torch.optim.Adam)([tp], lr=lr, betas=(beta1, beta2), eps=eps,
+                                                              weight_decay=wd, foreach=False)
+    p, m, v = p0.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for step in range(1, 5):
+        g = torch.randn(n) * float(rng.choice([1e-4, 1e-2, 1.0]))
+        tp.grad = g.clone()
+        topt.step()
+        oracle.adam(g.numpy().copy(), O.F32, p, m, v, lr=lr, beta1=beta1, beta2=beta2, eps=eps, weight_decay=wd,
+                    step=step, adamw_mode=adamw)
+        st = topt.state[tp]
+        want_p, want_m, want_v = tp.data.numpy(), st['exp_avg'].numpy(), st['exp_avg_sq'].numpy()
+        gmax = float(g.abs().max())
+        what = f'seed {seed} step {step} adamw {adamw} lr {lr} betas {(beta1, beta2)} eps {eps} wd {wd}'
+        # p = p - step: the bound is relative to the operands (|p| and the step size lr)
+        assert np.all(np.abs(p.astype(np.float64) - want_p) <= 1e-6 * (np.abs(want_p) + lr)), what
+        assert np.all(np.abs(m.astype(np.float64) - want_m) <= 1e-6 * (np.abs(want_m) + gmax)), what
+        assert np.all(np.abs(v.astype(np.float64) - want_v) <= 1e-6 * (np.abs(want_v) + gmax**2)), what
+        p[:], m[:], v[:] = want_p, want_m, want_v
+
+
 def test_adam_fp32_tracks_float64_closed_form(oracle):
     """A wrong sign, a dropped bias correction or a transposed beta shows up at the 1e-2 level
     here; fp32 rounding stays below 1e-5 of the operand sizes."""
