@@ -46,6 +46,7 @@ constexpr int kVec = 4;                                // elements per lane per 
 constexpr int kUnroll = 1;                             // independent accesses per lane per stream
 constexpr uint32_t kSpan = kWave * kVec;               // elements one wavefront access covers
 constexpr uint32_t kTile = kSpan * kUnroll;            // 256 elements per tile
+constexpr uint64_t kMaxBufferElems = 1ull << 40;       // longest buffer a table row may describe (tile arithmetic stays far from overflow)
 constexpr uint32_t kLdsPerCu = 160u * 1024u;           // gfx950
 constexpr uint32_t kDefaultBlocksPerCu = 12;
 constexpr uint32_t kMinBlocksPerCu = 3;                // keeps the reservation below 64 KiB
@@ -976,10 +977,10 @@ int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *
     uint64_t max_tiles = 0;
     for (uint32_t i = 0; i < n_chunks; ++i) {
         const ElxChunk &c = h_chunks[i];
-        if ((c.n_alloc + kTile - 1) / kTile > max_tiles) max_tiles = (c.n_alloc + kTile - 1) / kTile;
         if (!c.master || !c.m || !c.v) return ELX_E_NULL;
         if (c.lowp_out && lowp_dtype == ELX_NONE) return ELX_E_DTYPE;
-        if (c.n_alloc == 0) return ELX_E_SIZE;
+        if (c.n_alloc == 0 || c.n_alloc > kMaxBufferElems) return ELX_E_SIZE;
+        if ((c.n_alloc + kTile - 1) / kTile > max_tiles) max_tiles = (c.n_alloc + kTile - 1) / kTile;
         if (c.n_valid > c.n_alloc) return ELX_E_RANGE;
         const uintptr_t ptrs[5] = {(uintptr_t)c.grad, (uintptr_t)c.lowp_out, (uintptr_t)c.master, (uintptr_t)c.m,
                                    (uintptr_t)c.v};
@@ -1018,7 +1019,7 @@ int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t 
     for (uint32_t i = 0; i < n_rows; ++i) {
         const ElxChunk &r = h_rows[i];
         if (!r.lowp_out) return ELX_E_NULL;
-        if (r.n_alloc == 0) return ELX_E_SIZE;
+        if (r.n_alloc == 0 || r.n_alloc > kMaxBufferElems) return ELX_E_SIZE;
         if (r.n_valid > r.n_alloc) return ELX_E_RANGE;
         if (((uintptr_t)r.grad & smask) || ((uintptr_t)r.lowp_out & dmask)) return ELX_E_ALIGN;
         const uint64_t t = (r.n_alloc + tile - 1) / tile;

@@ -180,3 +180,84 @@ def test_header_is_plain_c(tmp_path):
     assert sizes == [lib.elx_sizeof_chunk(), lib.elx_sizeof_seg(), lib.elx_sizeof_hyper(), lib.elx_sizeof_stats(),
                      lib.elx_sizeof_decision()] == [72, 24, 48, 16, 32]
     assert _abi.DECISION_DTYPE.itemsize == 32
+
+
+def test_check_tables_property_random():
+    """The validator is what stands between a table and a launch.  Whatever table is drawn: if it is
+    accepted, every bound the kernels rely on holds (recomputed here); and each single corruption of an
+    accepted table is refused with a negative code, never accepted and never a crash."""
+    from hypothesis import given, settings, strategies as st
+    tile = _abi.tile_elems()
+
+    @st.composite
+    def tables(draw):
+        n_rows = draw(st.integers(1, 5))
+        n_hypers = draw(st.integers(1, 3))
+        rows = np.zeros(n_rows, dtype=_abi.CHUNK_DTYPE)
+        segs = []
+        tiles = 0
+        for i in range(n_rows):
+            n_alloc = draw(st.integers(1, 50_000))
+            n_valid = draw(st.integers(0, n_alloc))
+            base = (i + 1) << 32
+            rows[i]['grad'] = base if draw(st.booleans()) else 0
+            rows[i]['lowp_out'] = base + (1 << 28)
+            rows[i]['master'], rows[i]['m'], rows[i]['v'] = base + (2 << 28), base + (3 << 28), base + (4 << 28)
+            rows[i]['n_alloc'], rows[i]['n_valid'], rows[i]['tile_begin'] = n_alloc, n_valid, tiles
+            tiles += (n_alloc + tile - 1) // tile
+            rows[i]['seg_begin'] = len(segs)
+            cuts = sorted(set(draw(st.lists(st.integers(0, n_valid), max_size=6)) + [0, n_valid]))
+            for a, b in zip(cuts, cuts[1:]):
+                if b > a and draw(st.booleans()):
+                    segs.append((draw(st.integers(a, b - 1)), b, draw(st.integers(0, n_hypers - 1)), 0))
+            rows[i]['seg_end'] = len(segs)
+        seg_arr = np.array(segs, dtype=_abi.SEG_DTYPE) if segs else np.zeros(0, dtype=_abi.SEG_DTYPE)
+        return rows, seg_arr, n_hypers, tiles
+
+    def refused(rows, segs, n_hypers, gd=_abi.ELX_F16, ld=_abi.ELX_F16):
+        try:
+            _abi.check_tables(rows, segs if len(segs) else None, n_hypers, gd, ld)
+        except _abi.ElxError as e:
+            assert e.code < 0
+            return True
+        return False
+
+    @settings(max_examples=150, deadline=None)
+    @given(tables(), st.randoms(use_true_random=False))
+    def run(table, rnd):
+        rows, segs, n_hypers, tiles = table
+        info = _abi.check_tables(rows, segs if len(segs) else None, n_hypers, _abi.ELX_F16, _abi.ELX_F16)
+        assert info.total_tiles == tiles and info.aligned
+        assert info.max_tiles == max((int(r['n_alloc']) + tile - 1) // tile for r in rows)
+        i = rnd.randrange(len(rows))
+        corruptions = [
+            lambda r, s: r[i].__setitem__('master', 0),
+            lambda r, s: r[i].__setitem__('m', int(r[i]['m']) + 1),
+            lambda r, s: r[i].__setitem__('grad', int(r[i]['lowp_out']) + 1),
+            lambda r, s: r[i].__setitem__('n_valid', int(r[i]['n_alloc']) + 1),
+            lambda r, s: r[i].__setitem__('n_alloc', 0),
+            lambda r, s: r[i].__setitem__('n_alloc', (1 << 40) + 1),
+            lambda r, s: r[i].__setitem__('tile_begin', int(r[i]['tile_begin']) + 1),
+            lambda r, s: r[i].__setitem__('seg_end', len(s) + 1),
+            lambda r, s: r[i].__setitem__('seg_begin', int(r[i]['seg_end']) + 1),
+        ]
+        if len(segs):
+            j = rnd.randrange(len(segs))
+            owner = next(k for k in range(len(rows)) if rows[k]['seg_begin'] <= j < rows[k]['seg_end'])
+            corruptions += [
+                lambda r, s: s[j].__setitem__('hyper', n_hypers),
+                lambda r, s: s[j].__setitem__('end', int(r[owner]['n_valid']) + 1),
+                lambda r, s: s[j].__setitem__('begin', int(s[j]['end'])),
+            ]
+            if j + 1 < rows[owner]['seg_end']:
+                corruptions.append(lambda r, s: s[j].__setitem__('end', int(s[j + 1]['begin']) + 1))
+        for corrupt in corruptions:
+            r2, s2 = rows.copy(), segs.copy()
+            corrupt(r2, s2)
+            assert refused(r2, s2, n_hypers), (corruptions.index(corrupt), r2, s2)
+        assert refused(rows, segs, n_hypers, gd=_abi.ELX_F16, ld=_abi.ELX_BF16)
+        assert refused(rows, segs, n_hypers, gd=5)
+        if len(segs):
+            assert refused(rows, segs, 0)
+
+    run()
