@@ -72,6 +72,45 @@ def test_fp32_training_matches_torch_adamw():
             torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
 
 
+@pytest.mark.parametrize('make', [lambda ps: torch.optim.SGD(ps, lr=5e-2, momentum=0.9, nesterov=True),
+                                  lambda ps: torch.optim.RMSprop(ps, lr=1e-3)], ids=['sgd', 'rmsprop'])
+def test_inner_optimizer_outside_the_fused_list_runs_unfused(make):
+    """optimizer.py:54-56,211-214: any element-wise torch optimizer may sit inside the wrapper as long
+    as nothing has to be unscaled (fp32, no clipping); it then steps on views of the chunk storage.
+    Same optimizer on an identical plain copy: the same weights, to the reference's own tolerance."""
+    torch.manual_seed(0)
+    ref = Net().to(DEV)
+    model = copy.deepcopy(ref)
+    ropt = make(list(ref.parameters()))
+    named = [(n, p.numel()) for n, p in model.named_parameters()]
+    module = ea.ElixirModule(model, ea.greedy_search(named, 4096, torch.float32), dtype=torch.float32)
+    opt = ea.ElixirOptimizer(module, make(list(model.parameters())))
+    assert not opt.scaled_optimizer and opt.loss_scale == 1.0
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    for step in range(4):
+        x = batch(gen)
+        ropt.zero_grad()
+        ref(x).backward()
+        ropt.step()
+        opt.zero_grad()
+        opt.backward(module(x))
+        opt.step()
+        assert opt.last_step_info['found_inf'] is False and opt.last_step_info['combined_scale'] == -1
+        module.materialize_params()
+        sd = module.state_dict()
+        for name, want in ref.state_dict().items():
+            torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
+    # with clipping such an optimizer cannot be used: nothing would apply the coefficient
+    torch.manual_seed(0)
+    model = Net().to(DEV)
+    module = ea.ElixirModule(model, ea.greedy_search(named, 4096, torch.float32), dtype=torch.float32)
+    opt = ea.ElixirOptimizer(module, make(list(model.parameters())), max_norm=1e-3)
+    opt.zero_grad()
+    opt.backward(module(batch(gen)))
+    with pytest.raises(AssertionError):
+        opt.step()
+
+
 def test_fp16_training_matches_master_weight_amp_and_recovers_from_overflow():
     torch.manual_seed(0)
     master = Net().to(DEV)                         # fp32 master copy trained by plain torch
