@@ -236,7 +236,10 @@ void orc_adam(const void *g, int g_dtype, float *p, float *m, float *v, uint64_t
     const float decay_mul = (float)(1.0 - lr * weight_decay);
     const float wd_f = (float)weight_decay;
     const float w1 = (float)(1.0 - beta1);
-    const float one_minus_w1 = 1.0f - w1;
+    /* the coefficient of the second lerp form as torch's vectorised CPU kernel computes it: weight - 1
+     * (not -(1 - weight): the two differ in the sign of zero when beta1 = 0, and with it the sign of a
+     * zero exp_avg) */
+    const float w1_minus_one = w1 - 1.0f;
     const float beta2_f = (float)beta2;
     const float omb2 = (float)(1.0 - beta2);
     const float bc2_sqrt_f = (float)bc2_sqrt;
@@ -262,7 +265,7 @@ void orc_adam(const void *g, int g_dtype, float *p, float *m, float *v, uint64_t
         if (w1 < 0.5f)
             mi = fmaf(w1, diff, mi);
         else
-            mi = fmaf(-one_minus_w1, diff, gi);
+            mi = fmaf(w1_minus_one, diff, gi);
         /* v.mul_(beta2).addcmul_(g, g, value=1-beta2) (adam.py:476): the product v*beta2 is
          * rounded, (1-beta2)*g is rounded, and the last multiply-add is fused -- the form that
          * reproduces torch's CPU kernels bit for bit. */

@@ -567,9 +567,10 @@ def test_random_layouts_match_oracle(oracle, seed):
         assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'seed {seed} step {step}') == 0
 
 
+@pytest.mark.parametrize('beta1', [0.9, 0.5, 0.0])
 @pytest.mark.parametrize('div_scale', [-1.0, 64.0, 48.0])
 @pytest.mark.parametrize('gdtype', [torch.float32, torch.float16, torch.bfloat16])
-def test_signed_zeros_go_through_the_update_like_ieee(oracle, gdtype, div_scale):
+def test_signed_zeros_go_through_the_update_like_ieee(oracle, gdtype, div_scale, beta1):
     """Zeros of both signs in gradient, master and moments: every combination must come out with the
     bits the scalar C oracle produces (a multiply folded into a fused op with a +0 addend would not)."""
     vals = torch.tensor([0.0, -0.0, 1e-3, -2e-3])
@@ -581,7 +582,7 @@ def test_signed_zeros_go_through_the_update_like_ieee(oracle, gdtype, div_scale)
     v0 = torch.where(torch.arange(n) % 2 == 0, torch.zeros(n), torch.full((n,), 1e-6))
     for adamw, wd in ((True, 0.1), (False, 0.1), (True, 0.0)):
         p = torch.nn.Parameter(p0.clone().to(DEV))
-        opt = ea.HybridAdam([p], lr=1e-3, weight_decay=wd, adamw_mode=adamw)
+        opt = ea.HybridAdam([p], lr=1e-3, betas=(beta1, 0.999), weight_decay=wd, adamw_mode=adamw)
         p.grad_dtype = None
         p.grad = g0.to(gdtype).to(DEV)
         opt.step()                                               # creates the state (zeros)
@@ -592,7 +593,7 @@ def test_signed_zeros_go_through_the_update_like_ieee(oracle, gdtype, div_scale)
         p.grad = g0.to(gdtype).to(DEV)
         opt.step(div_scale=div_scale)
         pn, mn, vn = p0.numpy().copy(), m0.numpy().copy(), v0.numpy().copy()
-        oracle.adam(to_np(g0.to(gdtype)), CODE[gdtype], pn, mn, vn, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8,
+        oracle.adam(to_np(g0.to(gdtype)), CODE[gdtype], pn, mn, vn, lr=1e-3, beta1=beta1, beta2=0.999, eps=1e-8,
                     weight_decay=wd, step=2, adamw_mode=adamw, div_scale=div_scale)
         for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
             assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32)), (name, adamw, wd)

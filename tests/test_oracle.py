@@ -198,6 +198,34 @@ def test_adam_against_live_torch_cpu_random_hypers(oracle, seed):
         p[:], m[:], v[:] = want_p, want_m, want_v
 
 
+@pytest.mark.parametrize('beta1', [0.0, 0.3, 0.5, 0.9])
+def test_adam_signed_zero_moments_match_live_torch(oracle, beta1):
+    """Gradients of +0 and -0: the sign of a zero exp_avg depends on how the lerp coefficient of the
+    second form is computed (weight - 1, as torch's vectorised kernel does, against -(1 - weight));
+    with beta1 = 0 the two differ.  exp_avg and exp_avg_sq must carry torch's bits."""
+    n = 4096
+    torch.manual_seed(0)
+    p0 = torch.randn(n) * 0.02
+    g = torch.randn(n) * 1e-2
+    g[::3] = 0.0
+    g[1::7] = -0.0
+    tp = torch.nn.Parameter(p0.clone())
+    topt = torch.optim.Adam([tp], lr=1e-3, betas=(beta1, 0.999), foreach=False)
+    p, m, v = p0.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for step in (1, 2, 3):
+        gg = g.clone() if step != 2 else -g
+        tp.grad = gg.clone()
+        topt.step()
+        oracle.adam(gg.numpy().copy(), O.F32, p, m, v, lr=1e-3, beta1=beta1, beta2=0.999, eps=1e-8, weight_decay=0.0,
+                    step=step, adamw_mode=False)
+        st = topt.state[tp]
+        assert np.array_equal(st['exp_avg'].numpy().view(np.uint32), m.view(np.uint32)), f'beta1 {beta1} step {step}'
+        assert np.array_equal(st['exp_avg_sq'].numpy().view(np.uint32), v.view(np.uint32)), f'beta1 {beta1} step {step}'
+        if beta1 == 0.0:
+            assert np.array_equal(m.view(np.uint32), gg.numpy().view(np.uint32))    # exp_avg is the gradient, sign of zero included
+        p[:] = tp.data.numpy()
+
+
 def test_adam_fp32_tracks_float64_closed_form(oracle):
     """A wrong sign, a dropped bias correction or a transposed beta shows up at the 1e-2 level
     here; fp32 rounding stays below 1e-5 of the operand sizes."""
