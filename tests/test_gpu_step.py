@@ -567,6 +567,75 @@ def test_random_layouts_match_oracle(oracle, seed):
         assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'seed {seed} step {step}') == 0
 
 
+@pytest.mark.parametrize('seed', range(12))
+def test_random_trajectories_match_oracle(oracle, seed):
+    """Seven steps on a random layout with everything drawn at random: hysteresis and growth interval of
+    the scaler, clipping threshold, non-finite values in valid data (skip, back-off) or in the padding
+    (must not count), gradients landed by the fused launch or written into the shards, the step decided
+    on the device or on the host.  Flags, skips and the scale trajectory are exact at every step; the
+    state is bit-identical whenever no clip coefficient is involved, within 2e-6 otherwise (each step
+    compared on its own), and the low-precision copy is always the exact cast of the master."""
+    from elixir_amd.chunk import land_chunks
+    rng = np.random.default_rng(50_000 + seed)
+    n_tensors = int(rng.integers(1, 16))
+    sizes = [int(rng.choice([rng.integers(1, 9), rng.integers(9, 700), rng.integers(700, 9000), rng.integers(9000, 40000)]))
+             for _ in range(n_tensors)]
+    named = [(f't{i}.{"weight" if rng.random() < 0.7 else "bias"}', (n,)) for i, n in enumerate(sizes)]
+    chunk_size = int(max(sizes) + rng.integers(0, 30000))
+    dtype = [torch.float16, torch.bfloat16][seed % 2]
+    hyst, interval = int(rng.integers(1, 4)), int(rng.integers(2, 5))
+    loss_scale = float(2.0**rng.integers(0, 12)) if dtype == torch.float16 else 1.0
+    max_norm = float(rng.choice([0.0, 0.0, 1e-3, 0.05, 1.0]))
+    adamw = bool(rng.random() < 0.6)
+    kw = dict(initial_scale=loss_scale, hysteresis=hyst, growth_interval=interval) if dtype == torch.float16 else {}
+    module, opt, ochunks = build_workload(named, chunk_size, dtype, seed=seed, loss_scale=loss_scale, lr=3e-3,
+                                          weight_decay=float(rng.choice([0.0, 0.05])), adamw_mode=adamw,
+                                          max_norm=max_norm, **kw)
+    opt.gated_step = bool(rng.random() < 0.7)
+    scaler = (O.DynamicGradScalerOracle(initial_scale=loss_scale, min_scale=1, max_scale=2**24, hysteresis=hyst,
+                                        growth_interval=interval)
+              if dtype == torch.float16 else O.ConstantGradScalerOracle(1.0))
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(seed)
+    for step in range(7):
+        ls = float(opt.loss_scale)
+        fused = bool(rng.random() < 0.5)
+        payloads = []
+        for pc in module.param_chunks:
+            g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (float(rng.choice([1e-4, 2e-3, 0.3])) * ls)
+            g[pc.utilized_size:] = 0
+            g = g.to(dtype)
+            r = rng.random()
+            if r < 0.12 and pc.utilized_size > 0:
+                g[int(rng.integers(0, pc.utilized_size))] = float(rng.choice([np.inf, -np.inf, np.nan]))
+            elif r < 0.3 and pc.n_valid < pc.shard_size and not fused:
+                g[int(rng.integers(pc.n_valid, pc.shard_size))] = float('inf')    # garbage in the padding
+            payloads.append(g)
+        if fused:
+            land_chunks(list(module.param_chunks), payloads)
+        else:
+            for pc, g in zip(module.param_chunks, payloads):
+                pc.shard.copy_(g)
+                pc.invalidate_stats()
+        refresh_oracle_grads(module, ochunks)
+        tag = f'seed {seed} step {step} gated {opt.gated_step} fused {fused} {dtype} max_norm {max_norm}'
+        info = _run_and_compare(module, opt, ochunks, dtype, scaler, max_norm=max_norm, adamw_mode=adamw, tag=tag)
+        if info['found_inf'] or info['total_norm'] is None:
+            compare_state(module, opt, ochunks, dtype, exact=True, tag=tag)
+            continue
+        gmax = max(float(torch.nan_to_num(p.float(), posinf=0, neginf=0).abs().max()) for p in payloads) / ls
+        for i, (pc, oc) in enumerate(zip(module.param_chunks, ochunks)):
+            fc = pc.paired_chunk
+            m, v = opt._binding.moments(fc)
+            assert_close_f32(to_np(fc.shard), oc.master, f'{tag} chunk {i} master', rtol=2e-6, atol=1e-8)
+            assert_close_f32(to_np(m), oc.m, f'{tag} chunk {i} m', rtol=2e-6, atol=2e-6 * gmax)
+            assert_close_f32(to_np(v), oc.v, f'{tag} chunk {i} v', rtol=2e-6, atol=2e-6 * gmax * gmax)
+            want = O.writeback(to_np(fc.shard), CODE[dtype])
+            assert np.array_equal(to_np(pc.shard).view(np.uint16), want.view(np.uint16)), f'{tag} chunk {i} writeback'
+            # carry on from the GPU's state: every step is a comparison of its own
+            oc.master[:], oc.m[:], oc.v[:], oc.lowp[:] = to_np(fc.shard), to_np(m), to_np(v), to_np(pc.shard)
+
+
 @pytest.mark.parametrize('beta1', [0.9, 0.5, 0.0])
 @pytest.mark.parametrize('div_scale', [-1.0, 64.0, 48.0])
 @pytest.mark.parametrize('gdtype', [torch.float32, torch.float16, torch.bfloat16])
