@@ -18,6 +18,7 @@ not here: the replicated-cache block pool, the collectives and the tensor state 
 forward/backward pass.
 """
 import math
+import weakref
 from dataclasses import dataclass
 from enum import Enum
 from typing import Dict, List, Optional
@@ -140,7 +141,9 @@ LAND_BLOCKS_PER_CU = 0    # 0: the library default
 
 class StatsArena:
     """Device ElxStats records that landing launches leave behind, one slot per chunk, so that the
-    optimizer step can fetch the flags of all chunks with one device-to-host copy."""
+    optimizer step can fetch the flags of all chunks with one device-to-host copy.  Slots are handed
+    out in consecutive runs (the chunks of one landing sit side by side) and go back to the arena
+    when their chunk is given another slot or is garbage-collected."""
     CAPACITY = 8192
     _arenas: Dict[torch.device, 'StatsArena'] = {}
 
@@ -148,7 +151,7 @@ class StatsArena:
         self.device = device
         self.itemsize = _abi.STATS_DTYPE.itemsize
         self.buf = torch.zeros(self.CAPACITY * self.itemsize, dtype=torch.uint8, device=device)
-        self.next = 0
+        self.used = np.zeros(self.CAPACITY, dtype=bool)
 
     @classmethod
     def get(cls, device: torch.device) -> 'StatsArena':
@@ -159,12 +162,31 @@ class StatsArena:
         return arena
 
     def new_slots(self, count: int) -> int:
-        """First index of ``count`` consecutive fresh slots."""
-        if self.next + count > self.CAPACITY:
-            raise RuntimeError(f'more than {self.CAPACITY} stats slots in use on {self.device}')
-        first = self.next
-        self.next += count
-        return first
+        """First index of ``count`` consecutive free slots (first fit), now taken."""
+        assert count >= 1
+        if count <= self.CAPACITY:
+            filled = np.concatenate(([0], np.cumsum(self.used)))
+            runs = np.flatnonzero(filled[count:] == filled[:-count])    # windows without a used slot
+            if len(runs):
+                first = int(runs[0])
+                self.used[first:first + count] = True
+                return first
+        raise RuntimeError(f'no run of {count} free stats slots on {self.device} '
+                           f'({int(self.used.sum())} of {self.CAPACITY} in use)')
+
+    def release(self, slot: int) -> None:
+        self.used[slot] = False
+
+    def assign(self, chunks: List['Chunk']) -> None:
+        """Gives the chunks of one landing consecutive slots in list order, keeping the ones they hold
+        when those already are."""
+        slots = [c._stats_slot for c in chunks]
+        if slots[0] is not None and all(b is not None and b == a + 1 for a, b in zip(slots, slots[1:])) \
+                and all(c._stats_home[0] is self for c in chunks):
+            return
+        first = self.new_slots(len(chunks))
+        for i, c in enumerate(chunks):
+            c._take_stats_slot(self, first + i)
 
     def ptr(self, slot: int) -> int:
         return self.buf.data_ptr() + slot * self.itemsize
@@ -172,6 +194,13 @@ class StatsArena:
     def read(self, lo: int, hi: int) -> np.ndarray:
         """Slots [lo, hi) on the host: one blocking copy."""
         return self.buf[lo * self.itemsize:hi * self.itemsize].cpu().numpy().view(_abi.STATS_DTYPE).copy()
+
+
+def _release_stats_home(home: list) -> None:
+    """Finalizer of a chunk: its slot, if it still holds one, goes back to its arena."""
+    arena, slot = home
+    if arena is not None and slot is not None:
+        arena.release(slot)
 
 
 def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float = 1.0) -> None:
@@ -194,11 +223,7 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
         assert dtype_code(c.chunk_dtype) == dst_code and dtype_code(pl.dtype) == src_code
         assert pl.numel() == c.shard_size, 'the payload slice must cover the shard'
     arena = StatsArena.get(device)
-    slots = [c._stats_slot for c in chunks]
-    if slots[0] is None or any(b is None or b != a + 1 for a, b in zip(slots, slots[1:])):
-        first = arena.new_slots(len(chunks))
-        for i, c in enumerate(chunks):
-            c._stats_slot = first + i
+    arena.assign(chunks)
     rows = np.zeros(len(chunks), dtype=_abi.CHUNK_DTYPE)
     for i, (c, pl) in enumerate(zip(chunks, payloads)):
         rows[i]['grad'] = pl.data_ptr()
@@ -310,11 +335,7 @@ def land_tensors(chunks: List['Chunk'], grad_of, mul: float = 1.0) -> None:
         raise RuntimeError(f'{len(rows)} rows in one landing launch: land fewer chunks at a time')
 
     arena = StatsArena.get(device)
-    slots = [c._stats_slot for c in chunks]
-    if slots[0] is None or any(b is None or b != a + 1 for a, b in zip(slots, slots[1:])):
-        first = arena.new_slots(len(chunks))
-        for i, c in enumerate(chunks):
-            c._stats_slot = first + i
+    arena.assign(chunks)
     bpr = _abi.check_land_rows(rows, slot_offsets, src_code, dst_code)
     ws = chunks[0]._workspace
     need = _abi.land_workspace_records(len(rows), bpr, len(chunks)) * arena.itemsize
@@ -434,6 +455,8 @@ class Chunk:
         # True once overflow / l2_norm describe the gradients that sit in the shard now
         self._stats_fresh = False
         self._stats_slot: Optional[int] = None    # this chunk's record in the device arena
+        self._stats_home = [None, None]           # [arena, slot], shared with the finalizer that frees the slot
+        weakref.finalize(self, _release_stats_home, self._stats_home)
         self._stats_pending = False               # a landing launch has written it, nobody has read it
         self._stats_event = None                  # recorded behind that launch, on its stream
         self._workspace: Dict = {}
@@ -463,6 +486,14 @@ class Chunk:
     @l2_norm.setter
     def l2_norm(self, value: Optional[float]) -> None:
         self._l2_norm = value
+
+    def _take_stats_slot(self, arena: 'StatsArena', slot: int) -> None:
+        """This chunk's record moves to ``slot`` of ``arena``; the slot it held goes back."""
+        old_arena, old_slot = self._stats_home
+        if old_arena is not None and old_slot is not None:
+            old_arena.release(old_slot)
+        self._stats_slot = slot
+        self._stats_home[0], self._stats_home[1] = arena, slot
 
     def invalidate_stats(self) -> None:
         """The shard was written behind the chunk's back: forget flags and outstanding records."""

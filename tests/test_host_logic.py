@@ -512,3 +512,47 @@ def test_launch_plan_properties_random():
         assert covered == sum(se - sb for buf in bufs for sb, se, _ in buf.segs)
 
     check()
+
+
+def test_stats_arena_hands_out_runs_and_takes_them_back():
+    """Slots of the record arena: consecutive runs in list order, kept when a list lands again, given
+    back when a chunk moves to another run or is garbage-collected, and a clear error when no run is
+    free.  (The arena's buffer sits on the CPU here; nothing is launched.)"""
+    import gc
+    from elixir_amd.chunk import StatsArena
+
+    def chunk():
+        c = ea.Chunk(None, 64, torch.float16, None, shard_device='cpu', temp_device='cpu')
+        c.append_tensor(torch.zeros(8).half())
+        c.close_chunk()
+        return c
+
+    arena = StatsArena(torch.device('cpu'))
+    a, b, c = chunk(), chunk(), chunk()
+    arena.assign([a, b])
+    assert (a._stats_slot, b._stats_slot) == (0, 1)
+    arena.assign([a, b])                                     # the same list again: nothing moves
+    assert (a._stats_slot, b._stats_slot) == (0, 1) and arena.used.sum() == 2
+    arena.assign([b, c])                                     # b moves next to c; its old slot is free again
+    assert (b._stats_slot, c._stats_slot) == (2, 3) and list(np.flatnonzero(arena.used)) == [0, 2, 3]
+    arena.assign([a])
+    assert a._stats_slot == 0
+    arena.assign([a, b, c])                                  # a fresh run of three; 0, 2, 3 come back
+    assert [x._stats_slot for x in (a, b, c)] == [4, 5, 6] and list(np.flatnonzero(arena.used)) == [4, 5, 6]
+    d = chunk()
+    arena.assign([d])
+    assert d._stats_slot == 0                                # first fit reuses what was released
+    del d
+    gc.collect()
+    assert list(np.flatnonzero(arena.used)) == [4, 5, 6]     # a dead chunk gives its slot back
+    # churn: far more chunks over time than the arena has slots
+    for _ in range(3 * StatsArena.CAPACITY // 4):
+        xs = [chunk() for _ in range(4)]
+        arena.assign(xs)
+        del xs
+    gc.collect()
+    assert arena.used.sum() == 3
+    with pytest.raises(RuntimeError, match='free stats slots'):
+        arena.new_slots(StatsArena.CAPACITY - 2)
+    first = arena.new_slots(StatsArena.CAPACITY - 7)         # the longest free run is behind slot 6
+    assert first == 7
