@@ -154,6 +154,40 @@ def test_fp16_training_matches_master_weight_amp_and_recovers_from_overflow():
     assert opt.loss_scale == scale == 512.0
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_low_precision_training_is_bit_identical_to_a_master_weight_loop_with_the_same_optimizer(dtype):
+    """The shape of the reference's own test/wrapper/test_amp.py: the same optimizer on both sides, so
+    that the comparison pins the plumbing (packing, ranges, landing from hooks, unscale, writeback,
+    what the next forward pass sees) -- here to the bit: HybridAdam standing alone on an fp32 master
+    copy, fed the low-precision gradients of a rounded working copy and the loss scale as divisor."""
+    torch.manual_seed(0)
+    master = Net().to(DEV)
+    model = copy.deepcopy(master)
+    sopt = ea.HybridAdam(groups_of(master, 0.1), lr=1e-2, weight_decay=0.1)
+    scale = 256.0 if dtype == torch.float16 else 1.0
+    kw = dict(initial_scale=scale, hysteresis=1, growth_interval=1000) if dtype == torch.float16 else {}
+    module, opt = wrap(model, dtype, **kw)
+    gen = torch.Generator(device=DEV).manual_seed(2)
+    for step in range(5):
+        x = batch(gen)
+        work = copy.deepcopy(master).to(dtype)
+        (work(x) * scale).backward()
+        for p, w in zip(master.parameters(), work.parameters()):
+            p.grad_dtype = None    # an fp32 parameter carrying a low-precision gradient
+            p.grad = w.grad
+        sopt.step(div_scale=scale if scale != 1.0 else -1)
+        opt.zero_grad()
+        opt.backward(module(x))
+        opt.step()
+        assert opt.last_step_info['found_inf'] is False and opt.loss_scale == scale
+        module.materialize_params()
+        sd = module.state_dict()
+        for name, want in master.state_dict().items():
+            assert torch.equal(sd[name], want.cpu()), f'step {step} {name}'
+        for (name, p), w in zip(model.named_parameters(), master.parameters()):
+            assert torch.equal(p.data, w.data.to(dtype)), f'step {step} {name}: what the forward pass sees'
+
+
 def test_state_dict_round_trip_and_load():
     torch.manual_seed(3)
     model = Net().to(DEV)
