@@ -266,7 +266,7 @@ def offload_step_leg(mi_elements, steps=5):
             ts.append(time.perf_counter() - t0)
             assert opt.last_step_info['found_inf'] is False
         t = float(np.mean(ts[1:]))
-        out['blocks_per_cu_%d' % (bpc or 12)] = {'ms_per_step': t * 1e3, 'elements_per_sec': n / t,
+        out['blocks_per_cu_%d' % (bpc or 13)] = {'ms_per_step': t * 1e3, 'elements_per_sec': n / t,
                                                   'host_link_gbps_30B': 30 * n / t / 1e9}
     tc = float(np.median(cpu_s[1:]))
     out.update({'what': 'optimizer step over one host-resident (pinned) chunk pair, in place over the host link',

@@ -48,7 +48,8 @@ constexpr uint32_t kSpan = kWave * kVec;               // elements one wavefront
 constexpr uint32_t kTile = kSpan * kUnroll;            // 256 elements per tile
 constexpr uint64_t kMaxBufferElems = 1ull << 40;       // longest buffer a table row may describe (tile arithmetic stays far from overflow)
 constexpr uint32_t kLdsPerCu = 160u * 1024u;           // gfx950
-constexpr uint32_t kDefaultBlocksPerCu = 12;
+constexpr uint32_t kDefaultBlocksPerCu = 12;            // fp32 gradients (4 KiB of loads in flight per workgroup)
+constexpr uint32_t kDefaultBlocksPerCuLowp = 13;        // 16-bit gradients (3.5 KiB): one more workgroup pays
 constexpr uint32_t kMinBlocksPerCu = 3;                // keeps the reservation below 64 KiB
 constexpr uint32_t kMaxBlocksPerCu = 32;
 
@@ -898,8 +899,8 @@ bool exact_reciprocal(float s) {
 }
 
 // dynamic LDS bytes that let exactly `blocks_per_cu` update workgroups share a compute unit
-int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes) {
-    if (blocks_per_cu == 0) blocks_per_cu = kDefaultBlocksPerCu;
+int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes, uint32_t fallback = kDefaultBlocksPerCu) {
+    if (blocks_per_cu == 0) blocks_per_cu = fallback;
     if (blocks_per_cu < kMinBlocksPerCu || blocks_per_cu > kMaxBlocksPerCu) return ELX_E_SIZE;
     *lds_bytes = (kLdsPerCu / blocks_per_cu) & ~255u;
     return 0;
@@ -1073,7 +1074,8 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
     uint32_t lds = 0;
-    if (int rc = occupancy_reservation(blocks_per_cu, &lds)) return rc;
+    if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
+        return rc;
     Unscale us;
     us.div_scale = div_scale;
     us.inv_scale = 1.0f;
@@ -1111,7 +1113,8 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
     uint32_t lds = 0;
-    if (int rc = occupancy_reservation(blocks_per_cu, &lds)) return rc;
+    if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
+        return rc;
     Unscale us;
     us.div_scale = -1.0f;
     us.inv_scale = 1.0f;

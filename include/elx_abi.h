@@ -192,7 +192,8 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
  *                          over tile_begin;  otherwise the launch is a 2-D grid
  *                          (grid_tiles_per_chunk, n_chunks) without any lookup, and must be at least
  *                          the max_tiles_per_chunk that elx_check_tables reported (n_chunks <= 65535)
- *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (12).
+ *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (13 for
+ *                  16-bit gradients, 12 for fp32 gradients).
  *                  The update streams best with a shallow, orderly queue of memory requests.
  */
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
