@@ -27,7 +27,7 @@
 //   * every access is a fully coalesced 128-bit (fp32) / 64-bit (16-bit types) per-lane access,
 //     so one wavefront instruction covers one contiguous 1 KiB / 512 B span;
 //   * the number of resident workgroups per compute unit is capped through a dynamic LDS
-//     reservation (default 12), not by the register file;
+//     reservation (default 13 for 16-bit gradients, 12 for fp32 ones), not by the register file;
 //   * loads carry the non-temporal hint, stores go out non-temporal at agent scope.
 //
 // Arithmetic contract (what the parity tests pin): fp32 throughout, IEEE division and square
@@ -48,8 +48,8 @@ constexpr uint32_t kSpan = kWave * kVec;               // elements one wavefront
 constexpr uint32_t kTile = kSpan * kUnroll;            // 256 elements per tile
 constexpr uint64_t kMaxBufferElems = 1ull << 40;       // longest buffer a table row may describe (tile arithmetic stays far from overflow)
 constexpr uint32_t kLdsPerCu = 160u * 1024u;           // gfx950
-constexpr uint32_t kDefaultBlocksPerCu = 12;            // fp32 gradients (4 KiB of loads in flight per workgroup)
-constexpr uint32_t kDefaultBlocksPerCuLowp = 13;        // 16-bit gradients (3.5 KiB): one more workgroup pays
+constexpr uint32_t kDefaultBlocksPerCu = 12;           // fp32 gradients (4 KiB of loads in flight per workgroup)
+constexpr uint32_t kDefaultBlocksPerCuLowp = 13;       // 16-bit gradients (3.5 KiB): one more workgroup pays
 constexpr uint32_t kMinBlocksPerCu = 3;                // keeps the reservation below 64 KiB
 constexpr uint32_t kMaxBlocksPerCu = 32;
 
