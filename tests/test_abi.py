@@ -261,3 +261,23 @@ def test_check_tables_property_random():
             assert refused(rows, segs, 0)
 
     run()
+
+
+def test_missing_library_and_missing_gpu_fail_loudly(monkeypatch):
+    """There is no CPU path behind the optimizer: without the built library every entry raises and
+    says how to build it, and parameters that are not on a GPU are refused by name of the reason."""
+    import torch
+    import elixir_amd as ea
+    monkeypatch.setattr(_abi, '_lib', None)
+    monkeypatch.setattr(_abi, 'LIB_PATH', os.path.join(ROOT, 'elixir_amd', 'no_such_library.so'))
+    with pytest.raises(RuntimeError, match='has not been built'):
+        _abi.load()
+    with pytest.raises(RuntimeError, match='no CPU fallback'):
+        _abi.tile_elems()
+    monkeypatch.undo()
+    assert _abi.tile_elems() == 256
+    p = torch.nn.Parameter(torch.zeros(8))
+    p.grad = torch.ones(8)
+    with pytest.raises(RuntimeError, match='runs on the GPU'):
+        ea.HybridAdam([p]).step()
+    assert torch.count_nonzero(p.data) == 0          # nothing was updated by some other route
