@@ -169,3 +169,58 @@ def test_full_size_step_is_deterministic():
     assert b.optimizer.last_step_info == norm
     for (p0, l0), pc in zip(first, b.module.param_chunks):
         assert torch.equal(p0, pc.paired_chunk.shard) and torch.equal(l0, pc.shard)
+
+
+def test_one_buffer_beyond_two_to_the_32_elements():
+    """Element offsets are 64-bit everywhere: one flat fp32 parameter of 2**32 + 2**20 + 77 elements
+    with fp16 gradients goes through the update, the single-buffer stats and the single-buffer
+    refresh; windows at the start, across the 2**32 boundary and at the ragged end are replayed by
+    the oracle, and a non-finite value planted behind the boundary is found."""
+    import elixir_amd as ea
+    from elixir_amd import _abi
+    dev = 'cuda'
+    n = (1 << 32) + (1 << 20) + 77
+    gen = torch.Generator(device=dev).manual_seed(5)
+    p = torch.nn.Parameter(torch.empty(n, device=dev))
+    p.data.normal_(0, 0.02, generator=gen)
+    g = torch.empty(n, dtype=torch.float16, device=dev)
+    g.normal_(0, 0.5, generator=gen)
+    windows = [(0, 5000), ((1 << 32) - 3001, (1 << 32) + 2999), (n - 4000, n)]
+    pre = [(to_np(g[b:e]).copy(), to_np(p.data[b:e]).copy()) for b, e in windows]
+    opt = ea.HybridAdam([p], lr=1e-2, weight_decay=0.1)
+    p.grad_dtype = None
+    p.grad = g
+    opt.step(div_scale=48.0)
+    st = opt.state[p]
+    for (b, e), (gn, pn) in zip(windows, pre):
+        mn, vn = np.zeros(e - b, np.float32), np.zeros(e - b, np.float32)
+        O.adam(gn, O.F16, pn, mn, vn, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.1, step=1,
+               adamw_mode=True, div_scale=48.0)
+        for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
+            assert np.array_equal(to_np(got[b:e]).view(np.uint32), want.view(np.uint32)), (name, b, e)
+    # every element was updated exactly once: exp_avg = 0.1 * g / 48 everywhere
+    assert torch.equal(st['exp_avg'][::4099] != 0, g[::4099] != 0)
+    del st, opt
+    # single-buffer stats over the whole run, clean and with a NaN behind the 2**32 boundary
+    stream = torch.cuda.current_stream().cuda_stream
+    blocks = 1024
+    ws = torch.empty((blocks + 1) * 16, dtype=torch.uint8, device=dev)
+
+    def stats():
+        _abi.grad_stats(g.data_ptr(), O.F16, n, blocks, ws.data_ptr(), ws.data_ptr() + blocks * 16, stream)
+        return ws[blocks * 16:].cpu().numpy().view(_abi.STATS_DTYPE)[0]
+
+    rec = stats()
+    ref = sum(float(g[i:i + (1 << 28)].double().square().sum()) for i in range(0, n, 1 << 28))
+    assert rec['overflow'] == 0 and abs(float(rec['sumsq']) - ref) <= 1e-6 * ref
+    g[(1 << 32) + 12345] = float('nan')
+    assert stats()['overflow'] == 1
+    g[(1 << 32) + 12345] = 0.0
+    g[n - 1] = float('inf')
+    assert stats()['overflow'] == 1
+    # single-buffer refresh: the whole run, checked in the same windows
+    low = torch.zeros(n, dtype=torch.bfloat16, device=dev)
+    _abi.writeback(p.data.data_ptr(), low.data_ptr(), O.BF16, n, stream)
+    for b, e in windows:
+        assert torch.equal(low[b:e], p.data[b:e].to(torch.bfloat16)), (b, e)
+    assert int(torch.count_nonzero(low[::4099])) == int(torch.count_nonzero(p.data[::4099].to(torch.bfloat16)))
