@@ -672,6 +672,7 @@ __global__ __launch_bounds__(kStatsThreads) void stats_finish_kernel(const ElxSt
 constexpr int kLandUnroll = 4;
 constexpr uint32_t kMaxLandBlocks = 1u << 20;
 constexpr uint32_t kDefaultLandBlocksPerCu = 10;
+constexpr uint32_t kDefaultLandBlocksPerCuNarrowing = 13;    // fp32 payload into a 16-bit shard: half the bytes go out
 constexpr uint32_t kFoldBlocks = 64;           // first-stage workgroups per row when partials are many
 constexpr uint32_t kFoldThreshold = 2048;      // partials per row above which the fold has two stages
 
@@ -1200,7 +1201,9 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d
     const dim3 grid(blocks_per_row, n_rows), block(kWave);
     const uint32_t so = (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u;
     uint32_t lds = 0;
-    int rc = occupancy_reservation(((flags >> 8) & 0xFFu) ? ((flags >> 8) & 0xFFu) : kDefaultLandBlocksPerCu, &lds);
+    const uint32_t land_default = (src_dtype == ELX_F32 && dst_dtype != ELX_F32) ? kDefaultLandBlocksPerCuNarrowing
+                                                                                 : kDefaultLandBlocksPerCu;
+    int rc = occupancy_reservation(((flags >> 8) & 0xFFu) ? ((flags >> 8) & 0xFFu) : land_default, &lds);
     if (rc) return rc;
     rc = ELX_E_DTYPE;
 #define ELX_LAND(S, D)                                                                                       \

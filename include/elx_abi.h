@@ -282,7 +282,8 @@ int elx_grad_stats(const void *grad, int grad_dtype, uint64_t n, uint32_t blocks
  *   d_stats    n_slots results; fixed reduction order
  *   flags      ELX_FLAG_SCALAR_ONLY forces the element-by-element path (rows whose ends are not both
  *              16-byte aligned take it by themselves); bits 8..15: cap on resident workgroups per
- *              compute unit, 3..32 (0 = the library default, 10)
+ *              compute unit, 3..32 (0 = the library default: 10, or 13 when an fp32 payload lands in a
+ *              16-bit shard)
  */
 int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d_slot_offsets, uint32_t n_slots,
                       int src_dtype, int dst_dtype, float mul, uint32_t blocks_per_row, ElxStats *d_partials,
