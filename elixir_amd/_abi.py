@@ -65,8 +65,7 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
-                 'elx_sizeof_decision', 'elx_sizeof_decision', 'elx_decide', 'elx_adam_step_gated_mt',
-                 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks'):
+                 'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -95,7 +94,8 @@ def load() -> ctypes.CDLL:
 
     if L.elx_version() != ELX_ABI_VERSION:
         raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
-    for name, dt in (('chunk', CHUNK_DTYPE), ('seg', SEG_DTYPE), ('hyper', HYPER_DTYPE), ('stats', STATS_DTYPE)):
+    for name, dt in (('chunk', CHUNK_DTYPE), ('seg', SEG_DTYPE), ('hyper', HYPER_DTYPE), ('stats', STATS_DTYPE),
+                     ('decision', DECISION_DTYPE)):
         size = getattr(L, f'elx_sizeof_{name}')()
         if size != dt.itemsize:
             raise RuntimeError(f'{LIB_PATH}: sizeof {name} record is {size}, binding expects {dt.itemsize}')
