@@ -148,6 +148,9 @@ class ElixirModule(nn.Module):
         self._landing_in_backward = False
         self._ready: Dict[Chunk, set] = {}
         self._landed: set = set()
+        # set by the optimizer step: the shards hold new values that the module's parameters (private
+        # copies, as the blocks of the replicated cache are in the reference) have not seen yet
+        self._params_stale = False
         if not self.synthetic:
             for param in self.grad_state_dict.values():
                 param.register_post_accumulate_grad_hook(self._gradient_handler)
@@ -235,6 +238,7 @@ class ElixirModule(nn.Module):
         """Give every parameter of the wrapped module a private copy of its low-precision values
         (what a gather into the replicated cache would expose to the forward pass)."""
         assert not self.synthetic
+        self._params_stale = False
         blocks = {}
         for chunk in self.param_chunks:
             if not chunk.optim_sync_flag and torch.cuda.is_available():
@@ -250,8 +254,15 @@ class ElixirModule(nn.Module):
             src = blocks.get(chunk, chunk.shard)
             param.data = src[info.offset:info.end].clone().view(info.fake_data.shape)
 
+    def mark_params_stale(self) -> None:
+        """Called by the optimizer step: the next forward pass re-reads the parameters from the shards
+        (the reference's forward gathers its chunks anew after every step)."""
+        self._params_stale = True
+
     def forward(self, *args, **kwargs):
         assert not self.synthetic
+        if self._params_stale:
+            self.materialize_params()
         outputs = self.module(*args, **kwargs)
         if self.output_fp32:
             outputs = outputs.float()

@@ -288,6 +288,8 @@ class ElixirOptimizer:
 
         if not update_flag:
             return
+        if hasattr(self.module, 'mark_params_stale'):
+            self.module.mark_params_stale()    # the next forward pass reads the refreshed shards
         if self._binding is not None and self._binding.fused_writeback:
             self._binding.fused_writeback = False
             for param_chunk in self.param_chunk_set:

@@ -188,6 +188,32 @@ def test_low_precision_training_is_bit_identical_to_a_master_weight_loop_with_th
             assert torch.equal(p.data, w.data.to(dtype)), f'step {step} {name}: what the forward pass sees'
 
 
+def test_forward_after_a_step_sees_the_new_weights_without_being_told():
+    """The reference's forward pass gathers its chunks anew after every step; here the module's
+    parameters are private copies of the shards, refreshed by the first forward pass after a step.
+    A loop that never calls materialize_params must train exactly like one that does."""
+    torch.manual_seed(0)
+    base = Net().to(DEV)
+    runs = []
+    for explicit in (True, False):
+        model = copy.deepcopy(base)
+        module, opt = wrap(model, torch.float16, initial_scale=256.0, hysteresis=1)
+        gen = torch.Generator(device=DEV).manual_seed(7)
+        losses = []
+        for step in range(4):
+            loss = module(batch(gen))
+            losses.append(float(loss.detach()))
+            opt.zero_grad()
+            opt.backward(loss)
+            opt.step()
+            if explicit:
+                module.materialize_params()
+        runs.append((losses, {k: v.clone() for k, v in module.state_dict().items()}))
+    assert runs[0][0] == runs[1][0] and runs[0][0][0] != runs[0][0][-1]
+    for name, want in runs[0][1].items():
+        assert torch.equal(runs[1][1][name], want), name
+
+
 def test_state_dict_round_trip_and_load():
     torch.manual_seed(3)
     model = Net().to(DEV)
