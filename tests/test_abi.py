@@ -281,3 +281,25 @@ def test_missing_library_and_missing_gpu_fail_loudly(monkeypatch):
     with pytest.raises(RuntimeError, match='runs on the GPU'):
         ea.HybridAdam([p]).step()
     assert torch.count_nonzero(p.data) == 0          # nothing was updated by some other route
+
+
+def test_device_code_has_no_packed_fp32_and_no_spills(tmp_path):
+    """What the build flags promise about the device code, checked on the compiler's own listing:
+    no packed-fp32 arithmetic (the kernels' fp32 results must not depend on how the compiler pairs
+    lanes' operands), no register spills and no private memory in any kernel."""
+    import subprocess
+    from elixir_amd import build as B
+    asm = tmp_path / 'elx.s'
+    flags = [f for f in B.HIPCC_FLAGS if f not in ('-shared', '-fPIC')]
+    subprocess.run([B.hipcc_path()] + flags + ['--cuda-device-only', '-S', '-I', os.path.join(ROOT, 'include'), '-o', str(asm)]
+                   + B.SOURCES, check=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+    text = asm.read_text()
+    assert not re.search(r'\bv_pk_(add|mul|fma)_f32\b', text)
+    kernels = re.findall(r'\.amdhsa_kernel\s+(\S+)', text)
+    assert len(kernels) >= 30
+    for key in ('.private_segment_fixed_size', '.sgpr_spill_count', '.vgpr_spill_count'):
+        values = re.findall(re.escape(key) + r':\s*(\d+)', text)
+        assert len(values) == len(kernels) and set(values) == {'0'}, (key, set(values))
+    # the update kernels keep a small register footprint: residency is capped by the LDS reservation, not by registers
+    vgprs = [int(v) for v in re.findall(r'\.vgpr_count:\s*(\d+)', text)]
+    assert max(vgprs) <= 128
