@@ -195,7 +195,7 @@ def refresh_piece_elems() -> int:
 def writeback_mt(d_chunks: int, n_chunks: int, lowp_dtype: int, max_elems: int, aligned: bool, stream: int) -> None:
     """``max_elems``: the largest n_alloc among the records (sizes the grid)."""
     piece = refresh_piece_elems()
-    blocks = max(1, min(4096, (max_elems + piece - 1) // piece))
+    blocks = max(1, min(1 << 20, (max_elems + piece - 1) // piece))    # one piece per workgroup
     check('elx_writeback_mt',
           load().elx_writeback_mt(d_chunks, n_chunks, lowp_dtype, blocks, 0 if aligned else ELX_FLAG_SCALAR_ONLY, stream))
 

@@ -482,11 +482,16 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
 // ---------------------------------------------------------------------------------------------
 
 // lowp_out[0, n_alloc) = round-to-nearest-even(master) for every chunk.  4 bytes in, 2 bytes out per
-// element: a read-dominated stream that wants wide workgroups and a deep queue, the opposite of
-// the update.  Grid (blocks_per_chunk, n_chunks), each workgroup strides over 4096-element pieces.
-constexpr int kRefreshThreads = 256;
+// element.  The same shape as the landing launch (which, for an fp32 payload and a 16-bit shard, is
+// this copy plus the flags): one wavefront per workgroup, one piece of four 128-bit loads per lane,
+// residency capped through the LDS reservation, pieces handed out in address order.  Grid
+// (blocks_per_chunk, n_chunks); a workgroup takes several pieces only when a record has more pieces
+// than the grid has blocks.
+constexpr int kRefreshThreads = kWave;
 constexpr int kRefreshUnroll = 4;
-constexpr uint32_t kRefreshPiece = kRefreshThreads * kVec * kRefreshUnroll;
+constexpr uint32_t kRefreshPiece = kRefreshThreads * kVec * kRefreshUnroll;    // 1024 elements
+constexpr uint32_t kRefreshBlocksPerCu = 13;
+constexpr uint32_t kMaxRefreshBlocks = 1u << 20;
 
 template <int LD>
 __device__ __forceinline__ void refresh_body(const ElxChunk &c, uint32_t scalar_only) {
@@ -499,17 +504,18 @@ __device__ __forceinline__ void refresh_body(const ElxChunk &c, uint32_t scalar_
     for (uint64_t piece = blockIdx.x; piece < pieces; piece += gridDim.x) {
         const uint64_t base = piece * kRefreshPiece;
         if (base + kRefreshPiece <= n && !scalar_only) {
-            const f32x4 *pp = reinterpret_cast<const f32x4 *>(c.master + base) + threadIdx.x;
-            lvec *lp = reinterpret_cast<lvec *>(out + base) + threadIdx.x;
+            const __amdgpu_buffer_rsrc_t pr = tile_rsrc(c.master + base, kRefreshPiece * sizeof(float));
+            const __amdgpu_buffer_rsrc_t lr = tile_rsrc(out + base, kRefreshPiece * sizeof(lscalar));
             f32x4 P[kRefreshUnroll];
 #pragma unroll
-            for (int u = 0; u < kRefreshUnroll; ++u) P[u] = ld_stream(pp + u * kRefreshThreads);
+            for (int u = 0; u < kRefreshUnroll; ++u)
+                P[u] = TileIo<f32x4>::load(pr, (threadIdx.x + u * kRefreshThreads) * (uint32_t)sizeof(f32x4));
 #pragma unroll
             for (int u = 0; u < kRefreshUnroll; ++u) {
                 lvec L;
 #pragma unroll
                 for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
-                __builtin_nontemporal_store(L, lp + u * kRefreshThreads);
+                TileIo<lvec>::store(lr, (threadIdx.x + u * kRefreshThreads) * (uint32_t)sizeof(lvec), L);
             }
         } else {
             const uint64_t left = n - base;
@@ -1127,14 +1133,16 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
 int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype, uint32_t blocks_per_chunk,
                      uint32_t flags, void *stream) {
     if (!d_chunks) return ELX_E_NULL;
-    if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > 65535u) return ELX_E_SIZE;
+    if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxRefreshBlocks) return ELX_E_SIZE;
     const dim3 grid(blocks_per_chunk, n_chunks);
     const uint32_t so = (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u;
     hipStream_t st = (hipStream_t)stream;
+    uint32_t lds = 0;
+    if (int rc = occupancy_reservation(kRefreshBlocksPerCu, &lds)) return rc;
     switch (lowp_dtype) {
-        case ELX_F32: hipLaunchKernelGGL((refresh_kernel<ELX_F32>), grid, dim3(kRefreshThreads), 0, st, d_chunks, so); break;
-        case ELX_F16: hipLaunchKernelGGL((refresh_kernel<ELX_F16>), grid, dim3(kRefreshThreads), 0, st, d_chunks, so); break;
-        case ELX_BF16: hipLaunchKernelGGL((refresh_kernel<ELX_BF16>), grid, dim3(kRefreshThreads), 0, st, d_chunks, so); break;
+        case ELX_F32: hipLaunchKernelGGL((refresh_kernel<ELX_F32>), grid, dim3(kRefreshThreads), lds, st, d_chunks, so); break;
+        case ELX_F16: hipLaunchKernelGGL((refresh_kernel<ELX_F16>), grid, dim3(kRefreshThreads), lds, st, d_chunks, so); break;
+        case ELX_BF16: hipLaunchKernelGGL((refresh_kernel<ELX_BF16>), grid, dim3(kRefreshThreads), lds, st, d_chunks, so); break;
         default: return ELX_E_DTYPE;
     }
     return (int)hipGetLastError();
@@ -1153,12 +1161,14 @@ int elx_writeback(const float *master, void *lowp, int lowp_dtype, uint64_t n, v
     c.n_alloc = n;
     const uint32_t so = (((uintptr_t)master | (uintptr_t)lowp) & 15u) ? 1u : 0u;
     const uint64_t pieces = (n + kRefreshPiece - 1) / kRefreshPiece;
-    const dim3 grid((uint32_t)(pieces < 4096 ? pieces : 4096));
+    const dim3 grid((uint32_t)(pieces < kMaxRefreshBlocks ? pieces : kMaxRefreshBlocks));
     hipStream_t st = (hipStream_t)stream;
+    uint32_t lds = 0;
+    if (int rc = occupancy_reservation(kRefreshBlocksPerCu, &lds)) return rc;
     switch (lowp_dtype) {
-        case ELX_F32: hipLaunchKernelGGL((refresh_one_kernel<ELX_F32>), grid, dim3(kRefreshThreads), 0, st, c, so); break;
-        case ELX_F16: hipLaunchKernelGGL((refresh_one_kernel<ELX_F16>), grid, dim3(kRefreshThreads), 0, st, c, so); break;
-        default: hipLaunchKernelGGL((refresh_one_kernel<ELX_BF16>), grid, dim3(kRefreshThreads), 0, st, c, so); break;
+        case ELX_F32: hipLaunchKernelGGL((refresh_one_kernel<ELX_F32>), grid, dim3(kRefreshThreads), lds, st, c, so); break;
+        case ELX_F16: hipLaunchKernelGGL((refresh_one_kernel<ELX_F16>), grid, dim3(kRefreshThreads), lds, st, c, so); break;
+        default: hipLaunchKernelGGL((refresh_one_kernel<ELX_BF16>), grid, dim3(kRefreshThreads), lds, st, c, so); break;
     }
     return (int)hipGetLastError();
 }

@@ -9,7 +9,8 @@ left out of that launch and refreshed by the wide-workgroup refresh launch inste
 segments into
   * ``rows`` / ``segs``: the ElxChunk / ElxSeg tables of the update launch, one row per block of
     ``block_elems`` elements that contains at least one valid element;
-  * ``refresh_rows``: ElxChunk rows (lowp_out, master, n_alloc only) for the padding runs, or None.
+  * ``refresh_rows``: ElxChunk rows (lowp_out, master, n_alloc only) for the padding runs, cut into
+    blocks of the same size, or None.
 """
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence, Tuple
@@ -90,9 +91,11 @@ def build_plan(buffers: Sequence[FlatBuffer], grad_esize: int, lowp_esize: int, 
                          buf.master + 4 * b, buf.m + 4 * b, buf.v + 4 * b, n, max(0, min(n, buf.n_valid - b)), tiles,
                          seg_begin, len(segs)))
             tiles += (n + tile - 1) // tile
-        if buf.lowp_out and up_end < buf.n_alloc:
-            refresh.append((0, buf.lowp_out + up_end * lowp_esize, buf.master + 4 * up_end, buf.master + 4 * up_end,
-                            buf.master + 4 * up_end, buf.n_alloc - up_end, 0, 0, 0, 0))
+        if buf.lowp_out:
+            # the run of pure padding, in blocks of the same size: an even grid for the refresh launch
+            for b in range(up_end, buf.n_alloc, block):
+                refresh.append((0, buf.lowp_out + b * lowp_esize, buf.master + 4 * b, buf.master + 4 * b,
+                                buf.master + 4 * b, min(block, buf.n_alloc - b), 0, 0, 0, 0))
     rows_np = np.array(rows, dtype=_abi.CHUNK_DTYPE) if rows else np.zeros(0, dtype=_abi.CHUNK_DTYPE)
     segs_np = np.array(segs, dtype=_abi.SEG_DTYPE) if segs else np.zeros(0, dtype=_abi.SEG_DTYPE)
     info = _abi.check_tables(rows_np, segs_np, n_hypers, grad_dtype, lowp_dtype) if len(rows_np) else None

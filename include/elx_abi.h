@@ -185,8 +185,8 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
  *
  * A "chunk" of this table need not be a whole shard: callers get the best throughput by listing
  * equal-sized blocks of the shards that contain tensors as separate records and leaving runs of
- * pure padding to elx_writeback_mt (the update wants a shallow queue of small tiles, the refresh
- * a deep queue of large ones).
+ * pure padding to elx_writeback_mt (whose workgroups move four times as much per tile and read
+ * no tables).
  *   total_tiles            as returned by elx_check_tables for these tables
  *   grid_tiles_per_chunk   0: flat grid of total_tiles workgroups, each finds its chunk by a search
  *                          over tile_begin;  otherwise the launch is a 2-D grid
@@ -231,13 +231,14 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
  * record (only lowp_out, master and n_alloc are read).  The skip-step branch
  * (optimizer.py:196-203 -> chunk.py:403-414), state loading (elixir/wrapper/module.py:343) and the
  * padding runs left out of an update launch use it.
- *   blocks_per_chunk  workgroups per record, 1..65535; each strides over pieces of
- *                     elx_refresh_piece_elems() elements
+ *   blocks_per_chunk  workgroups per record, 1..2^20; best: ceil(max n_alloc / elx_refresh_piece_elems()),
+ *                     one piece per workgroup, with records of about equal size (with fewer, a
+ *                     workgroup takes several pieces)
  */
 int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype, uint32_t blocks_per_chunk,
                      uint32_t flags, void *stream);
 
-/* Elements one workgroup of the refresh launch handles per stride. */
+/* Elements of one piece of the refresh launch (one wavefront, four 128-bit loads per lane). */
 uint32_t elx_refresh_piece_elems(void);
 
 /*

@@ -126,7 +126,7 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_writeback_mt(None, 1, _abi.ELX_F16, 4, 0, None) == -1
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_NONE, 4, 0, None) == -2
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_F16, 0, 0, None) == -7
-    assert lib.elx_refresh_piece_elems() == 4096
+    assert lib.elx_refresh_piece_elems() == 1024
 
 
 def test_check_land_rows_accepts_and_rejects():

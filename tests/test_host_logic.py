@@ -502,8 +502,14 @@ def test_launch_plan_properties_random():
             up_end = pos
             assert up_end >= buf.n_valid and (up_end == buf.n_alloc or up_end % B == 0)
             if plan.refresh_rows is not None and buf.lowp_out:
-                tail = [r for r in plan.refresh_rows if r['master'] == buf.master + 4 * up_end]
-                assert (len(tail) == 1 and tail[0]['n_alloc'] == buf.n_alloc - up_end) or up_end == buf.n_alloc
+                # the padding run behind the update rows is tiled by refresh rows of at most one block
+                tail = sorted((int(r['master']), int(r['n_alloc'])) for r in plan.refresh_rows
+                              if buf.master + 4 * up_end <= r['master'] < buf.master + 4 * buf.n_alloc)
+                at = buf.master + 4 * up_end
+                for addr, cnt in tail:
+                    assert addr == at and 0 < cnt <= B
+                    at += 4 * cnt
+                assert at == buf.master + 4 * buf.n_alloc
             else:
                 assert up_end == buf.n_alloc or not buf.lowp_out
             for sb, se, h in buf.segs:    # the ends of every segment are covered with the right hyper index
