@@ -1,10 +1,18 @@
 """Shared pieces of the parity tests: seeded chunk sets on the GPU and their oracle twins."""
+import os
+
 import numpy as np
 import torch
 
 import elixir_amd as ea
 from elixir_amd import shapes as S
 from oracle import oracle as O
+
+
+def seeds(n: int) -> range:
+    """Seeds of a randomised test: ``n`` in the committed suite, ``n + ELX_EXTRA_SEEDS`` when that
+    environment variable is set (a long sweep: ``ELX_EXTRA_SEEDS=5000 python -m pytest tests -m gpu -k random``)."""
+    return range(n + int(os.environ.get('ELX_EXTRA_SEEDS', '0')))
 
 CODE = {torch.float32: O.F32, torch.float16: O.F16, torch.bfloat16: O.BF16}
 

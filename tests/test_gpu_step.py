@@ -18,7 +18,7 @@ from elixir_amd import shapes as S
 from elixir_amd.chunk import run_grad_stats
 from oracle import oracle as O
 
-from helpers import (CODE, assert_close_f32, build_workload, compare_state, from_bits, refresh_oracle_grads, to_np,
+from helpers import (CODE, assert_close_f32, build_workload, compare_state, from_bits, refresh_oracle_grads, seeds, to_np,
                      ulp_distance)
 
 pytestmark = pytest.mark.gpu
@@ -199,7 +199,7 @@ def test_flat_fp16_grads_fp32_params(oracle):
     assert np.array_equal(to_np(p.data).view(np.uint32), pn.view(np.uint32))
 
 
-@pytest.mark.parametrize('seed', range(12))
+@pytest.mark.parametrize('seed', seeds(12))
 def test_flat_random_hypers_match_oracle(oracle, seed):
     """Hyper-parameters, gradient type and divisor drawn at random, the edges included (beta1 of 0 and
     of exactly 0.5, beta2 of 0, no bias correction, a divisor that is not a power of two, two groups
@@ -530,7 +530,7 @@ def test_abi_rejects_bad_tables():
 # ------------------------------------------------------------------------------------------------
 
 
-@pytest.mark.parametrize('seed', list(range(16)))
+@pytest.mark.parametrize('seed', seeds(16))
 def test_random_layouts_match_oracle(oracle, seed):
     """Whatever the packing looks like -- boundaries inside vectors, tensors of one element, chunks
     that are not a multiple of the tile, a padded tail or none -- an unclipped step is bit-identical
@@ -567,7 +567,7 @@ def test_random_layouts_match_oracle(oracle, seed):
         assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'seed {seed} step {step}') == 0
 
 
-@pytest.mark.parametrize('seed', range(12))
+@pytest.mark.parametrize('seed', seeds(12))
 def test_random_trajectories_match_oracle(oracle, seed):
     """Seven steps on a random layout with everything drawn at random: hysteresis and growth interval of
     the scaler, clipping threshold, non-finite values in valid data (skip, back-off) or in the padding

@@ -16,6 +16,8 @@ import torch
 from oracle import oracle as O
 from oracle.torch_ref import TorchCpuStep
 
+from helpers import seeds
+
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'step_cases.npz')
 CODE = {'f32': O.F32, 'f16': O.F16, 'bf16': O.BF16}
 TORCH = {'f32': torch.float32, 'f16': torch.float16, 'bf16': torch.bfloat16}
@@ -163,7 +165,7 @@ def test_adam_against_live_torch_cpu(oracle, adamw, wd, betas):
         p[:], m[:], v[:] = want_p, st['exp_avg'].numpy(), st['exp_avg_sq'].numpy()
 
 
-@pytest.mark.parametrize('seed', range(12))
+@pytest.mark.parametrize('seed', seeds(12))
 def test_adam_against_live_torch_cpu_random_hypers(oracle, seed):
     """Hyper-parameters drawn at random, the edges included (beta1 of 0 and exactly 0.5, where torch's
     lerp changes formula; beta2 of 0; a large eps; no decay): every step compared on its own."""
