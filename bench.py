@@ -1,13 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the optimizer step (ElixirOptimizer.step over chunk-packed parameters) on one GPU.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c2|c1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c2|c1|velocity]
 
 A step is one full pass of the hot path over one set of synthetic gradients that already sit in
-the low-precision chunk shards: stats launch (overflow flag + sum of squares) -> 16 B/chunk
-device-to-host copy -> host scalars -> fused unscale + AdamW + low-precision writeback launch.
-Step time is host wall-clock between two device synchronisations, so host overhead counts.
-Prints ONE JSON line.
+the low-precision chunk shards: stats launch (overflow flag + sum of squares) -> decision kernel
+(skip, global norm, combined scale) -> fused unscale + AdamW + low-precision writeback launch ->
+refresh of the padding; the flags and the decision reach the host on a side stream for its
+bookkeeping.  Step time is host wall-clock between two device synchronisations, so host overhead
+counts.  Prints ONE JSON line.
 """
 import argparse
 import json
