@@ -35,7 +35,7 @@ EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 
            'elx_sizeof_stats', 'elx_sizeof_decision', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
            'elx_decide', 'elx_adam_step_gated_mt', 'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_writeback',
            'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems',
-           'elx_land_fold_blocks')
+           'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials')
 
 
 class ElxError(RuntimeError):
@@ -65,7 +65,7 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
-                 'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks'):
+                 'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -73,6 +73,8 @@ def load() -> ctypes.CDLL:
                                    ctypes.POINTER(cint)]
     L.elx_grad_stats_mt.restype = cint
     L.elx_grad_stats_mt.argtypes = [vp, u32, cint, u32, vp, vp, cint, vp]
+    L.elx_grad_stats_mt_static.restype = cint
+    L.elx_grad_stats_mt_static.argtypes = [vp, u32, cint, u32, vp, cint, vp]
     L.elx_adam_step_mt.restype = cint
     L.elx_adam_step_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_decide.restype = cint
@@ -161,6 +163,19 @@ def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chun
     check('elx_grad_stats_mt',
           load().elx_grad_stats_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, d_stats,
                                    int(scalar_only), stream))
+
+
+def static_partials() -> int:
+    return int(load().elx_static_partials())
+
+
+def grad_stats_mt_static(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_stats: int,
+                         scalar_only: bool, stream: int) -> None:
+    """``grad_stats_mt`` with the partials in the library's fixed device array: allocates nothing.  The
+    stream's device must be the current one; overlapping calls on one GPU race."""
+    check('elx_grad_stats_mt_static',
+          load().elx_grad_stats_mt_static(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_stats, int(scalar_only),
+                                          stream))
 
 
 def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int, info: TableInfo,

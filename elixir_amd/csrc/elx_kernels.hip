@@ -37,7 +37,18 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "elx_abi.h"
+
+// Partials workspace of elx_grad_stats_mt_static, the one entry point that takes no workspace from
+// its caller and allocates none: every GPU the library runs on holds this array until the process
+// ends.  In host code the name is only a handle for hipGetSymbolAddress; launches get the address
+// that call returned for the current device (scratch_of_current_device below).  No kernel names the
+// array: the compiler keeps it, and gives it the external linkage the runtime's lookup needs, because
+// host code names it (an explicit `used` attribute would keep it internal and the lookup would fail).
+constexpr uint32_t kStaticPartials = 65536;    // ElxStats records: 1 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticPartials * sizeof(ElxStats)];
 
 namespace {
 
@@ -943,6 +954,27 @@ int dispatch_step(int gd, int ld, uint32_t tiles, uint32_t lds, hipStream_t st, 
     return ELX_E_DTYPE;
 }
 
+// Device address of `scratch` on the current device, looked up once per device (each GPU holds its own
+// copy of the array at its own address).
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+int scratch_of_current_device(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return ELX_E_SIZE;
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return ELX_E_NULL;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);    // two threads racing here store the same address
+    }
+    *out = ptr;
+    return 0;
+}
+
 }    // namespace
 
 extern "C" {
@@ -1068,6 +1100,22 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(stats_finish_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, st, d_partials, blocks_per_chunk, d_stats);
     return (int)hipGetLastError();
+}
+
+uint32_t elx_static_partials(void) { return kStaticPartials; }
+
+int elx_grad_stats_mt_static(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
+                             ElxStats *d_stats, int scalar_only, void *stream) {
+    if (!d_chunks || !d_stats) return ELX_E_NULL;
+    if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxStatsBlocks)
+        return ELX_E_SIZE;
+    if ((uint64_t)n_chunks * blocks_per_chunk > kStaticPartials) return ELX_E_SIZE;
+    if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
+    void *partials = nullptr;
+    if (int rc = scratch_of_current_device(&partials)) return rc;
+    // every partial the finish launch reads is written by the stats launch first: nothing to clear
+    return elx_grad_stats_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, reinterpret_cast<ElxStats *>(partials),
+                             d_stats, scalar_only, stream);
 }
 
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,

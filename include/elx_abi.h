@@ -13,7 +13,8 @@
  * Conventions
  *   - plain C, no C++ or torch types; every pointer in a table is a DEVICE pointer;
  *   - the caller owns all memory (chunk buffers, tables, workspaces); the library allocates
- *     nothing and keeps no mutable global state; all entry points are reentrant;
+ *     nothing and keeps no mutable global state; all entry points are reentrant (the one exception,
+ *     elx_grad_stats_mt_static, says so in its own comment);
  *   - all device work is enqueued on the hipStream_t passed as `stream` (NULL = default
  *     stream) and is asynchronous with respect to the host; borrowed pointers must stay valid
  *     until that work has completed;
@@ -174,6 +175,26 @@ int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *
  */
 int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
                       ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream);
+
+/*
+ * elx_grad_stats_mt without a workspace argument, for callers that cannot allocate one (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  The partials go into a fixed array of elx_static_partials() ElxStats records (1 MiB)
+ * that the library holds in the memory of every GPU it runs on until the process ends; the call
+ * allocates and frees nothing.  Same kernels, same reduction order, same results as
+ * elx_grad_stats_mt.
+ *   - n_chunks * blocks_per_chunk must not exceed elx_static_partials(): ELX_E_SIZE otherwise;
+ *   - the device that owns `stream` must be the current device of the calling thread (the array's
+ *     address is looked up once per device, on the first call there);
+ *   - all calls on one GPU share the array: two calls whose work overlaps on that GPU (different
+ *     streams, or different threads) race.  Calls on one stream are ordered and safe; the array keeps
+ *     the last call's partials, and every record a call reads it has written first.
+ */
+int elx_grad_stats_mt_static(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
+                             ElxStats *d_stats, int scalar_only, void *stream);
+
+/* Capacity, in ElxStats records, of the fixed partials array of elx_grad_stats_mt_static. */
+uint32_t elx_static_partials(void);
 
 /*
  * Fused update over every chunk: for each element inside a segment
