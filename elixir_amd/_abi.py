@@ -179,13 +179,11 @@ def grad_stats_mt_static(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_p
 
 
 def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int, info: TableInfo,
-                 div_scale: float, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int, stream: int,
-                 flat_grid: bool = False) -> None:
-    """2-D grid (max tiles per chunk, chunks) unless ``flat_grid`` or there are too many chunks."""
-    grid_tiles = 0 if (flat_grid or n_chunks > 65535) else info.max_tiles
+                 div_scale: float, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int, stream: int) -> None:
+    """2-D grid (max tiles per record, records)."""
     check('elx_adam_step_mt',
-          load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles, grid_tiles,
-                                  div_scale, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
+          load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles,
+                                  info.max_tiles, div_scale, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
 
 
 def decide(d_stats: int, n_chunks: int, loss_scale: float, max_norm: float, clipping: bool, d_hypers: int,
@@ -197,10 +195,9 @@ def decide(d_stats: int, n_chunks: int, loss_scale: float, max_norm: float, clip
 def adam_step_gated_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int,
                        info: TableInfo, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int, stream: int) -> None:
     """``adam_step_mt`` with the unscale parameters and the skip flag read from the hyper records."""
-    grid_tiles = 0 if n_chunks > 65535 else info.max_tiles
     check('elx_adam_step_gated_mt',
           load().elx_adam_step_gated_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles,
-                                        grid_tiles, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
+                                        info.max_tiles, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
 
 
 def refresh_piece_elems() -> int:

@@ -366,34 +366,16 @@ static_assert(sizeof(ElxChunk) == 72, "load_chunk_row reads nine 64-bit words");
 // enqueued before the host knows whether the step happens.  They arrive with the hyper record the
 // tile loads anyway; on a skip the tile only refreshes its low-precision copy.
 template <int GD, int LD, bool GATED>
-__global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks, uint32_t n_chunks,
+__global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks,
                                                           const ElxSeg *__restrict__ segs,
-                                                          const ElxHyper *__restrict__ hypers,
-                                                          uint32_t grid_tiles_per_chunk, Unscale us,
+                                                          const ElxHyper *__restrict__ hypers, Unscale us,
                                                           uint32_t scalar_only) {
-    // chunk that owns this tile: on the 2-D grid (tiles, chunks) nothing has to be looked up
-    // (workgroups beyond a chunk's last tile exit); on the flat grid the owner is the last chunk
-    // whose tile_begin is <= the tile index (all uniform -> scalar loads)
-    uint32_t ci, local_tile;
-    if (grid_tiles_per_chunk) {
-        ci = blockIdx.y;
-        local_tile = blockIdx.x;
-    } else {
-        const uint32_t t = blockIdx.x;
-        uint32_t lo = 0, hi = n_chunks;
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (chunks[mid].tile_begin <= t)
-                lo = mid;
-            else
-                hi = mid;
-        }
-        ci = lo;
-        local_tile = t - (uint32_t)chunks[lo].tile_begin;
-    }
+    // 2-D grid (tiles, records): blockIdx.y names the record, blockIdx.x the tile; nothing is looked
+    // up, and workgroups beyond a record's last tile exit
+    const uint32_t ci = blockIdx.y, local_tile = blockIdx.x;
     const ElxChunk c = load_chunk_row(chunks + ci);
     const uint64_t base = (uint64_t)local_tile * kTile;
-    if (base >= c.n_alloc) return;    // a shorter chunk on the 2-D grid
+    if (base >= c.n_alloc) return;    // a shorter record
 
     typedef typename Elem<GD>::vec4 gvec;
     typedef typename Elem<GD>::scalar gscalar;
@@ -925,25 +907,24 @@ int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes, uint32_t 
 }
 
 template <int GD, int LD>
-int launch_step(uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
-                const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated,
-                uint32_t scalar_only) {
-    const dim3 grid = grid_tiles ? dim3(grid_tiles, n_chunks) : dim3(tiles);
+int launch_step(uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks, const ElxSeg *segs,
+                const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, uint32_t scalar_only) {
+    const dim3 grid(grid_tiles, n_chunks);
     if (gated)
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true>), grid, dim3(kWave), lds, st, chunks, n_chunks, segs, hypers,
-                           grid_tiles, us, scalar_only);
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+                           scalar_only);
     else
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false>), grid, dim3(kWave), lds, st, chunks, n_chunks, segs, hypers,
-                           grid_tiles, us, scalar_only);
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+                           scalar_only);
     return (int)hipGetLastError();
 }
 
-int dispatch_step(int gd, int ld, uint32_t tiles, uint32_t lds, hipStream_t st, const ElxChunk *chunks,
-                  uint32_t n_chunks, const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us,
-                  bool gated, uint32_t scalar_only) {
-#define ELX_CASE(G, L)                                                                                         \
-    if (gd == G && ld == L)                                                                                    \
-        return launch_step<G, L>(tiles, lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, scalar_only);
+int dispatch_step(int gd, int ld, uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
+                  const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated,
+                  uint32_t scalar_only) {
+#define ELX_CASE(G, L)                                                                                   \
+    if (gd == G && ld == L)                                                                              \
+        return launch_step<G, L>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -1125,7 +1106,7 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
     if (!d_chunks || (n_segs && (!d_segs || !d_hypers))) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u || total_tiles == 0 || total_tiles > 0x7FFFFFFFull || (n_segs && n_hypers == 0))
         return ELX_E_SIZE;
-    if (grid_tiles_per_chunk && (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
+    if (grid_tiles_per_chunk == 0 || (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
     uint32_t lds = 0;
@@ -1143,8 +1124,8 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
             us.mode = kDivTrue;
         }
     }
-    return dispatch_step(grad_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
-                         d_segs, d_hypers, grid_tiles_per_chunk, us, false, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+    return dispatch_step(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, d_chunks, n_chunks, d_segs, d_hypers,
+                         grid_tiles_per_chunk, us, false, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
 int elx_decide(const ElxStats *d_stats, uint32_t n_chunks, double loss_scale, double max_norm, int clipping,
@@ -1164,7 +1145,7 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
     if (!d_chunks || (n_segs && (!d_segs || !d_hypers))) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u || total_tiles == 0 || total_tiles > 0x7FFFFFFFull || (n_segs && n_hypers == 0))
         return ELX_E_SIZE;
-    if (grid_tiles_per_chunk && (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
+    if (grid_tiles_per_chunk == 0 || (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
     uint32_t lds = 0;
@@ -1174,8 +1155,8 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
     us.div_scale = -1.0f;
     us.inv_scale = 1.0f;
     us.mode = kDivNone;
-    return dispatch_step(grad_dtype, lowp_dtype, (uint32_t)total_tiles, lds, (hipStream_t)stream, d_chunks, n_chunks,
-                         d_segs, d_hypers, grid_tiles_per_chunk, us, true, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+    return dispatch_step(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, d_chunks, n_chunks, d_segs, d_hypers,
+                         grid_tiles_per_chunk, us, true, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
 int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype, uint32_t blocks_per_chunk,

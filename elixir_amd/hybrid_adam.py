@@ -447,14 +447,10 @@ class HybridAdam(torch.optim.Optimizer):
         self._bound_entries = (signature, entries)
         return entries
 
-    def _prepare_bound(self, hypers: Dict) -> Optional[_Prepared]:
-        b = self._binding
-        b.require_gpu()
-        entries = self._walk_bound()
-        if not entries:
-            return None
+    def _bound_hyper_indices(self, entries, hypers: Dict) -> List[int]:
+        """Index of the hyper record of every bound entry -- the (group, step + 1) pair it will be
+        updated with -- filling ``hypers`` on the way.  Host arithmetic only."""
         groups = self.param_groups
-        # hyper record per entry: the (group, step + 1) pair it will be updated with
         seen: Dict = {}    # (group, step) -> hyper index: nearly always one step count per group
         idx_of = []
         for state, gi, _, _, _ in entries:
@@ -463,6 +459,23 @@ class HybridAdam(torch.optim.Optimizer):
             if h is None:
                 h = seen[k] = self._hyper_index(hypers, groups[gi], k[1] + 1)
             idx_of.append(h)
+        return idx_of
+
+    def hyper_table_of_next_step(self) -> np.ndarray:
+        """The ElxHyper records the next step over the bound chunks would upload (a host array; nothing
+        is launched or prepared): what a changed ``group['lr']`` turns into."""
+        assert self._binding is not None, 'only for an optimizer bound to chunk storage'
+        hypers: Dict = {}
+        self._bound_hyper_indices(self._walk_bound(), hypers)
+        return self._hyper_table(hypers)
+
+    def _prepare_bound(self, hypers: Dict) -> Optional[_Prepared]:
+        b = self._binding
+        b.require_gpu()
+        entries = self._walk_bound()
+        if not entries:
+            return None
+        idx_of = self._bound_hyper_indices(entries, hypers)
         lowp_dtype = b.chunks[0].paired_chunk.chunk_dtype
         grad_code = dtype_code(lowp_dtype)
         lowp_code = _abi.ELX_NONE if b.zero_grads else grad_code

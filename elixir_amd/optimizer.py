@@ -79,8 +79,13 @@ class _EventPair:
         return False
 
 
-class ElixirOptimizer:
+class ElixirOptimizer(torch.optim.Optimizer):
     """A wrapper for optimizers; one ElixirOptimizer corresponds to one chunked module.
+
+    Like the reference's wrapper (optimizer.py:27, a ``ColossalaiOptimizer``) it IS a
+    ``torch.optim.Optimizer`` -- learning-rate schedulers and anything else that checks the type accept
+    it -- without running ``Optimizer.__init__``: ``param_groups``, ``state`` and ``defaults`` are those
+    of the inner optimizer, so a scheduler that edits ``group['lr']`` edits what the next step uploads.
 
     Args:
         module: the chunked module (``param_chunk_group``, ``optim_chunk_group``,
@@ -170,19 +175,34 @@ class ElixirOptimizer:
             # allocate memory before training
             self.__zero_step()
 
-    # ------------------------------------------------------------------ torch.optim.Optimizer facade
+    # ------------------------------------------------------------------ torch.optim.Optimizer through the inner optimizer
 
     @property
     def param_groups(self):
         return self.optim.param_groups
 
+    @param_groups.setter
+    def param_groups(self, value):
+        self.optim.param_groups = value
+
     @property
     def defaults(self):
         return self.optim.defaults
 
+    @defaults.setter
+    def defaults(self, value):
+        self.optim.defaults = value
+
     @property
     def state(self):
         return self.optim.state
+
+    @state.setter
+    def state(self, value):
+        self.optim.state = value
+
+    def __repr__(self):
+        return f'{type(self).__name__}({self.optim!r})'
 
     def add_param_group(self, *args, **kwargs):
         return self.optim.add_param_group(*args, **kwargs)

@@ -69,7 +69,7 @@ typedef struct ElxChunk {
     uint64_t n_alloc;    /* shard_size: elements allocated, padding included */
     uint64_t n_valid;    /* elements of the head of the shard that hold tensors (valid_end clipped to n_alloc) */
     uint64_t tile_begin; /* launch-wide index of this chunk's first tile: sum over earlier chunks of
-                            ceil(n_alloc / elx_tile_elems()) */
+                            ceil(n_alloc / elx_tile_elems()); checked by elx_check_tables, not read by kernels */
     uint32_t seg_begin;  /* this chunk's segments are segs[seg_begin, seg_end) */
     uint32_t seg_end;
 } ElxChunk;
@@ -209,10 +209,10 @@ uint32_t elx_static_partials(void);
  * pure padding to elx_writeback_mt (whose workgroups move four times as much per tile and read
  * no tables).
  *   total_tiles            as returned by elx_check_tables for these tables
- *   grid_tiles_per_chunk   0: flat grid of total_tiles workgroups, each finds its chunk by a search
- *                          over tile_begin;  otherwise the launch is a 2-D grid
- *                          (grid_tiles_per_chunk, n_chunks) without any lookup, and must be at least
- *                          the max_tiles_per_chunk that elx_check_tables reported (n_chunks <= 65535)
+ *   grid_tiles_per_chunk   x extent of the 2-D launch grid (grid_tiles_per_chunk, n_chunks): record y,
+ *                          tile x, nothing is looked up.  At least the max_tiles_per_chunk that
+ *                          elx_check_tables reported; 0, or a grid that cannot hold total_tiles, is
+ *                          ELX_E_TILES.  n_chunks <= 65535: list a long shard as several records
  *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (13 for
  *                  16-bit gradients, 12 for fp32 gradients).
  *                  The update streams best with a shallow, orderly queue of memory requests.

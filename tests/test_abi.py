@@ -120,9 +120,12 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_grad_stats_mt(1, 1, _abi.ELX_F16, 2000, 1, 1, 0, None) == -7
     assert lib.elx_adam_step_mt(None, 1, None, 0, None, 0, 1, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -1
     assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 0, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -7
-    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, 9, _abi.ELX_NONE, 0, 0, None) == -2
-    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 2, None) == -7
+    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 4, -1.0, 9, _abi.ELX_NONE, 0, 0, None) == -2
+    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 4, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 2, None) == -7
     assert lib.elx_adam_step_mt(1, 2, None, 0, None, 0, 5, 2, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -6
+    # a grid of zero tiles per record is refused, by both update entry points
+    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -6
+    assert lib.elx_adam_step_gated_mt(1, 1, None, 0, None, 0, 4, 0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -6
     assert lib.elx_writeback_mt(None, 1, _abi.ELX_F16, 4, 0, None) == -1
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_NONE, 4, 0, None) == -2
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_F16, 0, 0, None) == -7

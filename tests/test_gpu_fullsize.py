@@ -12,6 +12,11 @@ ones that do not depend on size:
   * a skipped step (overflow) leaves master / exp_avg / exp_avg_sq bit-identical, restores the
     low-precision shards, and moves the loss scale as the state machine says;
   * the step is deterministic: replaying it from the same state gives the same bits.
+
+The C oracle does run at about 10**9 elements a second on the box's cores, which is enough to replay
+EVERY element once: ``test_full_size_every_element`` steps each set on the GPU, replays it chunk by
+chunk on the CPU from a pre-step clone and compares all of master, exp_avg, exp_avg_sq and the
+low-precision shard bit for bit.
 """
 import math
 
@@ -154,6 +159,76 @@ def test_full_size_step(oracle, name):
     assert np.array_equal(to_np(oc.shard[b:e]).view(np.uint32), wp.view(np.uint32))
     assert np.array_equal(to_np(m[b:e]).view(np.uint32), wm.view(np.uint32))
     assert ulp_distance(to_np(pc.shard[b:e]), wl) == 0
+
+
+def _host(t: torch.Tensor) -> np.ndarray:
+    """Device tensor -> numpy without a second host copy; 16-bit floats as uint16 bit patterns."""
+    t = t.detach()
+    if t.dtype in (torch.float16, torch.bfloat16):
+        return t.view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.cpu().numpy()
+
+
+@pytest.mark.parametrize('name', ['c2', 'c4', 'c5'])
+def test_full_size_every_element(oracle, name):
+    """Element for element at full size: the pre-step state of every chunk is cloned on the device, the
+    set is stepped once on the GPU, and every chunk is then replayed on the CPU by the oracle (one
+    ``adam`` call per tensor, with the combined scale the GPU's step reports, then the cast of the whole
+    shard).  Identical bits for master / exp_avg / exp_avg_sq and for the low-precision shard over all
+    ``shard_size`` elements of every chunk: padding refreshed, nothing outside the tensors touched."""
+    import time
+    built = workloads.build(name, seed=2468)
+    opt, module, dtype = built.optimizer, built.module, built.spec.dtype
+    code = CODE[dtype]
+    binding, inner = opt._binding, opt.optim
+    built.land_gradients()
+    need = 12 * built.n_alloc
+    free, _ = torch.cuda.mem_get_info()
+    assert free > need + (4 << 30), f'{name}: {free >> 30} GiB free, the pre-step clone needs {need >> 30} GiB'
+    pre = []
+    for pc in module.param_chunks:
+        oc = pc.paired_chunk
+        m, v = binding.moments(oc)
+        pre.append((oc.shard.clone(), m.clone(), v.clone()))    # the gradients are built.grads
+    opt.step()
+    info = opt.last_step_info
+    assert info['found_inf'] is False
+    comb = float(info['combined_scale'])
+    if built.spec.max_norm > 0:
+        assert comb > built.spec.loss_scale    # the clip is active: a divisor that is not a power of two
+    torch.cuda.synchronize()
+
+    t0 = time.perf_counter()
+    checked = 0
+    for ci, pc in enumerate(module.param_chunks):
+        oc = pc.paired_chunk
+        gm, gv = binding.moments(oc)
+        p0, m0, v0 = pre[ci]
+        pn, mn, vn, gn = _host(p0), _host(m0), _host(v0), _host(built.grads[ci])
+        pre[ci] = None
+        del p0, m0, v0
+        covered = 0
+        for group in inner.param_groups:
+            for fake in group['params']:
+                if opt.param_to_optim_chunk[fake] is not oc:
+                    continue
+                b, e = opt.param_to_range[fake]
+                assert inner.state[fake]['step'] == 1
+                oracle.adam(gn[b:e], code, pn[b:e], mn[b:e], vn[b:e], lr=group['lr'], beta1=group['betas'][0],
+                            beta2=group['betas'][1], eps=group['eps'], weight_decay=group['weight_decay'], step=1,
+                            adamw_mode=inner.adamw_mode, bias_correction=group['bias_correction'], div_scale=comb)
+                covered += e - b
+        assert covered == pc.utilized_size
+        tag = f'{name} chunk {ci}'
+        assert np.array_equal(_host(oc.shard).view(np.uint32), pn.view(np.uint32)), tag + ' master'
+        assert np.array_equal(_host(gm).view(np.uint32), mn.view(np.uint32)), tag + ' exp_avg'
+        assert np.array_equal(_host(gv).view(np.uint32), vn.view(np.uint32)), tag + ' exp_avg_sq'
+        assert np.array_equal(_host(pc.shard), oracle.writeback(pn, code)), tag + ' low-precision shard'
+        if pc.utilized_size < pc.shard_size:    # the padding: zero master, never updated, refreshed to zero
+            assert not pn[pc.utilized_size:].any() and not mn[pc.utilized_size:].any()
+        checked += pc.shard_size
+        print(f'{tag}: {pc.shard_size} elements identical ({time.perf_counter() - t0:.1f} s)', flush=True)
+    assert checked == built.n_alloc
 
 
 def test_full_size_step_is_deterministic():

@@ -750,6 +750,107 @@ def test_single_buffer_stats_and_writeback(oracle, dtype, n, offset):
 
 
 # ------------------------------------------------------------------------------------------------
+# the update launch on buffers that are not 16-byte aligned
+# ------------------------------------------------------------------------------------------------
+
+
+def _offset_view(data: torch.Tensor, offset: int) -> torch.Tensor:
+    """A copy of ``data`` that starts ``offset`` elements into a fresh allocation."""
+    big = torch.zeros(data.numel() + offset + 8, dtype=data.dtype, device=DEV)
+    view = big[offset:offset + data.numel()]
+    view.copy_(data)
+    return view
+
+
+@pytest.mark.parametrize('gdtype', [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('how', ['host', 'gated', 'gated_skip'])
+def test_update_on_misaligned_buffers(oracle, gdtype, how):
+    """One misaligned base pointer makes the host pass ELX_FLAG_SCALAR_ONLY and every tile of the
+    update launch takes the element-by-element path (optimizer.py:115-124 hands the inner optimizer
+    arbitrary slices).  Two records whose gradient / master / exp_avg / exp_avg_sq views start at odd
+    element offsets, with a segment boundary inside a tile, a gap no segment covers, a padding tail
+    that starts inside a tile, two hyper records (decoupled decay and L2) and a divisor that is not a
+    power of two: identical bits to the oracle and to the same launch on aligned copies; decided by
+    the host, decided on the device, and skipped on the device."""
+    from elixir_amd.chunk import DeviceTable
+    from elixir_amd.hybrid_adam import make_hyper_record
+    code = CODE[gdtype]
+    tile = _abi.tile_elems()
+    div = 3.7
+    layout = [    # (n_alloc, n_valid, [(begin, end, hyper)])
+        (20 * tile + 77, 4500, [(0, 1000, 0), (1000, 2051, 1), (2100, 4500, 0)]),
+        (4 * tile, 4 * tile, [(0, 4 * tile, 1)]),
+    ]
+    hyp = [dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.1, step=3, adamw_mode=True),
+           dict(lr=2e-3, beta1=0.5, beta2=0.95, eps=1e-6, weight_decay=0.01, step=7, adamw_mode=False)]
+    hyper_host = np.concatenate([make_hyper_record(h['lr'], h['beta1'], h['beta2'], h['eps'], h['weight_decay'],
+                                                   h['step'], True, h['adamw_mode']) for h in hyp])
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    data = []
+    for n_alloc, n_valid, _ in layout:
+        master = torch.randn(n_alloc, generator=gen, device=DEV) * 0.02
+        m = torch.randn(n_alloc, generator=gen, device=DEV) * 1e-4
+        v = torch.rand(n_alloc, generator=gen, device=DEV) * 1e-6
+        # the padding holds garbage gradients (an inf among them): the update must not read them
+        g = (torch.randn(n_alloc, generator=gen, device=DEV) * 1e-3 * div).to(gdtype)
+        if n_valid < n_alloc:
+            g[n_valid] = float('inf')
+        data.append((g, master, m, v))
+
+    def launch(offsets):
+        """Runs the update on copies of ``data`` placed at the given element offsets; returns the
+        buffers afterwards and whether the tables were reported aligned."""
+        bufs, rows, segs, tiles = [], np.zeros(len(layout), dtype=_abi.CHUNK_DTYPE), [], 0
+        for i, ((n_alloc, n_valid, seg_list), (g, master, m, v)) in enumerate(zip(layout, data)):
+            views = [_offset_view(t, o) for t, o in zip((g, master, m, v), offsets)]
+            bufs.append(views)
+            rows[i]['grad'] = rows[i]['lowp_out'] = views[0].data_ptr()    # in place, as in a chunk shard
+            rows[i]['master'], rows[i]['m'], rows[i]['v'] = (t.data_ptr() for t in views[1:])
+            rows[i]['n_alloc'], rows[i]['n_valid'], rows[i]['tile_begin'] = n_alloc, n_valid, tiles
+            tiles += -(-n_alloc // tile)
+            rows[i]['seg_begin'] = len(segs)
+            segs += [(b, e, h, 0) for b, e, h in seg_list]
+            rows[i]['seg_end'] = len(segs)
+        segs = np.array(segs, dtype=_abi.SEG_DTYPE)
+        info = _abi.check_tables(rows, segs, len(hyper_host), code, code)
+        d_rows, d_segs = DeviceTable(rows, torch.device(DEV, 0)), DeviceTable(segs, torch.device(DEV, 0))
+        d_hyp = DeviceTable(hyper_host, torch.device(DEV, 0))
+        stream = torch.cuda.current_stream().cuda_stream
+        if how == 'host':
+            _abi.adam_step_mt(d_rows.ptr, len(rows), d_segs.ptr, len(segs), d_hyp.ptr, len(hyper_host), info, div, code,
+                              code, 0, stream)
+        else:
+            stats = np.zeros(1, dtype=_abi.STATS_DTYPE)
+            stats['overflow'] = 1 if how == 'gated_skip' else 0
+            d_stats = DeviceTable(stats, torch.device(DEV, 0))
+            decision = torch.zeros(_abi.DECISION_DTYPE.itemsize, dtype=torch.uint8, device=DEV)
+            _abi.decide(d_stats.ptr, 1, div, 0.0, False, d_hyp.ptr, len(hyper_host), decision.data_ptr(), stream)
+            _abi.adam_step_gated_mt(d_rows.ptr, len(rows), d_segs.ptr, len(segs), d_hyp.ptr, len(hyper_host), info,
+                                    code, code, 0, stream)
+        torch.cuda.synchronize()
+        return bufs, info.aligned
+
+    odd, odd_aligned = launch((1, 1, 2, 3))
+    even, even_aligned = launch((0, 0, 0, 0))
+    assert not odd_aligned and even_aligned
+
+    for i, ((n_alloc, n_valid, seg_list), (g, master, m, v)) in enumerate(zip(layout, data)):
+        gn, pn, mn, vn = to_np(g), to_np(master), to_np(m), to_np(v)
+        if how != 'gated_skip':
+            for b, e, h in seg_list:
+                hh = hyp[h]
+                oracle.adam(gn[b:e], code, pn[b:e], mn[b:e], vn[b:e], lr=hh['lr'], beta1=hh['beta1'], beta2=hh['beta2'],
+                            eps=hh['eps'], weight_decay=hh['weight_decay'], step=hh['step'], adamw_mode=hh['adamw_mode'],
+                            div_scale=div)
+        else:
+            assert np.array_equal(pn, to_np(master))
+        want = (oracle.writeback(pn, code), pn, mn, vn)    # the whole record is refreshed, padding included
+        for name, w, a, b in zip(('lowp', 'master', 'm', 'v'), want, odd[i], even[i]):
+            assert np.array_equal(to_np(a).view(np.uint8), w.view(np.uint8)), f'{how} record {i} {name}: misaligned vs oracle'
+            assert np.array_equal(to_np(b).view(np.uint8), w.view(np.uint8)), f'{how} record {i} {name}: aligned vs oracle'
+
+
+# ------------------------------------------------------------------------------------------------
 # the decisions of the step taken on the device
 # ------------------------------------------------------------------------------------------------
 
@@ -935,3 +1036,32 @@ def test_per_tensor_step_counts_and_changing_learning_rates(oracle):
         assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'step {step}') == 0
     want = sorted(s + 3 for s in steps.values())
     assert sorted(st['step'] for st in opt.state.values()) == want
+
+
+def test_lr_scheduler_drives_the_wrapped_optimizer(oracle):
+    """A torch learning-rate scheduler built on the wrapper (example/fine-tune/elixir_mini.py:90 does
+    exactly that): it accepts the wrapper as an Optimizer, counts its steps, and the learning rate it
+    sets between two steps is the one the second step runs with -- identical bits to the oracle."""
+    dtype = torch.float16
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=31, loss_scale=128.0, weight_decay=0.05,
+                                          lr=2e-3, initial_scale=128.0, hysteresis=1)
+    scaler = O.DynamicGradScalerOracle(initial_scale=128.0, min_scale=1, max_scale=2**24, hysteresis=1)
+    sched = torch.optim.lr_scheduler.LambdaLR(opt, lr_lambda=lambda epoch: 1.0 / (1 + epoch))
+    gen = torch.Generator(device=DEV).manual_seed(32)
+    for step in range(3):
+        lr = 2e-3 / (1 + step)
+        assert all(g['lr'] == lr for g in opt.param_groups)
+        for oc in ochunks:
+            for seg in oc.segments:
+                seg.lr = lr
+        if step:
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (1e-3 * 128.0)
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+                pc.invalidate_stats()
+            refresh_oracle_grads(module, ochunks)
+        _run_and_compare(module, opt, ochunks, dtype, scaler, tag=f'step {step}')
+        assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'step {step}') == 0
+        sched.step()    # warns when the optimizer's step() was not seen before it
+    assert opt._opt_called and sched.last_epoch == 3

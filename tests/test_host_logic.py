@@ -429,6 +429,37 @@ def test_optimizer_state_dict_round_trip_keeps_flat_storage():
         other.load_state_dict(bad)
 
 
+def test_wrapper_is_a_torch_optimizer_and_schedulers_reach_the_hyper_table():
+    """The reference's wrapper is an Optimizer (optimizer.py:27) and its own callers hand it to a
+    learning-rate scheduler (example/fine-tune/elixir_mini.py:90).  torch's schedulers accept this one,
+    and the learning rate they set is the one the next step's hyper records are made from."""
+    module, opt = _cpu_optimizer(3)
+    assert isinstance(opt, torch.optim.Optimizer)
+    assert opt.param_groups is opt.optim.param_groups and opt.state is opt.optim.state
+    assert opt.defaults is opt.optim.defaults and 'HybridAdam' in repr(opt)
+    sched = torch.optim.lr_scheduler.LambdaLR(opt, lr_lambda=lambda epoch: 0.5**epoch)
+    assert [g['initial_lr'] for g in opt.param_groups] == [1e-3, 1e-3]
+
+    def neg_steps():
+        return sorted(set(float(x) for x in opt.optim.hyper_table_of_next_step()['neg_step']))
+
+    bc1 = 1.0 - 0.9**1    # the first step of every tensor
+    assert neg_steps() == [float(np.float32(-(1e-3 / bc1)))]
+    opt._opt_called = True    # what the scheduler's wrapper around step() records; no GPU, no step here
+    sched.step()
+    assert [g['lr'] for g in opt.param_groups] == [5e-4, 5e-4]
+    assert neg_steps() == [float(np.float32(-(5e-4 / bc1)))]
+    # a warm-up schedule on one group only: two different records
+    opt.param_groups[1]['lr'] = 1e-4
+    assert neg_steps() == sorted([float(np.float32(-(5e-4 / bc1))), float(np.float32(-(1e-4 / bc1)))])
+    # decoupled decay follows the learning rate as well (torch/optim/adam.py:414-419)
+    table = opt.optim.hyper_table_of_next_step()
+    assert sorted(float(x) for x in table['decay_mul']) == sorted([float(np.float32(1 - 5e-4 * 0.1)), 1.0])
+    # other schedulers construct too
+    torch.optim.lr_scheduler.StepLR(opt, step_size=2)
+    torch.optim.lr_scheduler.CosineAnnealingLR(opt, T_max=10)
+
+
 def test_chunk_cpu_copy_and_load_tensors():
     a, b = torch.randn(3, 5), torch.randn(7)
     chunk = ea.Chunk(None, 32, torch.float, None, shard_device='cpu', temp_device='cpu')
