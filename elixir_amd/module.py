@@ -66,6 +66,41 @@ def greedy_search(named_sizes: Sequence[Tuple[str, int]], chunk_size: int, dtype
     return SearchResult(ChunkGroup(None), plans)
 
 
+def simple_groups(sizes: Sequence[int], split_number: int) -> Tuple[List[List[int]], int]:
+    """The split rule of search/simple.py:30-74: the tensors, in order, are cut into
+    ``min(len, split_number)`` runs by COUNT (the first ``len % split_number`` runs hold one tensor more);
+    every public chunk gets the size of the fullest run.  Returns (groups of indices, that size)."""
+    n = len(sizes)
+    split_number = min(n, split_number)
+    if split_number <= 0:
+        return [], 0
+    average, left = divmod(n, split_number)
+    groups, at = [], 0
+    for i in range(split_number):
+        count = average + (1 if i < left else 0)
+        groups.append(list(range(at, at + count)))
+        at += count
+    return groups, max(sum(sizes[i] for i in g) for g in groups)
+
+
+def simple_search(named_sizes: Sequence[Tuple[str, int]], group_size: int, split_number: int, dtype: torch.dtype,
+                  private_names: Sequence[str] = (), shard_device: Optional[torch.device] = None) -> SearchResult:
+    """The chunk plans of the reference's ``simple_search`` (search/simple.py:77-110, search/base.py:87-108)
+    for a tensor list given by name and size: every tensor named in ``private_names`` (the parameters a
+    model uses more than once, search/utils.py:24-33) gets a private chunk of its own size rounded up
+    to ``group_size``, marked ``rcache_fused``; the others are split by ``simple_groups`` into public
+    chunks of one size (rounded up to ``group_size``).  Private plans come first."""
+    private = set(private_names)
+    kwargs = {} if shard_device is None else dict(shard_device=shard_device)
+    plans = [ChunkPlan([n], to_divide(s, group_size), dtype, dict(kwargs, rcache_fused=True))
+             for n, s in named_sizes if n in private]
+    public = [(n, s) for n, s in named_sizes if n not in private]
+    groups, block = simple_groups([s for _, s in public], split_number)
+    block = to_divide(block, group_size)
+    plans += [ChunkPlan([public[i][0] for i in g], block, dtype, dict(kwargs)) for g in groups]
+    return SearchResult(ChunkGroup(None), plans)
+
+
 def get_param_optim_data(param_data: torch.Tensor, param_dtype: torch.dtype, device: torch.device):
     """module.py:21-25: the master copy is fp32, the parameter takes the training dtype."""
     param_data = param_data.to(device)

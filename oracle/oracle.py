@@ -287,6 +287,34 @@ def greedy_pack(sizes: Sequence[int], chunk_size: int) -> List[List[int]]:
     return groups
 
 
+def simple_pack(sizes: Sequence[int], private: Sequence[bool], group_size: int,
+                split_number: int) -> Tuple[List[int], List[List[int]], int]:
+    """search/simple.py:30-74 with search/base.py:87-108 -- the plan of ``simple_search``: every
+    private tensor (one a model uses more than once, search/utils.py:24-33) gets a chunk of its own,
+    its size rounded up to a multiple of ``group_size``; the public tensors, in order, are cut into
+    ``min(count, split_number)`` runs by count (the remainder goes one each to the first runs) and every
+    public chunk has the size of the fullest run, rounded up the same way.
+
+    Returns (private chunk sizes, public groups as index lists into ``sizes``, public chunk size)."""
+    def to_divide(a, b):    # search/utils.py:5-6
+        return a + (-a % b)
+
+    private_sizes = [to_divide(s, group_size) for s, p in zip(sizes, private) if p]
+    public = [i for i, p in enumerate(private) if not p]
+    split_number = min(len(public), split_number)
+    groups: List[List[int]] = []
+    block = 0
+    if split_number > 0:
+        average, left = divmod(len(public), split_number)
+        at = 0
+        for i in range(split_number):
+            count = average + (1 if i < left else 0)
+            groups.append(public[at:at + count])
+            at += count
+        block = max(sum(sizes[i] for i in g) for g in groups)
+    return private_sizes, groups, to_divide(block, group_size)
+
+
 def chunk_offsets(sizes: Sequence[int]) -> List[Tuple[int, int]]:
     """chunk.py:223-247 -- tensors are appended back to back with no alignment padding."""
     out, used = [], 0

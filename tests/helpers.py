@@ -56,12 +56,14 @@ def assert_close_f32(got: np.ndarray, want: np.ndarray, name: str, rtol: float =
 
 def build_workload(named_shapes, chunk_size, dtype, *, seed=0, grad_std=1e-3, loss_scale=1.0, lr=1e-3,
                    betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, adamw_mode=True, decay_exempt=True,
-                   warm_state=True, device='cuda', host_resident=False, **opt_kwargs):
+                   warm_state=True, device='cuda', host_resident=False, search_result=None, **opt_kwargs):
     """A synthetic chunk set on the GPU with seeded contents, its ElixirOptimizer, and the oracle's
     copy of the same data.  Gradients (already multiplied by ``loss_scale``) sit in the
     low-precision shards, as they do after backward."""
     named_shapes = list(named_shapes)
-    if host_resident == 'mixed':    # every other chunk in pinned host memory, the rest on the GPU
+    if search_result is not None:    # chunk plans made by the caller
+        sr = search_result
+    elif host_resident == 'mixed':    # every other chunk in pinned host memory, the rest on the GPU
         sr = ea.greedy_search([(n, S.numel(s)) for n, s in named_shapes], chunk_size, dtype)
         for plan in sr.param_chunk_plans[::2]:
             plan.kwargs.update(shard_device=torch.device('cpu'), cpu_pin_memory=True)

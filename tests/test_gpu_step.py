@@ -1065,3 +1065,36 @@ def test_lr_scheduler_drives_the_wrapped_optimizer(oracle):
         assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'step {step}') == 0
         sched.step()    # warns when the optimizer's step() was not seen before it
     assert opt._opt_called and sched.last_epoch == 3
+
+
+def test_step_over_simple_search_plans(oracle):
+    """The chunk plans of the reference's own planner fixture (test/search/test_simple.py:29-42: a
+    private, fused chunk of 320 for the tied embedding and five public chunks of 1088): the wrapper
+    steps `fused_chunks | float_chunks` (optimizer.py:58-66), chunks of two sizes in one launch.
+    Three steps, the second with an overflow in the private chunk: identical bits to the oracle."""
+    dtype = torch.float16
+    named = [('embed.weight', (20, 16)), ('norm1.weight', (16, )), ('norm1.bias', (16, )), ('mlp.proj1.weight', (64, 16)),
+             ('mlp.proj1.bias', (64, )), ('mlp.proj2.weight', (16, 64)), ('mlp.proj2.bias', (16, )),
+             ('norm2.weight', (16, )), ('norm2.bias', (16, ))]
+    sr = ea.simple_search([(n, S.numel(s)) for n, s in named], 1, 5, dtype, private_names=['embed.weight'])
+    module, opt, ochunks = build_workload(named, 0, dtype, seed=41, loss_scale=256.0, weight_decay=0.1, max_norm=1.0,
+                                          grad_std=0.05, search_result=sr, initial_scale=256.0, hysteresis=1)
+    assert [pc.chunk_size for pc in module.param_chunks] == [320] + [1088] * 5
+    assert len(opt.param_chunk_group.fused_chunks) == 1 and len(opt.param_chunk_group.float_chunks) == 5
+    scaler = O.DynamicGradScalerOracle(initial_scale=256.0, min_scale=1, max_scale=2**24, hysteresis=1)
+    gen = torch.Generator(device=DEV).manual_seed(42)
+    for step in range(3):
+        if step:
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (0.05 * opt.loss_scale)
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+                pc.invalidate_stats()
+            if step == 1:
+                fused = next(iter(opt.param_chunk_group.fused_chunks))
+                fused.shard[7] = float('-inf')
+            refresh_oracle_grads(module, ochunks)
+        info = _run_and_compare(module, opt, ochunks, dtype, scaler, max_norm=1.0, tag=f'step {step}')
+        assert info['found_inf'] == (step == 1)
+        compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-8, atol_v=1e-10, tag=f'step {step}')
+    assert opt.loss_scale == 128.0

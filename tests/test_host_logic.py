@@ -42,6 +42,19 @@ def test_dynamic_scaler_follows_the_oracle(hysteresis, factors):
         assert a.scale.dtype == torch.float32 and a.scale.item() == float(b.scale)
 
 
+def test_dynamic_scaler_corner_cases_as_literals():
+    """The same literal trajectories the oracle is pinned with (hysteresis 0 / 1 / 3, clamps hit
+    exactly and passed, counter resets, factors that are not powers of two rounded to fp32)."""
+    from test_oracle import SCALER_LITERALS
+    for kwargs, seq, want in SCALER_LITERALS:
+        sc = ea.DynamicGradScaler(**kwargs)
+        got = []
+        for f in seq:
+            sc.update(f)
+            got.append(sc.scale_value)
+        assert got == want, kwargs
+
+
 def test_default_scaler_settings_skip_without_backoff_on_first_overflow():
     """With the wrapper's default hysteresis of 2 the first overflow only arms the back-off."""
     sc = ea.DynamicGradScaler(initial_scale=32768, min_scale=1, growth_factor=2, backoff_factor=0.5,

@@ -355,8 +355,13 @@ def test_combined_scale_rules():
 
 
 def test_global_norm_passes_through_fp32(oracle):
-    norms = [1.0 + 2.0**-30, 3.0, 5.0]
-    assert oracle.global_norm(norms) == math.sqrt(float(np.float32(sum(norms))))
+    # the float64 sum 9 + 2**-30 is not an fp32 number: the one-element fp32 buffer of
+    # optimizer.py:158-162 rounds it to 9, so the norm is exactly 3 (without the detour it would be
+    # 3.0000000001552...)
+    assert oracle.global_norm([1.0 + 2.0**-30, 3.0, 5.0]) == 3.0
+    assert math.sqrt(1.0 + 2.0**-30 + 3.0 + 5.0) != 3.0
+    # and the square root is taken in float64, not in fp32: sqrt(2) keeps all its digits
+    assert oracle.global_norm([0.5, 1.5]) == 1.4142135623730951
 
 
 def test_scaler_hysteresis_and_clamps():
@@ -371,6 +376,86 @@ def test_scaler_hysteresis_and_clamps():
     const = O.ConstantGradScalerOracle(1.0)
     const.update(True)
     assert float(const.scale) == 1.0
+
+
+# The state machine's corner cases as literals.  Every product is rounded to fp32 (the scale is a
+# one-element fp32 tensor): 3 * fp32(1.1) = 3.30000007152557373046875 is an exact tie between two fp32
+# neighbours and goes to the even one, 3.3000001907348633 -- float64 arithmetic would give
+# 3.3000000000000003, fp32(3.3) is 3.299999952316284.
+SCALER_LITERALS = [
+    # (constructor arguments, overflow sequence, scale after every update)
+    (dict(initial_scale=64.0, hysteresis=0), [True, True, False], [32.0, 16.0, 16.0]),
+    (dict(initial_scale=64.0, hysteresis=1), [True, True, False], [32.0, 16.0, 16.0]),
+    (dict(initial_scale=64.0, hysteresis=3), [True, True, True, True], [64.0, 64.0, 32.0, 16.0]),
+    # back-off landing exactly on min_scale, then held there
+    (dict(initial_scale=32.0, hysteresis=1, min_scale=16.0), [True, True, True], [16.0, 16.0, 16.0]),
+    # back-off that would pass below min_scale is clamped to it
+    (dict(initial_scale=24.0, hysteresis=1, min_scale=16.0), [True, True], [16.0, 16.0]),
+    # growth landing exactly on max_scale, then held there
+    (dict(initial_scale=64.0, growth_interval=1, max_scale=128.0), [False, False, False], [128.0, 128.0, 128.0]),
+    # growth that would pass above max_scale is clamped to it
+    (dict(initial_scale=96.0, growth_interval=1, max_scale=128.0), [False, False], [128.0, 128.0]),
+    # an overflow resets the growth counter; a growth resets the hysteresis counter
+    (dict(initial_scale=64.0, growth_interval=2, hysteresis=2), [False, True, False, False, True, True],
+     [64.0, 64.0, 64.0, 128.0, 128.0, 64.0]),
+    # factors that are not powers of two, rounded to fp32 at every step
+    (dict(initial_scale=3.0, growth_factor=1.1, growth_interval=1), [False] * 4,
+     [3.3000001907348633, 3.630000352859497, 3.9930005073547363, 4.392300605773926]),
+    (dict(initial_scale=1000.0, backoff_factor=0.3, hysteresis=1), [True] * 4,
+     [300.0, 90.0, 27.000001907348633, 8.100001335144043]),
+]
+
+
+@pytest.mark.parametrize('case', range(len(SCALER_LITERALS)))
+def test_scaler_corner_cases_as_literals(case):
+    kwargs, seq, want = SCALER_LITERALS[case]
+    sc = O.DynamicGradScalerOracle(**kwargs)
+    got = []
+    for f in seq:
+        sc.update(f)
+        got.append(float(sc.scale))
+    assert got == want
+
+
+def test_the_fp32_tie_of_the_scaler_literal_by_exact_arithmetic():
+    from fractions import Fraction
+    exact = Fraction(float(np.float32(1.1))) * 3
+    lo, hi = Fraction(float.fromhex('0x1.a66666p+1')), Fraction(float.fromhex('0x1.a66668p+1'))
+    assert exact - lo == hi - exact                      # a tie ...
+    assert float(hi) == 3.3000001907348633               # ... that goes to the neighbour with the even mantissa
+    assert int(np.float32(float(hi)).view(np.uint32)) % 2 == 0 and int(np.float32(float(lo)).view(np.uint32)) % 2 == 1
+
+
+def test_simple_search_known_answer():
+    """The reference's own fixture for its chunk plans, test/search/test_simple.py:29-42: the `small`
+    model of test/utils/small.py (embedding 20 x 16 tied to the output projection, LayerNorm 16, an MLP
+    16 -> 64 -> 16, LayerNorm 16) under simple_search(group_size=1, split_number=5) gets one private
+    chunk of 320 for the tied embedding and five public chunks of 1088 with these name lists.  (The
+    fixture pins the split-by-count rule and the private/public split; the greedy rule of
+    mini_waste.py:78-96 has no fixture in the reference and is pinned by test_greedy_packing_rule.)"""
+    named = [('embed.weight', 20 * 16), ('norm1.weight', 16), ('norm1.bias', 16), ('mlp.proj1.weight', 64 * 16),
+             ('mlp.proj1.bias', 64), ('mlp.proj2.weight', 16 * 64), ('mlp.proj2.bias', 16), ('norm2.weight', 16),
+             ('norm2.bias', 16)]    # named_parameters() order; proj.weight is embed.weight
+    names = [n for n, _ in named]
+    sizes = [s for _, s in named]
+    private_sizes, groups, block = O.simple_pack(sizes, [n == 'embed.weight' for n in names], 1, 5)
+    assert private_sizes == [320] and block == 1088
+    assert [[names[i] for i in g] for g in groups] == [['norm1.weight', 'norm1.bias'],
+                                                       ['mlp.proj1.weight', 'mlp.proj1.bias'],
+                                                       ['mlp.proj2.weight', 'mlp.proj2.bias'], ['norm2.weight'],
+                                                       ['norm2.bias']]
+    # rounding up to the group size (search/simple.py:26-30)
+    assert O.simple_pack(sizes, [n == 'embed.weight' for n in names], 256, 5)[::2] == ([512], 1280)
+    # fewer tensors than groups: one tensor per chunk
+    assert O.simple_pack([5, 7], [False, False], 1, 10) == ([], [[0], [1]], 7)
+
+    # the product's planner gives the same plans
+    import elixir_amd as ea
+    sr = ea.simple_search(named, 1, 5, torch.float16, private_names=['embed.weight'])
+    plans = sr.param_chunk_plans
+    assert plans[0].name_list == ['embed.weight'] and plans[0].chunk_size == 320 and plans[0].kwargs['rcache_fused']
+    assert [p.name_list for p in plans[1:]] == [[names[i] for i in g] for g in groups]
+    assert all(p.chunk_size == 1088 and not p.kwargs.get('rcache_fused') for p in plans[1:])
 
 
 def test_greedy_packing_rule():
