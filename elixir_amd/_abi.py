@@ -10,7 +10,7 @@ from typing import Optional
 
 import numpy as np
 
-ELX_ABI_VERSION = 1
+ELX_ABI_VERSION = 2
 ELX_F32, ELX_F16, ELX_BF16, ELX_NONE = 0, 1, 2, -1
 ELX_FLAG_SCALAR_ONLY = 1
 ELX_E_NULL, ELX_E_DTYPE, ELX_E_ALIGN, ELX_E_RANGE, ELX_E_ORDER, ELX_E_TILES, ELX_E_SIZE = -1, -2, -3, -4, -5, -6, -7
@@ -28,6 +28,12 @@ STATS_DTYPE = np.dtype([('sumsq', '<f8'), ('overflow', '<u4'), ('reserved', '<u4
 DECISION_DTYPE = np.dtype([('div_scale', '<f4'), ('inv_scale', '<f4'), ('mode', '<u4'), ('skip', '<u4'),
                            ('total_norm', '<f8'), ('combined_scale', '<f8')])
 
+STEP_CTL_DTYPE = np.dtype([('loss_scale', '<f8'), ('max_norm', '<f8'), ('clipping', '<u4'), ('n_hypers', '<u4'),
+                           ('seq', '<u8')])
+STEP_REPORT_DTYPE = np.dtype([('div_scale', '<f4'), ('inv_scale', '<f4'), ('mode', '<u4'), ('skip', '<u4'),
+                              ('total_norm', '<f8'), ('combined_scale', '<f8'), ('seq', '<u8'), ('n_chunks', '<u4'),
+                              ('status', '<i4')])
+
 LIB_NAME = 'libelx_hip.so'
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
@@ -35,7 +41,8 @@ EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 
            'elx_sizeof_stats', 'elx_sizeof_decision', 'elx_check_tables', 'elx_grad_stats_mt', 'elx_adam_step_mt',
            'elx_decide', 'elx_adam_step_gated_mt', 'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_writeback',
            'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems',
-           'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials')
+           'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
+           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers')
 
 
 class ElxError(RuntimeError):
@@ -65,7 +72,8 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
-                 'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials'):
+                 'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
+           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -73,6 +81,10 @@ def load() -> ctypes.CDLL:
                                    ctypes.POINTER(cint)]
     L.elx_grad_stats_mt.restype = cint
     L.elx_grad_stats_mt.argtypes = [vp, u32, cint, u32, vp, vp, cint, vp]
+    L.elx_grad_partials_mt.restype = cint
+    L.elx_grad_partials_mt.argtypes = [vp, u32, cint, u32, vp, cint, vp]
+    L.elx_finish_decide.restype = cint
+    L.elx_finish_decide.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp]
     L.elx_grad_stats_mt_static.restype = cint
     L.elx_grad_stats_mt_static.argtypes = [vp, u32, cint, u32, vp, cint, vp]
     L.elx_adam_step_mt.restype = cint
@@ -97,7 +109,7 @@ def load() -> ctypes.CDLL:
     if L.elx_version() != ELX_ABI_VERSION:
         raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
     for name, dt in (('chunk', CHUNK_DTYPE), ('seg', SEG_DTYPE), ('hyper', HYPER_DTYPE), ('stats', STATS_DTYPE),
-                     ('decision', DECISION_DTYPE)):
+                     ('decision', DECISION_DTYPE), ('step_ctl', STEP_CTL_DTYPE), ('step_report', STEP_REPORT_DTYPE)):
         size = getattr(L, f'elx_sizeof_{name}')()
         if size != dt.itemsize:
             raise RuntimeError(f'{LIB_PATH}: sizeof {name} record is {size}, binding expects {dt.itemsize}')
@@ -163,6 +175,26 @@ def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chun
     check('elx_grad_stats_mt',
           load().elx_grad_stats_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, d_stats,
                                    int(scalar_only), stream))
+
+
+def grad_partials_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_partials: int,
+                     scalar_only: bool, stream: int) -> None:
+    """The first launch of ``grad_stats_mt`` alone: the partials are left for ``finish_decide``."""
+    check('elx_grad_partials_mt',
+          load().elx_grad_partials_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, int(scalar_only),
+                                      stream))
+
+
+def finish_decide(d_partials: int, n_chunks: int, blocks_per_chunk: int, d_stats: int, ctl: int, d_hypers: int,
+                  max_hypers: int, d_decision: int, report: int, d_counter: int, stream: int) -> None:
+    """Fold of the partials + the decisions of the step, everything that changes read from ``ctl``."""
+    check('elx_finish_decide',
+          load().elx_finish_decide(d_partials, n_chunks, blocks_per_chunk, d_stats, ctl, d_hypers, max_hypers, d_decision,
+                                   report or None, d_counter, stream))
+
+
+def max_ctl_hypers() -> int:
+    return int(load().elx_max_ctl_hypers())
 
 
 def static_partials() -> int:

@@ -841,15 +841,16 @@ __device__ __forceinline__ bool exact_reciprocal_dev(float s) {
 // norm exceeds max_norm).  Per chunk the squared norm passes through an fp32 norm
 // (chunk.py:218-221), the sum over chunks through an fp32 buffer (optimizer.py:158-162).  The
 // result goes into *out and into the gate words of every hyper record.
-__global__ void decide_kernel(const ElxStats *__restrict__ stats, uint32_t n, double loss_scale, double max_norm,
-                              int clipping, ElxHyper *__restrict__ hypers, uint32_t n_hypers,
-                              ElxDecision *__restrict__ out) {
-    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+// `stats` may have been written by other workgroups of the same launch: read through agent-scope loads.
+__device__ __forceinline__ ElxDecision decide_from_stats(const ElxStats *stats, uint32_t n, double loss_scale,
+                                                         double max_norm, int clipping) {
     uint32_t found = 0;
     double norm_sqr = 0.0;
     for (uint32_t i = 0; i < n; ++i) {
-        found |= stats[i].overflow;
-        const float nrm = (float)sqrt(stats[i].sumsq);
+        found |= __hip_atomic_load(&stats[i].overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint64_t bits = __hip_atomic_load(reinterpret_cast<const uint64_t *>(&stats[i].sumsq), __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+        const float nrm = (float)sqrt(__builtin_bit_cast(double, bits));
         norm_sqr += (double)nrm * (double)nrm;
     }
     ElxDecision d;
@@ -874,12 +875,127 @@ __global__ void decide_kernel(const ElxStats *__restrict__ stats, uint32_t n, do
             d.mode = kDivTrue;
         }
     }
+    return d;
+}
+
+__global__ void decide_kernel(const ElxStats *__restrict__ stats, uint32_t n, double loss_scale, double max_norm,
+                              int clipping, ElxHyper *__restrict__ hypers, uint32_t n_hypers,
+                              ElxDecision *__restrict__ out) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    const ElxDecision d = decide_from_stats(stats, n, loss_scale, max_norm, clipping);
     *out = d;
     for (uint32_t i = 0; i < n_hypers; ++i) {
         hypers[i].gate_div_scale = d.div_scale;
         hypers[i].gate_inv_scale = d.inv_scale;
         hypers[i].gate = d.mode | (d.skip << 8);
     }
+}
+
+// The fold of the stats partials and the decisions of the step in ONE launch whose arguments never
+// change from step to step (so that it can sit in a recorded graph): what does change -- loss scale,
+// clipping threshold, the hyper records of the step -- is read from a control block in memory, which
+// may be pinned host memory that the host rewrites before every step.
+//
+// Grid: one workgroup per chunk.  Workgroup b folds the partials of chunk b exactly as
+// stats_finish_kernel does (same order, same bits) and publishes the record; the workgroup that
+// finds every other one done (a counter, left at zero again for the next launch) decides: it copies
+// the hyper records of the control block into the device table of the update launch with the gate
+// words filled in, writes the decision, and reports to the host -- decision and per-chunk records
+// first, the sequence number of the control block last, all with system-scope stores, so that a host
+// polling the sequence number in pinned memory sees a complete report while the update launch that
+// follows is still running.
+constexpr uint32_t kMaxCtlHypers = 64;
+constexpr uint32_t kCtlWords = (uint32_t)(sizeof(ElxStepCtl) + kMaxCtlHypers * sizeof(ElxHyper)) / 4u;
+
+template <typename T>
+__device__ __forceinline__ void store_system(T *p, T v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxStats *__restrict__ partials, uint32_t bpc,
+                                                                      ElxStats *stats, uint32_t n_chunks,
+                                                                      const ElxStepCtl *ctl, ElxHyper *hypers,
+                                                                      uint32_t max_hypers, ElxDecision *out,
+                                                                      ElxStepReport *report, uint32_t *counter) {
+    __shared__ uint32_t s_last;
+    __shared__ __align__(16) uint32_t s_ctl[kCtlWords];
+    __shared__ ElxDecision s_decision;
+    {
+        const ElxStats *row = partials + (uint64_t)blockIdx.x * bpc;
+        double sum = 0.0;
+        uint32_t flag = 0;
+        for (uint32_t i = threadIdx.x; i < bpc; i += kStatsThreads) {
+            sum += row[i].sumsq;
+            flag |= row[i].overflow;
+        }
+        block_fold(sum, flag);
+        if (threadIdx.x == 0) {
+            __hip_atomic_store(reinterpret_cast<uint64_t *>(&stats[blockIdx.x].sumsq), __builtin_bit_cast(uint64_t, sum),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&stats[blockIdx.x].overflow, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&stats[blockIdx.x].reserved, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // release the record, then count this workgroup as done; the one that completes the count decides
+            const uint32_t done = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = done == n_chunks - 1 ? 1u : 0u;
+        }
+    }
+    __syncthreads();
+    if (!s_last) return;
+
+    // ---- the last workgroup: control block -> LDS (system-scope loads: it may live in host memory)
+    const uint32_t *cw = reinterpret_cast<const uint32_t *>(ctl);
+    for (uint32_t i = threadIdx.x; i < sizeof(ElxStepCtl) / 4u; i += kStatsThreads)
+        s_ctl[i] = __hip_atomic_load(cw + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __syncthreads();
+    const ElxStepCtl *c = reinterpret_cast<const ElxStepCtl *>(s_ctl);
+    const uint32_t cap = max_hypers < kMaxCtlHypers ? max_hypers : kMaxCtlHypers;
+    const bool valid = c->loss_scale > 0.0 && (!c->clipping || c->max_norm > 0.0) && c->n_hypers <= cap;
+    const uint32_t n_hypers = valid ? c->n_hypers : 0u;
+    for (uint32_t i = sizeof(ElxStepCtl) / 4u + threadIdx.x; i < (sizeof(ElxStepCtl) + n_hypers * sizeof(ElxHyper)) / 4u;
+         i += kStatsThreads)
+        s_ctl[i] = __hip_atomic_load(cw + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (threadIdx.x == 0) {
+        ElxDecision d = decide_from_stats(stats, n_chunks, valid ? c->loss_scale : 1.0, valid ? c->max_norm : 1.0,
+                                          valid ? (int)c->clipping : 0);
+        if (!valid) d.skip = 1u;    // an unusable control block: nothing is updated, and the report says why
+        s_decision = d;
+        *out = d;
+    }
+    __syncthreads();
+    const ElxDecision d = s_decision;
+    // the hyper table of the update launch: the step's records with the gate words of this decision.  When
+    // the control block is unusable every record the table can hold gets the skip gate.
+    const ElxHyper *src = reinterpret_cast<const ElxHyper *>(s_ctl + sizeof(ElxStepCtl) / 4u);
+    for (uint32_t i = threadIdx.x; i < (valid ? n_hypers : max_hypers); i += kStatsThreads) {
+        ElxHyper h = {};
+        if (valid) h = src[i];
+        h.gate_div_scale = d.div_scale;
+        h.gate_inv_scale = d.inv_scale;
+        h.gate = d.mode | (d.skip << 8);
+        hypers[i] = h;
+    }
+    if (report) {
+        const uint32_t *dw = reinterpret_cast<const uint32_t *>(&s_decision);
+        uint32_t *rw = reinterpret_cast<uint32_t *>(&report->decision);
+        for (uint32_t i = threadIdx.x; i < sizeof(ElxDecision) / 4u; i += kStatsThreads) store_system(rw + i, dw[i]);
+        ElxStats *rs = reinterpret_cast<ElxStats *>(report + 1);
+        for (uint32_t i = threadIdx.x; i < n_chunks; i += kStatsThreads) {
+            const uint64_t bits = __hip_atomic_load(reinterpret_cast<const uint64_t *>(&stats[i].sumsq), __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+            store_system(reinterpret_cast<uint64_t *>(&rs[i].sumsq), bits);
+            store_system(&rs[i].overflow, __hip_atomic_load(&stats[i].overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            store_system(&rs[i].reserved, 0u);
+        }
+        if (threadIdx.x == 0) {
+            store_system(&report->n_chunks, n_chunks);
+            store_system(&report->status, valid ? 0 : (int32_t)ELX_E_RANGE);
+        }
+        __threadfence_system();
+        __syncthreads();
+        if (threadIdx.x == 0)
+            __hip_atomic_store(&report->seq, c->seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1057,9 +1173,22 @@ int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t 
     return 0;
 }
 
+int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
+                         ElxStats *d_partials, int scalar_only, void *stream);
+
 int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
                       ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream) {
-    if (!d_chunks || !d_partials || !d_stats) return ELX_E_NULL;
+    if (!d_stats) return ELX_E_NULL;
+    if (int rc = elx_grad_partials_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, scalar_only, stream))
+        return rc;
+    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, (hipStream_t)stream, d_partials,
+                       blocks_per_chunk, d_stats);
+    return (int)hipGetLastError();
+}
+
+int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
+                         ElxStats *d_partials, int scalar_only, void *stream) {
+    if (!d_chunks || !d_partials) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxStatsBlocks)
         return ELX_E_SIZE;
     hipStream_t st = (hipStream_t)stream;
@@ -1077,11 +1206,25 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
             break;
         default: return ELX_E_DTYPE;
     }
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(stats_finish_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, st, d_partials, blocks_per_chunk, d_stats);
     return (int)hipGetLastError();
 }
+
+int elx_finish_decide(const ElxStats *d_partials, uint32_t n_chunks, uint32_t blocks_per_chunk, ElxStats *d_stats,
+                      const ElxStepCtl *ctl, ElxHyper *d_hypers, uint32_t max_hypers, ElxDecision *d_decision,
+                      ElxStepReport *report, uint32_t *d_counter, void *stream) {
+    if (!d_partials || !d_stats || !ctl || !d_decision || !d_counter || (max_hypers && !d_hypers)) return ELX_E_NULL;
+    if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxLandBlocks ||
+        max_hypers > kMaxCtlHypers)
+        return ELX_E_SIZE;
+    if (((uintptr_t)ctl | (uintptr_t)report | (uintptr_t)d_stats | (uintptr_t)d_decision) & 7u) return ELX_E_ALIGN;
+    hipLaunchKernelGGL(finish_decide_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, (hipStream_t)stream, d_partials,
+                       blocks_per_chunk, d_stats, n_chunks, ctl, d_hypers, max_hypers, d_decision, report, d_counter);
+    return (int)hipGetLastError();
+}
+
+uint32_t elx_sizeof_step_ctl(void) { return (uint32_t)sizeof(ElxStepCtl); }
+uint32_t elx_sizeof_step_report(void) { return (uint32_t)sizeof(ElxStepReport); }
+uint32_t elx_max_ctl_hypers(void) { return kMaxCtlHypers; }
 
 uint32_t elx_static_partials(void) { return kStaticPartials; }
 

@@ -257,23 +257,32 @@ class HybridAdam(torch.optim.Optimizer):
             self._plans[key] = dplan
         return dplan
 
-    def prepare_step(self) -> None:
+    def prepare_step(self, upload: bool = True) -> None:
         """Builds the tables of the next step without touching the optimizer state, so that a caller
         can overlap this host work with device work whose result decides whether the step happens
         (``ElixirOptimizer`` calls it between launching and reading the gradient flags).  The next
-        ``step()`` consumes what was prepared; ``discard_prepared()`` drops it."""
+        ``step()`` consumes what was prepared; ``discard_prepared()`` drops it.  ``upload`` False leaves
+        the hyper records on the host: the caller gets them to the device its own way (or the launch
+        uploads them after all)."""
         sig = self._prepare_signature()
         if self._prepared is not None and sig is not None and self._prepared.sig == sig:
-            return    # prepared ahead of time (ElixirOptimizer.backward does) and still valid
-        hypers: Dict = {}
-        if self._binding is not None:
-            self._prepared = self._prepare_bound(hypers)
+            prep = self._prepared    # prepared ahead of time (ElixirOptimizer.backward does) and still valid
         else:
-            self._prepared = self._prepare_standalone(hypers)
-        prep = self._prepared
-        if prep is not None:
-            prep.sig = sig
+            hypers: Dict = {}
+            if self._binding is not None:
+                self._prepared = self._prepare_bound(hypers)
+            else:
+                self._prepared = self._prepare_standalone(hypers)
+            prep = self._prepared
+            if prep is not None:
+                prep.sig = sig
+        if prep is not None and upload and not prep.d_hypers:
             prep.d_hypers = self._hyper_uploader.upload(prep.hyper_host, prep.device)
+
+    def adopt_prepared(self) -> None:
+        """The prepared step counts as launched without a launch from here: its launches were recorded
+        earlier (a HIP graph of the same tables) and the caller replays them."""
+        self._launched, self._prepared = self._prepared, None
 
     def _prepare_signature(self):
         """Everything a prepared step of bound chunks depends on besides the step counts (which only
@@ -315,6 +324,8 @@ class HybridAdam(torch.optim.Optimizer):
         if prep is None:
             return loss
 
+        if not prep.d_hypers:
+            prep.d_hypers = self._hyper_uploader.upload(prep.hyper_host, prep.device)
         plan = prep.dplan.plan
         stream = torch.cuda.current_stream(prep.device).cuda_stream
         events = self.kernel_events

@@ -64,16 +64,27 @@ def choose_block_elems(buffers: Sequence[FlatBuffer], tile: int) -> int:
     return max(16 * tile, min(block, _pow2_at_least(longest)))
 
 
+FOLD_PADDING_BELOW = 24 << 20    # elements: about 20 us of refresh, less than what a launch of its own costs a small set
+
+
 def build_plan(buffers: Sequence[FlatBuffer], grad_esize: int, lowp_esize: int, n_hypers: int, grad_dtype: int,
-               lowp_dtype: int) -> LaunchPlan:
+               lowp_dtype: int, fold_padding_below: int = FOLD_PADDING_BELOW) -> LaunchPlan:
+    """``fold_padding_below``: when the runs of pure padding hold fewer elements than this in total they
+    are listed as rows of the update launch (n_valid = 0: refreshed tile by tile there) instead of going
+    to a refresh launch of their own."""
     tile = _abi.tile_elems()
     block = choose_block_elems(buffers, tile)
     rows, segs, refresh = [], [], []
     tiles = 0
+    padding = sum(max(0, b.n_alloc - min(b.n_alloc, -(-b.n_valid // block) * block)) for b in buffers if b.lowp_out)
+    fold = 0 < padding < fold_padding_below
     for buf in buffers:
         assert 0 <= buf.n_valid <= buf.n_alloc
-        # the update covers whole blocks up to the one that holds the last valid element
+        # the update covers whole blocks up to the one that holds the last valid element (and, when the
+        # padding is folded in, the rest of the buffer as well)
         up_end = min(buf.n_alloc, -(-buf.n_valid // block) * block)
+        if fold and buf.lowp_out:
+            up_end = buf.n_alloc
         seg_arr = np.array(buf.segs, dtype=np.int64).reshape(-1, 3)
         if len(seg_arr):
             assert np.all(seg_arr[:, 0] < seg_arr[:, 1]) and np.all(seg_arr[1:, 0] >= seg_arr[:-1, 1]), \

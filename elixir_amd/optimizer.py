@@ -24,6 +24,7 @@ Differences from the reference, all on purpose:
   * shards in pinned host memory are stepped by the same launches, in place over the host link.
 """
 import math
+import time
 from collections import defaultdict
 from enum import Enum
 from typing import Dict, List, Set, Tuple
@@ -34,7 +35,7 @@ from torch.nn import Parameter
 
 from . import _abi
 from .chunk import (Chunk, DeviceTable, StatsArena, dtype_code, kernel_device, launch_grad_stats, read_grad_stats,
-                    resolve_pending_stats)
+                    resolve_pending_stats, stats_launch_blocks)
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
 from .hybrid_adam import HybridAdam
 
@@ -77,6 +78,72 @@ class _EventPair:
         if self.sink is not None:
             self.end.record()
         return False
+
+
+class _DeviceStep:
+    """Plumbing of a step that is decided on the device.
+
+    What changes from step to step (loss scale, clipping threshold, the hyper records) is written into a
+    control block in pinned host memory that the decision kernel reads; that kernel reports back into
+    pinned host memory, the sequence number last, and the host polls it.  No launch of the step takes
+    an argument that changes, so the launches can be recorded once as a HIP graph and replayed."""
+
+    POLL_LIMIT_S = 0.05    # then the stream is synchronised instead (the report has arrived by then)
+    MAX_GRAPHS = 4
+
+    def __init__(self, device: torch.device, n_chunks: int):
+        self.device, self.n_chunks = device, n_chunks
+        self.max_hypers = _abi.max_ctl_hypers()
+        ctl_head, rep_head = _abi.STEP_CTL_DTYPE.itemsize, _abi.STEP_REPORT_DTYPE.itemsize
+        hyp, rec = _abi.HYPER_DTYPE.itemsize, _abi.STATS_DTYPE.itemsize
+        self.ctl = torch.zeros(ctl_head + self.max_hypers * hyp, dtype=torch.uint8, pin_memory=True)
+        self.report = torch.zeros(rep_head + n_chunks * rec, dtype=torch.uint8, pin_memory=True)
+        self._ctl_bytes = self.ctl.numpy()
+        self._ctl_head = self._ctl_bytes[:ctl_head].view(_abi.STEP_CTL_DTYPE)
+        report_bytes = self.report.numpy()
+        self.report_head = report_bytes[:rep_head].view(_abi.STEP_REPORT_DTYPE)
+        self.report_stats = report_bytes[rep_head:].view(_abi.STATS_DTYPE)
+        # device side: hyper table of the update launch | decision | counter | per-chunk records
+        self.dev = torch.zeros(self.max_hypers * hyp + 64 + n_chunks * rec, dtype=torch.uint8, device=device)
+        base = self.dev.data_ptr()
+        self.d_hypers = base
+        self.d_decision = base + self.max_hypers * hyp
+        self.d_counter = self.d_decision + 32
+        self.d_stats = self.d_decision + 64
+        self.seq = 0
+        self.partials = None             # workspace of the stats launch
+        self.seen = set()                # launch sequences that have run once (eagerly)
+        self.graphs: Dict = {}           # launch sequence -> (graph, objects its launches point into)
+
+    def write_ctl(self, loss_scale: float, max_norm: float, clipping: bool, hyper_host: np.ndarray) -> int:
+        self.seq += 1
+        n = len(hyper_host)
+        head = self._ctl_head
+        at = head.itemsize
+        self._ctl_bytes[at:at + hyper_host.nbytes] = hyper_host.view(np.uint8).reshape(-1)
+        head['loss_scale'], head['max_norm'], head['clipping'], head['n_hypers'] = loss_scale, max_norm, int(clipping), n
+        head['seq'] = self.seq
+        return self.seq
+
+    def partials_buffer(self, records: int) -> int:
+        need = records * _abi.STATS_DTYPE.itemsize
+        if self.partials is None or self.partials.numel() < need:
+            self.partials = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return self.partials.data_ptr()
+
+    def wait_report(self, seq: int, stream: torch.cuda.Stream):
+        """Polls the sequence number of the report; returns (decision record, per-chunk records)."""
+        head = self.report_head
+        give_up = time.perf_counter() + self.POLL_LIMIT_S
+        while int(head['seq'][0]) != seq:
+            if time.perf_counter() > give_up:
+                stream.synchronize()
+                if int(head['seq'][0]) != seq:
+                    raise RuntimeError('the decision kernel has run but its report did not arrive in host memory')
+                break
+        if int(head['status'][0]) != 0:
+            raise RuntimeError(f'the decision kernel refused its control block (status {int(head["status"][0])})')
+        return head[0], self.report_stats
 
 
 class ElixirOptimizer(torch.optim.Optimizer):
@@ -158,11 +225,15 @@ class ElixirOptimizer(torch.optim.Optimizer):
             if ranges:
                 self._binding = self.optim.bind_chunks(ranges)
         self._stats_table = None
+        self._all_stats_table = None
         self._stats_workspace: Dict = {}
         # the step decided on the device (no wait between the flags and the update); False: the host
         # fetches the flags, decides and only then launches
         self.gated_step = True
-        self._gate = None
+        # with gated_step: record the launches of a step once as a HIP graph and replay it (from the third
+        # step with the same tables on; nothing is recorded while kernel_events is set)
+        self.graph_step = False
+        self._device_step: _DeviceStep = None
         self._wb_table = None
         self.last_step_info: Dict = {}
         # when set to a dict, step() records (begin, end) torch.cuda.Event pairs on the launch
@@ -435,68 +506,97 @@ class ElixirOptimizer(torch.optim.Optimizer):
 
     # ------------------------------------------------------------------ the step, decided on the device
 
-    def _gate_buffers(self, device: torch.device, n_chunks: int):
-        g = self._gate
-        if g is None or g['device'] != device or g['host'].numel() < n_chunks * _abi.STATS_DTYPE.itemsize + 32:
-            g = self._gate = dict(device=device, decision=torch.zeros(32, dtype=torch.uint8, device=device),
-                                  host=torch.zeros(n_chunks * _abi.STATS_DTYPE.itemsize + 32, dtype=torch.uint8,
-                                                   pin_memory=True),
-                                  side=torch.cuda.Stream(device), decided=torch.cuda.Event(), copied=torch.cuda.Event())
-        return g
-
-    def _records_of_all_chunks(self, launched):
-        """The address of ONE run of ElxStats records that covers every parameter chunk in list order,
-        or None: either this step's stats launch covered them all, or fused landings left them all
-        in consecutive arena slots."""
+    def _stats_source(self):
+        """Where the decision kernel finds the flags of ALL parameter chunks, or None when they are not
+        all in one place: ('launch', None) -- no chunk has flags, one stats launch over all of them is
+        needed -- or ('arena', first slot) -- fused landings left every chunk's record in consecutive
+        slots of the device arena."""
         chunks = self._param_chunk_list
-        if launched is not None:
-            pending, records = launched
-            return records if len(pending) == len(chunks) else None
-        if not chunks or not all(c._stats_pending for c in chunks):
+        if not chunks:
             return None
-        first = chunks[0]._stats_slot
-        if any(c._stats_slot != first + i for i, c in enumerate(chunks)):
-            return None
-        device = kernel_device(c.shard for c in chunks)
-        main = torch.cuda.current_stream(device)
-        for event in {c._stats_event for c in chunks if c._stats_event is not None}:
-            main.wait_event(event)    # the landings may have run on another stream
-        arena = StatsArena.get(chunks[0].shard_device)
-        rec = arena.itemsize
-        return arena.buf[first * rec:(first + len(chunks)) * rec]
+        if all(not c._stats_fresh and not c._stats_pending for c in chunks):
+            return ('launch', None)
+        if all(c._stats_pending for c in chunks):
+            first = chunks[0]._stats_slot
+            if all(c._stats_slot == first + i for i, c in enumerate(chunks)):
+                return ('arena', first)
+        return None
 
-    def _step_gated(self, launched, records) -> bool:
+    def _all_chunks_stats_table(self, device: torch.device):
+        chunks = self._param_chunk_list
+        ids = tuple(c.chunk_id for c in chunks)
+        ptrs = tuple(c.shard.data_ptr() for c in chunks)
+        if self._all_stats_table is None or self._all_stats_table[0] != (ids, ptrs):
+            rows = np.zeros(len(chunks), dtype=_abi.CHUNK_DTYPE)
+            for i, c in enumerate(chunks):
+                rows[i]['grad'] = c.shard.data_ptr()
+                rows[i]['n_alloc'] = c.shard_size
+                rows[i]['n_valid'] = c.n_valid
+            self._all_stats_table = ((ids, ptrs), rows, DeviceTable(rows, device))
+        return self._all_stats_table[1], self._all_stats_table[2]
+
+    def _step_on_device(self, source) -> bool:
         """The step without a wait between the flags and the update: the decisions of
-        optimizer.py:137-183 are taken by a one-thread kernel that leaves them in the hyper table of
-        the update launch; the update is enqueued at once and reads them there (on a skip it only
-        refreshes the low-precision copies).  The flags and the decision travel to the host on a side
-        stream meanwhile, for the host's bookkeeping (scaler, step counts, chunk flags).  Returns False
-        when nothing was prepared to launch."""
+        optimizer.py:137-183 are taken by the kernel that folds the flags, which leaves them in the hyper
+        table of the update launch; the update is enqueued right behind it and reads them there (on a skip
+        it only refreshes the low-precision copies).  The decision and the flags come back through pinned
+        host memory while the update runs, for the host's bookkeeping (scaler, step counts, chunk flags).
+        Returns False when nothing was prepared to launch this way."""
         inner = self.optim
+        inner.prepare_step(upload=False)
         prep = inner._prepared
-        if prep is None or prep.dplan.rows is None:
+        if prep is None or prep.dplan.rows is None or len(prep.hyper_host) > _abi.max_ctl_hypers():
             return False
         chunks = self._param_chunk_list
-        n, rec = len(chunks), _abi.STATS_DTYPE.itemsize
-        g = self._gate_buffers(prep.device, n)
+        n = len(chunks)
+        eng = self._device_step
+        if eng is None or eng.device != prep.device or eng.n_chunks != n:
+            eng = self._device_step = _DeviceStep(prep.device, n)
         main = torch.cuda.current_stream(prep.device)
-        _abi.decide(records.data_ptr(), n, float(self.loss_scale), float(self.max_norm), self.clipping_flag,
-                    prep.d_hypers, len(prep.hyper_host), g['decision'].data_ptr(), main.cuda_stream)
-        decided = g['decided']    # reused: the wait on 'copied' below ends before the next step records it again
-        decided.record(main)
-        with self._timed('update'):
-            inner.launch_step(gated=True, defer_commit=True)
+        kind, first_slot = source
+        if kind == 'launch':
+            rows, table = self._all_chunks_stats_table(prep.device)
+            bpc = stats_launch_blocks(int(rows['n_valid'].max()))
+            partials = eng.partials_buffer(n * bpc)
+            stats_args = (table.ptr, n, dtype_code(chunks[0].chunk_dtype), bpc, partials,
+                          not bool(np.all(rows['grad'] % 16 == 0)))
+            keep = (table, eng.partials)
+        else:
+            arena = StatsArena.get(chunks[0].shard_device)
+            for event in {c._stats_event for c in chunks if c._stats_event is not None}:
+                main.wait_event(event)    # the landings may have run on another stream
+            bpc, partials, stats_args, keep = 1, arena.ptr(first_slot), None, (arena, )
+        seq = eng.write_ctl(float(self.loss_scale), float(self.max_norm), self.clipping_flag, prep.hyper_host)
+        prep.d_hypers = eng.d_hypers
 
-        side = g['side']
-        side.wait_event(decided)
-        with torch.cuda.stream(side):
-            g['host'][:n * rec].copy_(records, non_blocking=True)
-            g['host'][n * rec:n * rec + 32].copy_(g['decision'], non_blocking=True)
-            g['copied'].record(side)
-        g['copied'].synchronize()
-        host = g['host'].numpy()
-        stats = host[:n * rec].view(_abi.STATS_DTYPE)
-        device_says = host[n * rec:n * rec + 32].view(_abi.DECISION_DTYPE)[0]
+        def enqueue():
+            stream = torch.cuda.current_stream(prep.device).cuda_stream
+            with self._timed('stats' if stats_args is not None else 'decide'):
+                if stats_args is not None:
+                    _abi.grad_partials_mt(*stats_args, stream)
+                _abi.finish_decide(partials, n, bpc, eng.d_stats, eng.ctl.data_ptr(), eng.d_hypers, eng.max_hypers,
+                                   eng.d_decision, eng.report.data_ptr(), eng.d_counter, stream)
+            with self._timed('update'):
+                inner.launch_step(gated=True, defer_commit=True)
+
+        timing = self.kernel_events is not None or inner.kernel_events is not None
+        key = (id(prep.dplan), kind, partials, bpc, inner.blocks_per_cu, stats_args[0] if stats_args else 0)
+        if self.graph_step and not timing and key in eng.graphs:
+            inner.adopt_prepared()
+            eng.graphs[key][0].replay()
+        elif self.graph_step and not timing and key in eng.seen:
+            if len(eng.graphs) >= eng.MAX_GRAPHS:
+                eng.graphs.clear()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, capture_error_mode='thread_local'):
+                enqueue()
+            eng.graphs[key] = (graph, prep.dplan, keep)    # what the recorded launches point into stays alive
+            graph.replay()
+        else:
+            eng.seen.add(key)
+            enqueue()
+
+        device_says, stats = eng.wait_report(seq, main)
         for c, r in zip(chunks, stats):
             c._stats_pending = False
             c._stats_event = None
@@ -525,15 +625,14 @@ class ElixirOptimizer(torch.optim.Optimizer):
     # ------------------------------------------------------------------ the step
 
     def step(self, *args, **kwargs):
-        launched = self._launch_chunk_stats()
         if (self.gated_step and self._binding is not None and self.scaled_optimizer and not args and not kwargs
                 and not self._binding.zero_grads and self.optim_state == OptimState.SCALED):
-            records = self._records_of_all_chunks(launched)
-            if records is not None:
-                self.optim.prepare_step()
+            source = self._stats_source()
+            if source is not None:
                 self._set_grad_ptr()
-                if self._step_gated(launched, records):
+                if self._step_on_device(source):
                     return None
+        launched = self._launch_chunk_stats()
         if self._binding is not None and not args and not kwargs:
             # host work of the update launch, done while the flags pass runs on the device
             self.optim.prepare_step()
@@ -588,7 +687,8 @@ class ElixirOptimizer(torch.optim.Optimizer):
         if a hyper-parameter has changed in between)."""
         if self._binding is not None:
             try:
-                self.optim.prepare_step()
+                # a step decided on the device hands the hyper records over in its control block
+                self.optim.prepare_step(upload=not self.gated_step)
             except RuntimeError:
                 self.optim.discard_prepared()    # nothing to prepare for: step() is where the refusal belongs
 

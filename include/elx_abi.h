@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define ELX_ABI_VERSION 1
+#define ELX_ABI_VERSION 2
 
 /* element types of gradient / low-precision buffers */
 enum { ELX_F32 = 0, ELX_F16 = 1, ELX_BF16 = 2, ELX_NONE = -1 };
@@ -135,6 +135,32 @@ typedef struct ElxDecision {
     double combined_scale; /* loss scale x clip coefficient as a float64, -1 when it equals 1 */
 } ElxDecision;
 
+/*
+ * Control block of one step for elx_finish_decide: what changes from step to step, kept in memory so
+ * that the launches of a step take the same arguments every time (and can be replayed from a recorded
+ * HIP graph).  The host rewrites it before every step; it may live in device memory or in pinned host
+ * memory (the kernel reads it with system-scope loads).  n_hypers ElxHyper records follow it directly.
+ */
+typedef struct ElxStepCtl {
+    double loss_scale;  /* > 0 */
+    double max_norm;    /* > 0 when clipping */
+    uint32_t clipping;  /* 0 / 1 */
+    uint32_t n_hypers;  /* records that follow; at most elx_max_ctl_hypers() and the max_hypers of the call */
+    uint64_t seq;       /* any number the host chooses; echoed in ElxStepReport.seq */
+} ElxStepCtl;
+
+/*
+ * What elx_finish_decide reports back: the decision, then one ElxStats record per chunk directly behind
+ * this header.  Written with system-scope stores, `seq` last (release): a host that polls `seq` in pinned
+ * host memory and finds the number it put into the control block may read the rest.
+ */
+typedef struct ElxStepReport {
+    ElxDecision decision;
+    uint64_t seq;
+    uint32_t n_chunks;
+    int32_t status;     /* 0, or ELX_E_RANGE when the control block was unusable (then decision.skip = 1) */
+} ElxStepReport;
+
 /* ABI version of the loaded library (ELX_ABI_VERSION). */
 int elx_version(void);
 
@@ -150,6 +176,8 @@ uint32_t elx_sizeof_seg(void);
 uint32_t elx_sizeof_hyper(void);
 uint32_t elx_sizeof_stats(void);
 uint32_t elx_sizeof_decision(void);
+uint32_t elx_sizeof_step_ctl(void);
+uint32_t elx_sizeof_step_report(void);
 
 /*
  * Host-side validation of HOST copies of the tables, to be called once before they are uploaded:
@@ -175,6 +203,34 @@ int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *
  */
 int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
                       ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream);
+
+/*
+ * The first launch of elx_grad_stats_mt alone: n_chunks * blocks_per_chunk partials, chunk by chunk, left
+ * for elx_finish_decide (or any fold of the caller's) to reduce.
+ */
+int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
+                         ElxStats *d_partials, int scalar_only, void *stream);
+
+/*
+ * The fold of the partials and elx_decide in one launch whose arguments do not change from step to step:
+ * loss scale, clipping threshold and the hyper records of the step come from *ctl.  Per chunk the
+ * blocks_per_chunk partials at d_partials are folded exactly as elx_grad_stats_mt folds them into
+ * d_stats (with blocks_per_chunk = 1 the "partials" are finished records, e.g. those a landing launch
+ * left: 1..elx_land_max_blocks()); then the decisions of optimizer.py:137-183 are taken as by elx_decide,
+ * the ctl->n_hypers records behind *ctl are copied to d_hypers with their gate words filled in (the table
+ * elx_adam_step_gated_mt reads next on the same stream), *d_decision is written and, when `report` is not
+ * NULL, so is the report (see ElxStepReport; room for n_chunks ElxStats records behind the header).
+ *   max_hypers  capacity of d_hypers in records, at most elx_max_ctl_hypers()
+ *   d_counter   one uint32 of device memory, zero before the first call; the launch leaves it zero
+ * An unusable control block (loss_scale <= 0, n_hypers > max_hypers ...) cannot be refused by the host
+ * (it may be device memory): the kernel then sets the skip gate in all max_hypers records, so that the
+ * update launch changes nothing, and reports status ELX_E_RANGE.
+ */
+int elx_finish_decide(const ElxStats *d_partials, uint32_t n_chunks, uint32_t blocks_per_chunk, ElxStats *d_stats,
+                      const ElxStepCtl *ctl, ElxHyper *d_hypers, uint32_t max_hypers, ElxDecision *d_decision,
+                      ElxStepReport *report, uint32_t *d_counter, void *stream);
+
+uint32_t elx_max_ctl_hypers(void);
 
 /*
  * elx_grad_stats_mt without a workspace argument, for callers that cannot allocate one (code under

@@ -246,7 +246,7 @@ def test_optimizer_ranges_groups_and_refusal_to_run_on_cpu():
         ea.ElixirOptimizer(m32, ea.HybridAdam(m32.parameters()), max_norm=1.0, norm_type=1.0)
     # no GPU, no step: the product has no CPU path
     opt.mark_gradients_scaled()
-    with pytest.raises(RuntimeError, match='HIP'):
+    with pytest.raises(RuntimeError, match='HIP|GPU'):
         opt.step()
     p = nn.Parameter(torch.zeros(4))
     p.grad = torch.ones(4)
@@ -298,7 +298,7 @@ def test_launch_plan_blocks_segments_and_padding():
     # a 64 Ki-element buffer with 40,000 valid elements in three tensors; the rest is padding
     buf = FlatBuffer(grad=base, lowp_out=base, master=base + (1 << 24), m=base + (2 << 24), v=base + (3 << 24),
                      n_alloc=65536, n_valid=40000, segs=[(0, 5000, 0), (5000, 5003, 1), (5003, 40000, 0)])
-    plan = build_plan([buf], 2, 2, 2, _abi.ELX_F16, _abi.ELX_F16)
+    plan = build_plan([buf], 2, 2, 2, _abi.ELX_F16, _abi.ELX_F16, fold_padding_below=0)
     B = plan.block_elems
     assert B % tile == 0 and B >= 16 * tile
     n_rows = -(-40000 // B)
@@ -328,8 +328,21 @@ def test_launch_plan_blocks_segments_and_padding():
     assert build_plan([solo], 4, 4, 1, _abi.ELX_F32, _abi.ELX_NONE).refresh_rows is None
     empty = FlatBuffer(grad=base, lowp_out=base, master=base + (1 << 24), m=base + (2 << 24), v=base + (3 << 24),
                        n_alloc=65536, n_valid=0, segs=[])
-    plan = build_plan([empty], 2, 2, 1, _abi.ELX_F16, _abi.ELX_F16)
+    plan = build_plan([empty], 2, 2, 1, _abi.ELX_F16, _abi.ELX_F16, fold_padding_below=0)
     assert len(plan.rows) == 0 and plan.refresh_rows[0]['n_alloc'] == 65536
+    # a little padding rides the update launch instead: every block of the buffer is a row (those behind the
+    # valid head with no valid element and no segment), and there is no refresh launch
+    for b in (buf, empty):
+        folded = build_plan([b], 2, 2, 2, _abi.ELX_F16, _abi.ELX_F16)
+        assert folded.refresh_rows is None and len(folded.rows) == -(-65536 // folded.block_elems)
+        assert int(folded.rows['n_alloc'].sum()) == 65536 and int(folded.rows['n_valid'].sum()) == b.n_valid
+        tail = folded.rows[folded.rows['n_valid'] == 0]
+        assert all(r['seg_begin'] == r['seg_end'] for r in tail)
+    # ... but not when there is a lot of it
+    big = FlatBuffer(grad=base, lowp_out=base, master=base + (1 << 32), m=base + (2 << 32), v=base + (3 << 32),
+                     n_alloc=1 << 26, n_valid=1 << 20, segs=[(0, 1 << 20, 0)])
+    plan = build_plan([big], 2, 2, 1, _abi.ELX_F16, _abi.ELX_F16)
+    assert plan.refresh_rows is not None and int(plan.rows['n_alloc'].sum()) + int(plan.refresh_rows['n_alloc'].sum()) == 1 << 26
 
 
 def test_launch_plan_keeps_rows_bounded_for_the_large_workloads():
