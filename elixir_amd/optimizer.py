@@ -230,8 +230,8 @@ class ElixirOptimizer(torch.optim.Optimizer):
         # the step decided on the device (no wait between the flags and the update); False: the host
         # fetches the flags, decides and only then launches
         self.gated_step = True
-        # with gated_step: record the launches of a step once as a HIP graph and replay it (from the third
-        # step with the same tables on; nothing is recorded while kernel_events is set)
+        # with gated_step: record the launches of a step once as a HIP graph and replay it (the first step
+        # over a set of tables runs eagerly, the second records; nothing is recorded while kernel_events is set)
         self.graph_step = False
         self._device_step: _DeviceStep = None
         self._wb_table = None

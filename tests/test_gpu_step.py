@@ -904,6 +904,178 @@ def test_decide_kernel_matches_host_arithmetic(oracle):
     assert cases > 200
 
 
+def test_finish_decide_matches_the_two_separate_launches():
+    """elx_finish_decide (fold of the partials + decision in one launch, everything that changes read
+    from a control block, the result reported into pinned host memory) against elx_grad_stats_mt followed
+    by elx_decide on the same gradients: identical per-chunk records, decision and gate words, the step's
+    hyper records copied unchanged, the report complete when its sequence number shows, the counter left
+    at zero.  The control block sits in pinned host memory in odd trials and in device memory in even
+    ones; an unusable control block closes every gate and says so."""
+    rng = np.random.default_rng(17)
+    stream = torch.cuda.current_stream().cuda_stream
+    rec, hsz = _abi.STATS_DTYPE.itemsize, _abi.HYPER_DTYPE.itemsize
+    ctl_head, rep_head = _abi.STEP_CTL_DTYPE.itemsize, _abi.STEP_REPORT_DTYPE.itemsize
+    H = _abi.max_ctl_hypers()
+    assert (ctl_head, rep_head, H) == (32, 48, 64)
+    counter = torch.zeros(4, dtype=torch.int32, device=DEV)
+    for trial in range(24):
+        n = int(rng.integers(1, 9))
+        bpc = int(rng.choice([1, 3, 64, 1024]))
+        dtype = [torch.float16, torch.bfloat16, torch.float32][trial % 3]
+        sizes = [int(rng.integers(1, 200_000)) for _ in range(n)]
+        gen = torch.Generator(device=DEV).manual_seed(trial)
+        grads = [(torch.randn(k, generator=gen, device=DEV) * float(rng.choice([1e-3, 1.0, 50.0]))).to(dtype) for k in sizes]
+        overflow = trial % 5 == 2
+        if overflow:
+            grads[int(rng.integers(0, n))][0] = float('nan')
+        rows = np.zeros(n, dtype=_abi.CHUNK_DTYPE)
+        for i, g in enumerate(grads):
+            rows[i]['grad'], rows[i]['n_alloc'], rows[i]['n_valid'] = g.data_ptr(), g.numel(), g.numel()
+        table = DeviceTableOf(rows)
+        n_hyp = int(rng.integers(1, 6))
+        hyp_host = np.concatenate([ea.hybrid_adam.make_hyper_record(1e-3 * (k + 1), 0.9, 0.999, 1e-8, 0.01 * k, 1 + k, True,
+                                                                    k % 2 == 0) for k in range(n_hyp)])
+        loss_scale = float(rng.choice([1.0, 64.0, 65536.0, 3.0]))
+        max_norm = float(rng.choice([0.0, 0.5, 2.5]))
+
+        # the two separate launches
+        ws = torch.empty((n * bpc + n) * rec, dtype=torch.uint8, device=DEV)
+        _abi.grad_stats_mt(table.ptr, n, CODE[dtype], bpc, ws.data_ptr(), ws.data_ptr() + n * bpc * rec, False, stream)
+        hyp_a = torch.from_numpy(hyp_host.view(np.uint8).copy()).to(DEV)
+        dec_a = torch.zeros(32, dtype=torch.uint8, device=DEV)
+        _abi.decide(ws.data_ptr() + n * bpc * rec, n, loss_scale, max_norm, max_norm > 0, hyp_a.data_ptr(), n_hyp,
+                    dec_a.data_ptr(), stream)
+
+        # the one launch
+        ctl = torch.zeros(ctl_head + H * hsz, dtype=torch.uint8, pin_memory=True)
+        cb = ctl.numpy()
+        head = cb[:ctl_head].view(_abi.STEP_CTL_DTYPE)
+        head['loss_scale'], head['max_norm'], head['clipping'], head['n_hypers'], head['seq'] = \
+            loss_scale, max_norm, int(max_norm > 0), n_hyp, 1000 + trial
+        cb[ctl_head:ctl_head + hyp_host.nbytes] = hyp_host.view(np.uint8).reshape(-1)
+        ctl_dev = ctl if trial % 2 else ctl.to(DEV)
+        report = torch.zeros(rep_head + n * rec, dtype=torch.uint8, pin_memory=True)
+        partials = torch.empty(n * bpc * rec, dtype=torch.uint8, device=DEV)
+        stats_b = torch.zeros(n * rec, dtype=torch.uint8, device=DEV)
+        hyp_b = torch.full((H * hsz, ), 0xEE, dtype=torch.uint8, device=DEV)
+        dec_b = torch.zeros(32, dtype=torch.uint8, device=DEV)
+        _abi.grad_partials_mt(table.ptr, n, CODE[dtype], bpc, partials.data_ptr(), False, stream)
+        _abi.finish_decide(partials.data_ptr(), n, bpc, stats_b.data_ptr(), ctl_dev.data_ptr(), hyp_b.data_ptr(), H,
+                           dec_b.data_ptr(), report.data_ptr(), counter.data_ptr(), stream)
+        torch.cuda.synchronize()
+        assert ws[n * bpc * rec:].cpu().numpy().tobytes() == stats_b.cpu().numpy().tobytes(), trial
+        assert dec_a.cpu().numpy().tobytes() == dec_b.cpu().numpy().tobytes(), trial
+        assert hyp_a.cpu().numpy().tobytes() == hyp_b[:n_hyp * hsz].cpu().numpy().tobytes(), trial
+        assert bool((hyp_b[n_hyp * hsz:] == 0xEE).all())          # nothing written behind the step's records
+        rb = report.numpy()
+        rh = rb[:rep_head].view(_abi.STEP_REPORT_DTYPE)[0]
+        assert rh['seq'] == 1000 + trial and rh['n_chunks'] == n and rh['status'] == 0
+        assert rb[:32].tobytes() == dec_b.cpu().numpy().tobytes()
+        assert rb[rep_head:].tobytes() == stats_b.cpu().numpy().tobytes()
+        assert bool(rh['skip']) == overflow
+        assert int(counter[0]) == 0
+
+    # finished records as "partials" (one per chunk, as a landing launch leaves them)
+    recs = np.zeros(3, dtype=_abi.STATS_DTYPE)
+    recs['sumsq'] = [4.0, 9.0, 12.0]
+    d_recs = torch.from_numpy(recs.view(np.uint8).copy()).to(DEV)
+    head['loss_scale'], head['max_norm'], head['clipping'], head['n_hypers'], head['seq'] = 2.0, 1.0, 1, 1, 77
+    report = torch.zeros(rep_head + 3 * rec, dtype=torch.uint8, pin_memory=True)
+    _abi.finish_decide(d_recs.data_ptr(), 3, 1, stats_b.data_ptr(), ctl.data_ptr(), hyp_b.data_ptr(), H, dec_b.data_ptr(),
+                       report.data_ptr(), counter.data_ptr(), stream)
+    torch.cuda.synchronize()
+    rh = report.numpy()[:rep_head].view(_abi.STEP_REPORT_DTYPE)[0]
+    assert rh['seq'] == 77 and rh['total_norm'] == 5.0 and rh['combined_scale'] == ((5.0 / 2.0) + 1e-6) / 1.0 * 2.0
+
+    # an unusable control block: every gate closed, status says why, nothing else happens
+    for bad in (dict(loss_scale=0.0), dict(n_hypers=H + 1), dict(clipping=1, max_norm=0.0)):
+        head['loss_scale'], head['max_norm'], head['clipping'], head['n_hypers'], head['seq'] = 2.0, 1.0, 0, 1, 99
+        for k, val in bad.items():
+            head[k] = val
+        hyp_b.fill_(0)
+        _abi.finish_decide(d_recs.data_ptr(), 3, 1, stats_b.data_ptr(), ctl.data_ptr(), hyp_b.data_ptr(), H,
+                           dec_b.data_ptr(), report.data_ptr(), counter.data_ptr(), stream)
+        torch.cuda.synchronize()
+        rh = report.numpy()[:rep_head].view(_abi.STEP_REPORT_DTYPE)[0]
+        assert rh['seq'] == 99 and rh['status'] == _abi.ELX_E_RANGE and rh['skip'] == 1
+        gates = hyp_b.cpu().numpy().view(_abi.HYPER_DTYPE)
+        assert len(gates) == H and all(int(g) >> 8 == 1 for g in gates['gate'])
+    with pytest.raises(_abi.ElxError):
+        _abi.finish_decide(d_recs.data_ptr(), 3, 1, stats_b.data_ptr(), ctl.data_ptr(), hyp_b.data_ptr(), H + 1,
+                           dec_b.data_ptr(), report.data_ptr(), counter.data_ptr(), stream)
+
+
+def DeviceTableOf(rows):
+    from elixir_amd.chunk import DeviceTable
+    return DeviceTable(rows, torch.device(DEV, 0))
+
+
+@pytest.mark.parametrize('fused_landing', [False, True])
+def test_recorded_step_replays_like_the_eager_one(oracle, fused_landing):
+    """A seven-step trajectory -- clean steps, an overflow that only arms the back-off (hysteresis 2),
+    one that backs off, clean steps until the scale grows again -- three times: decided on the host,
+    decided on the device with eager launches, and with the launches of the step recorded as a HIP
+    graph and replayed (the first step runs eagerly, the second records, all later ones replay -- the
+    overflows among them).  Identical bits in every buffer after every step, identical scale, reports and step counts;
+    the eager run is also held against the oracle."""
+    dtype = torch.float16
+    overflow_at = {3, 4}
+    runs = []
+    for mode in ('host', 'eager', 'graph'):
+        module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=19, grad_std=2e-2, loss_scale=512.0,
+                                              weight_decay=0.1, max_norm=1.0, initial_scale=512.0, hysteresis=2,
+                                              growth_interval=2)
+        opt.gated_step = mode != 'host'
+        opt.graph_step = mode == 'graph'
+        scaler = O.DynamicGradScalerOracle(initial_scale=512.0, min_scale=1, max_scale=2**24, hysteresis=2,
+                                           growth_interval=2)
+        gen = torch.Generator(device=DEV).manual_seed(23)
+        trace = []
+        for step in range(7):
+            payloads = []
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (2e-2 * opt.loss_scale)
+                g[pc.utilized_size:] = 0
+                g = g.to(dtype)
+                if step in overflow_at and pc is module.param_chunks[1]:
+                    g[5] = float('inf')
+                payloads.append(g)
+            if fused_landing:
+                from elixir_amd.chunk import land_chunks
+                land_chunks(module.param_chunks, payloads)
+            else:
+                for pc, g in zip(module.param_chunks, payloads):
+                    pc.shard.copy_(g)
+                    pc.invalidate_stats()
+            torch.cuda.synchronize()    # eager work and a synchronisation between the replays
+            if mode == 'eager':
+                refresh_oracle_grads(module, ochunks)
+                _run_and_compare(module, opt, ochunks, dtype, scaler, max_norm=1.0, tag=f'step {step}')
+                compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-8, atol_v=1e-10,
+                              tag=f'step {step}')
+            else:
+                opt.mark_gradients_scaled()
+                opt.step()
+            info = dict(opt.last_step_info)
+            trace.append((info, opt.loss_scale, sorted(st['step'] for st in opt.state.values()),
+                          [(pc.paired_chunk.shard.clone(), pc.shard.clone(),
+                            *[t.clone() for t in opt._binding.moments(pc.paired_chunk)]) for pc in module.param_chunks]))
+        if mode == 'graph':
+            assert len(opt._device_step.graphs) == 1
+        runs.append(trace)
+    assert [t[0]['found_inf'] for t in runs[0]] == [False, False, False, True, True, False, False]
+    assert [t[1] for t in runs[0]] == [512.0, 1024.0, 1024.0, 1024.0, 512.0, 512.0, 1024.0]
+    for other in runs[1:]:
+        for step, (a, b) in enumerate(zip(runs[0], other)):
+            assert a[1] == b[1] and a[2] == b[2], step
+            assert a[0]['found_inf'] == b[0]['found_inf'] and a[0]['chunk_overflow'] == b[0]['chunk_overflow'], step
+            if not a[0]['found_inf']:
+                assert a[0]['combined_scale'] == b[0]['combined_scale'] and a[0]['total_norm'] == b[0]['total_norm'], step
+            for x, y in zip(a[3], b[3]):
+                for s, t in zip(x, y):
+                    assert torch.equal(s, t), step
+
+
 def test_device_decided_and_host_decided_steps_agree(oracle):
     """The same three steps (clean, overflow, clean) with the decisions on the device and on the host:
     identical state, scale and reports."""
