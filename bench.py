@@ -1,14 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the optimizer step (ElixirOptimizer.step over chunk-packed parameters) on one GPU.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c2|c1|velocity]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c2|c1|velocity] [--no-configs]
 
 A step is one full pass of the hot path over one set of synthetic gradients that already sit in
-the low-precision chunk shards: stats launch (overflow flag + sum of squares) -> decision kernel
-(skip, global norm, combined scale) -> fused unscale + AdamW + low-precision writeback launch ->
-refresh of the padding; the flags and the decision reach the host on a side stream for its
-bookkeeping.  Step time is host wall-clock between two device synchronisations, so host overhead
-counts.  Prints ONE JSON line.
+the low-precision chunk shards: stats launch (overflow flag + sum of squares) -> fold + decision
+kernel (skip, global norm, combined scale) -> fused unscale + AdamW + low-precision writeback launch
+-> refresh of the padding; the decision and the flags reach the host through pinned memory for its
+bookkeeping while the update runs.  Step time is host wall-clock between two device
+synchronisations, so host overhead counts.  Prints ONE JSON line: the headline workload (c5 unless
+--workload says otherwise) and, on the default run, a `configs` object with the other configurations
+(c1, c2, c4 and the reference's own flat-parameter micro-benchmark) measured the same way.
 """
 import argparse
 import json
@@ -27,11 +29,34 @@ HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
 BYTES_UPDATE = 28               # per valid element: read g(2)+p,m,v(12); write p,m,v(12)+lowp(2)
 BYTES_STATS = 2                 # per valid element: the compulsory second read of g
 # HBM bytes per adam_step_kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script, scaled by what the same counters read for a plain copy of known size (--calibrate-copy):
-# 94.411e9 read + 94.364e9 written for c5, i.e. the algorithmic 188.676e9 plus the padding inside
-# the last block of each chunk.  (The padding refresh launch moves another 1.984e9 + 0.992e9.)
-# Counter runs cannot ride along with a timed run, hence a recorded figure.
-MEASURED_TRAFFIC_BYTES = {'c5': 188.775e9}
+# script, scaled by what the same counters read for a plain copy of known size (--calibrate-copy).
+# Counter runs cannot ride along with a timed run, so the figure is a recorded one: it is only put into
+# the line while the kernel source is still the one it was measured on (sha256 of elx_kernels.hip,
+# first 16 hex digits), and the line names the summary it comes from.
+RECORDED_TRAFFIC = {
+    # workload: (bytes per launch, summary under profiles/, kernel source the counters were read on)
+}
+KERNEL_SOURCE = os.path.join(ROOT, 'elixir_amd', 'csrc', 'elx_kernels.hip')
+
+
+def kernel_source_sha16() -> str:
+    import hashlib
+    with open(KERNEL_SOURCE, 'rb') as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def traffic_fields(workload: str):
+    """(traffic, traffic_source) of the roofline object: the recorded counter figure when it was read on
+    the kernel source that is built now, else None with the reason."""
+    rec = RECORDED_TRAFFIC.get(workload)
+    if rec is None:
+        return None, None
+    nbytes, summary, sha = rec
+    now = kernel_source_sha16()
+    if sha != now:
+        return None, {'summary': summary, 'note': f'counters were read on kernel source {sha}, this build is {now}: stale'}
+    return nbytes, {'summary': summary, 'kernel_source_sha16': sha,
+                    'method': 'rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy of known size'}
 
 
 def cpu_baseline(built, sample_elems: int, steps: int = 8):
@@ -76,6 +101,8 @@ def cpu_baseline(built, sample_elems: int, steps: int = 8):
         'kind': 'port',
         'sample': f'first {n} elements of chunk 0 of {spec.name}; torch CPU ops (isinf/isnan, float().norm, '
                   f'float().div_, torch.optim.AdamW, .to(lowp)); median of {steps} steps after 1 warm-up',
+        'extrapolation': f'per-element rate of the sample, linear: the whole set of {built.n_valid} elements at this '
+                         f'rate takes {built.n_valid / (n / t):.1f} s per step',
         'ms_per_step_sample': t * 1e3,
         'gbps_30B': 30 * n / t / 1e9,
         'oracle_c_openmp': {'value': n / tc, 'unit': 'elements/s', 'cores': O.num_threads()},
@@ -277,12 +304,13 @@ def offload_step_leg(mi_elements, steps=5):
     return out
 
 
-def config1_line(args):
+def config1_line(args, with_cpu: bool = True):
     """Configuration 1: plain fp32 Adam on one flat buffer of 16,777,216 elements (p ~ N(0, 0.02),
     g ~ N(0, 1e-2), m = v = 0 at the start, lr 1e-3, betas (0.9, 0.999), eps 1e-8, no weight decay,
     no loss scale, no stats pass, no low-precision copy) -- the case torch.optim.Adam runs on the
     CPU.  28 B per element: read p, g, m, v, write p, m, v.  The whole state (268 MB) is about the
-    size of the last-level cache, so this line says little about HBM; it is the latency case."""
+    size of the last-level cache, so this line says little about HBM; it is the latency case.
+    The timed steps carry no event records; the launch itself is timed in extra steps afterwards."""
     import elixir_amd as ea
     n = 1 << 24
     gen = torch.Generator(device='cuda')
@@ -292,15 +320,18 @@ def config1_line(args):
     opt = ea.HybridAdam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
     p.grad = g
     step_s, adam_ms = [], []
-    opt.kernel_events = {}
-    for i in range(args.warmup + args.steps):
+    extra = 6
+    for i in range(args.warmup + args.steps + extra):
+        if i == args.warmup + args.steps:
+            opt.kernel_events = {}
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         opt.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        if i >= args.warmup:
+        if args.warmup <= i < args.warmup + args.steps:
             step_s.append(dt)
+        elif i > args.warmup + args.steps:    # the first instrumented step creates the event pair
             ev = opt.kernel_events['adam_step']
             adam_ms.append(ev[0].elapsed_time(ev[1]))
     opt.kernel_events = None
@@ -315,9 +346,10 @@ def config1_line(args):
                  'frac_28B': BYTES_UPDATE * n / t_step / 1e9 / HBM_PEAK_GBPS},
         'roofline': {'kernel': 'adam_step_kernel', 'bound': 'hbm', 'achieved': BYTES_UPDATE * n / t_upd / 1e9,
                      'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': BYTES_UPDATE * n / t_upd / 1e9 / HBM_PEAK_GBPS,
-                     'traffic': None, 'bytes_per_launch': BYTES_UPDATE * n, 'ms_per_launch': t_upd * 1e3},
+                     'traffic': None, 'bytes_per_launch': BYTES_UPDATE * n, 'ms_per_launch': t_upd * 1e3,
+                     'timed_in': f'{extra - 1} extra steps after the timed ones'},
     }
-    if args.cpu_sample > 0:
+    if with_cpu:
         # the reference's own path for this configuration: torch.optim.Adam on CPU tensors, full size
         cp = torch.nn.Parameter(p.detach().cpu())
         copt = torch.optim.Adam([cp], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
@@ -330,8 +362,9 @@ def config1_line(args):
         t = float(np.median(ts[1:]))
         out['cpu_baseline'] = {'value': n / t, 'unit': 'elements/s', 'cores': torch.get_num_threads(), 'kind': 'port',
                                'sample': 'the whole configuration: torch.optim.Adam on CPU fp32 tensors, median of 5 '
-                                         'steps after 1 warm-up', 'ms_per_step_sample': t * 1e3}
-    print(json.dumps(out))
+                                         'steps after 1 warm-up', 'extrapolation': 'none: full size',
+                               'ms_per_step_sample': t * 1e3}
+    return out
 
 
 def velocity_line(args):
@@ -368,7 +401,7 @@ def velocity_line(args):
     velocity = len(step_s) * (n / 1e9) / float(np.sum(step_s))
     t_step, t_upd = float(np.mean(step_s)), float(np.mean(adam_ms)) * 1e-3
     published = 50.0
-    out = {
+    return {
         'metric': 'adam_velocity', 'value': velocity, 'unit': '1e9 elements/s', 'n_gpus': 1, 'steps': args.steps,
         'warmup': args.warmup, 'ms_per_step': t_step * 1e3, 'higher_is_better': True, 'scaling': 'weak',
         'vs_baseline': velocity / published, 'dtype': 'f32', 'data': 'synthetic',
@@ -381,7 +414,162 @@ def velocity_line(args):
                      'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': BYTES_UPDATE * n / t_upd / 1e9 / HBM_PEAK_GBPS,
                      'traffic': None, 'bytes_per_launch': BYTES_UPDATE * n, 'ms_per_launch': t_upd * 1e3},
     }
-    print(json.dumps(out))
+
+
+def chunk_set_line(args, workload: str, device, events_in_timed_steps: bool):
+    """One chunk-set workload (c2, c4, c5) measured end to end; returns the JSON object of its line.
+
+    ``events_in_timed_steps``: bracket the update launch with HIP events in every timed step (three
+    records on the launch stream, about 6 us each: nothing next to 30 ms, 2 % of the GPT-2 step).
+    Otherwise the timed steps run clean and every launch is timed in extra steps afterwards."""
+    from elixir_amd import workloads
+    t_build = time.perf_counter()
+    built = workloads.build(workload, device)
+    t_build = time.perf_counter() - t_build
+    opt = built.optimizer
+    opt.optim.blocks_per_cu = args.blocks_per_cu
+    opt.blocks_per_cu = args.blocks_per_cu
+    opt.graph_step = bool(args.graph)
+    n_valid = built.n_valid
+
+    step_s, upd_ms, stats_ms, adam_ms, refresh_ms = [], [], [], [], []
+    if events_in_timed_steps:
+        opt.optim.kernel_events = {}
+    extra = 4
+    for i in range(args.warmup + args.steps + extra):
+        instrumented = i >= args.warmup + args.steps
+        if instrumented and opt.kernel_events is None:
+            opt.kernel_events = {}
+            if opt.optim.kernel_events is None:
+                opt.optim.kernel_events = {}
+        built.land_gradients()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert opt.last_step_info['found_inf'] is False
+        iev = opt.optim.kernel_events
+        if instrumented:
+            ev = opt.kernel_events
+            upd_ms.append(ev['update'][0].elapsed_time(ev['update'][1]))
+            stats_ms.append(ev['stats'][0].elapsed_time(ev['stats'][1]))
+            if not events_in_timed_steps:
+                adam_ms.append(iev['adam_step'][0].elapsed_time(iev['adam_step'][1]))
+                refresh_ms.append(iev['refresh'][0].elapsed_time(iev['refresh'][1]) if 'refresh' in iev else 0.0)
+        elif i >= args.warmup:
+            step_s.append(dt)
+            if events_in_timed_steps:
+                adam_ms.append(iev['adam_step'][0].elapsed_time(iev['adam_step'][1]))
+                refresh_ms.append(iev['refresh'][0].elapsed_time(iev['refresh'][1]) if 'refresh' in iev else 0.0)
+    opt.kernel_events = None
+    opt.optim.kernel_events = None
+    upd_ms, stats_ms = upd_ms[1:], stats_ms[1:]    # the first instrumented step creates the event pairs
+    if not events_in_timed_steps:
+        adam_ms, refresh_ms = adam_ms[1:], refresh_ms[1:]
+
+    t_step = float(np.mean(step_s))
+    t_pair = float(np.mean(upd_ms)) * 1e-3        # update launch + padding refresh launch + host time between
+    t_upd = float(np.mean(adam_ms)) * 1e-3         # adam_step_kernel alone
+    t_refresh = float(np.mean(refresh_ms)) * 1e-3
+    t_stats = float(np.mean(stats_ms)) * 1e-3      # stats launch + fold-and-decide launch
+    upd_gbps = BYTES_UPDATE * n_valid / t_upd / 1e9
+    plan = next(iter(opt.optim._plans.values())).plan
+    traffic, traffic_source = traffic_fields(built.spec.name)
+    out = {
+        'metric': 'adam_elements_per_sec',
+        'value': n_valid / t_step,
+        'unit': 'elements/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': t_step * 1e3,
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'f32',
+        'data': 'synthetic',
+        'config': {
+            'workload': built.spec.name + ': ' + built.spec.description,
+            'valid_elements': n_valid,
+            'allocated_elements': built.n_alloc,
+            'chunks': len(built.module.param_chunks),
+            'tensors': len(opt.param_to_range),
+            'loss_scale': built.spec.loss_scale,
+            'combined_scale': opt.last_step_info['combined_scale'],
+            'blocks_per_cu': args.blocks_per_cu,
+            'graph_replay': bool(args.graph),
+            'update_rows': len(plan.rows),
+            'padding_in_update_launch': plan.refresh_rows is None and built.n_alloc > n_valid,
+        },
+        'step': {
+            'ms_min': float(np.min(step_s)) * 1e3,
+            'ms_median': float(np.median(step_s)) * 1e3,
+            'gbps_30B': (BYTES_UPDATE + BYTES_STATS) * n_valid / t_step / 1e9,
+            'frac_30B': (BYTES_UPDATE + BYTES_STATS) * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
+            'gbps_touch_once_28B': BYTES_UPDATE * n_valid / t_step / 1e9,
+            'frac_touch_once_28B': BYTES_UPDATE * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
+        },
+        'roofline': {
+            'kernel': 'adam_step_kernel',
+            'bound': 'hbm',
+            'achieved': upd_gbps,
+            'peak': HBM_PEAK_GBPS,
+            'unit': 'GB/s',
+            'frac': upd_gbps / HBM_PEAK_GBPS,
+            'traffic': traffic,
+            'traffic_source': traffic_source,
+            'bytes_per_launch': BYTES_UPDATE * n_valid,
+            'ms_per_launch': t_upd * 1e3,
+            'timed_in': 'every timed step' if events_in_timed_steps else f'{extra - 1} extra steps after the timed ones',
+        },
+        'refresh_kernel': {
+            'what': 'low-precision refresh of the chunk padding left out of the update launch',
+            'ms_per_launch': t_refresh * 1e3,
+            'update_plus_refresh_ms': t_pair * 1e3,
+            'achieved_28B_over_both': BYTES_UPDATE * n_valid / t_pair / 1e9,
+        },
+        'stats_kernel': {
+            'kernel': 'grad_stats_kernel+finish_decide_kernel',
+            'achieved': BYTES_STATS * n_valid / t_stats / 1e9,
+            'unit': 'GB/s',
+            'frac': BYTES_STATS * n_valid / t_stats / 1e9 / HBM_PEAK_GBPS,
+            'ms_per_launch': t_stats * 1e3,
+        },
+        'build_s': t_build,
+    }
+    if args.landing_steps > 0:
+        out['fused_landing'] = fused_landing_leg(built, args.landing_steps)
+    return out, built
+
+
+def summary_of(line):
+    """What the `configs` object keeps of a workload's line."""
+    keep = {'workload': line['config']['workload'], 'valid_elements': line['config']['valid_elements'],
+            'metric': line['metric'], 'value': line['value'], 'unit': line['unit'], 'steps': line['steps'],
+            'ms_per_step': line['ms_per_step'], 'ms_min': line['step']['ms_min'],
+            'roofline_frac_update_launch': line['roofline']['frac'],
+            'update_launch_ms': line['roofline']['ms_per_launch'], 'update_launch_timed_in': line['roofline'].get('timed_in')}
+    for k in ('frac_30B', 'frac_touch_once_28B', 'frac_28B'):
+        if k in line['step']:
+            keep['step_' + k] = line['step'][k]
+    if 'stats_kernel' in line:
+        keep['stats_launch_ms'] = line['stats_kernel']['ms_per_launch']
+        keep['stats_frac'] = line['stats_kernel']['frac']
+    if 'fused_landing' in line:
+        keep['step_after_fused_landing_ms'] = line['fused_landing']['ms_per_step']
+        keep['step_after_fused_landing_frac_28B'] = line['fused_landing']['step_frac_28B']
+    if line.get('vs_baseline') is not None:
+        keep['vs_baseline'] = line['vs_baseline']
+    if 'cpu_baseline' in line:
+        keep['cpu_baseline'] = line['cpu_baseline']
+    return keep
+
+
+def free_device_memory():
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
 
 
 def main():
@@ -393,6 +581,10 @@ def main():
     ap.add_argument('--cpu-sample', type=int, default=256 << 20, help='elements of the CPU baseline sample; 0 skips it')
     ap.add_argument('--blocks-per-cu', type=int, default=0,
                     help='cap on resident update workgroups per compute unit (0 = library default)')
+    ap.add_argument('--graph', action='store_true',
+                    help='replay the launches of a step from a recorded HIP graph (ElixirOptimizer.graph_step)')
+    ap.add_argument('--no-configs', action='store_true',
+                    help='only the headline workload: leave the `configs` object with the other configurations out')
     ap.add_argument('--calibrate-copy', type=float, default=0.0,
                     help='instead of the benchmark, run three plain device copies of this many GiB (a kernel of '
                     'known traffic, to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit')
@@ -430,123 +622,43 @@ def main():
         print(json.dumps({'calibrate_copy_bytes_read': n * 4, 'calibrate_copy_bytes_written': n * 4, 'copies': 3}))
         return
 
-    from elixir_amd import _abi, workloads
+    from elixir_amd import _abi
     _abi.load()
     device = torch.device('cuda', 0)
     torch.cuda.set_device(device)
     if args.workload == 'c1':
-        config1_line(args)
+        print(json.dumps(config1_line(args, with_cpu=args.cpu_sample > 0)))
         return
     if args.workload == 'velocity':
-        velocity_line(args)
+        print(json.dumps(velocity_line(args)))
         return
 
-    t_build = time.perf_counter()
-    built = workloads.build(args.workload, device)
-    t_build = time.perf_counter() - t_build
-    opt = built.optimizer
-    opt.optim.blocks_per_cu = args.blocks_per_cu
-    opt.blocks_per_cu = args.blocks_per_cu
-    n_valid = built.n_valid
-
-    step_s, upd_ms, stats_ms, adam_ms, refresh_ms = [], [], [], [], []
-    # In the timed steps only the update launch is bracketed by events (three records on its stream;
-    # the pairs are created in the first warm-up step and re-recorded afterwards).  The brackets around
-    # the stats pass and around the whole update + refresh cost a few records more and are taken in
-    # three extra steps after the timed ones.
-    opt.optim.kernel_events = {}
-    extra = 3
-    for i in range(args.warmup + args.steps + extra):
-        instrumented = i >= args.warmup + args.steps
-        if instrumented and opt.kernel_events is None:
-            opt.kernel_events = {}
-        built.land_gradients()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        opt.step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        assert opt.last_step_info['found_inf'] is False
-        iev = opt.optim.kernel_events
-        if instrumented:
-            ev = opt.kernel_events
-            upd_ms.append(ev['update'][0].elapsed_time(ev['update'][1]))
-            stats_ms.append(ev['stats'][0].elapsed_time(ev['stats'][1]))
-        elif i >= args.warmup:
-            step_s.append(dt)
-            adam_ms.append(iev['adam_step'][0].elapsed_time(iev['adam_step'][1]))
-            refresh_ms.append(iev['refresh'][0].elapsed_time(iev['refresh'][1]) if 'refresh' in iev else 0.0)
-    opt.kernel_events = None
-    opt.optim.kernel_events = None
-    upd_ms, stats_ms = upd_ms[1:], stats_ms[1:]    # the first instrumented step creates the event pairs
-
-    t_step = float(np.mean(step_s))
-    t_pair = float(np.mean(upd_ms)) * 1e-3        # update launch + padding refresh launch + host time between
-    t_upd = float(np.mean(adam_ms)) * 1e-3         # adam_step_kernel alone
-    t_refresh = float(np.mean(refresh_ms)) * 1e-3
-    t_stats = float(np.mean(stats_ms)) * 1e-3
-    upd_gbps = BYTES_UPDATE * n_valid / t_upd / 1e9
-    out = {
-        'metric': 'adam_elements_per_sec',
-        'value': n_valid / t_step,
-        'unit': 'elements/s',
-        'n_gpus': 1,
-        'steps': args.steps,
-        'warmup': args.warmup,
-        'ms_per_step': t_step * 1e3,
-        'higher_is_better': True,
-        'scaling': 'weak',
-        'vs_baseline': None,
-        'dtype': 'f32',
-        'data': 'synthetic',
-        'config': {
-            'workload': built.spec.name + ': ' + built.spec.description,
-            'valid_elements': n_valid,
-            'allocated_elements': built.n_alloc,
-            'chunks': len(built.module.param_chunks),
-            'tensors': len(opt.param_to_range),
-            'loss_scale': built.spec.loss_scale,
-            'combined_scale': opt.last_step_info['combined_scale'],
-            'blocks_per_cu': args.blocks_per_cu,
-        },
-        'step': {
-            'ms_min': float(np.min(step_s)) * 1e3,
-            'ms_median': float(np.median(step_s)) * 1e3,
-            'gbps_30B': (BYTES_UPDATE + BYTES_STATS) * n_valid / t_step / 1e9,
-            'frac_30B': (BYTES_UPDATE + BYTES_STATS) * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
-            'gbps_touch_once_28B': BYTES_UPDATE * n_valid / t_step / 1e9,
-            'frac_touch_once_28B': BYTES_UPDATE * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
-        },
-        'roofline': {
-            'kernel': 'adam_step_kernel',
-            'bound': 'hbm',
-            'achieved': upd_gbps,
-            'peak': HBM_PEAK_GBPS,
-            'unit': 'GB/s',
-            'frac': upd_gbps / HBM_PEAK_GBPS,
-            'traffic': MEASURED_TRAFFIC_BYTES.get(built.spec.name),
-            'bytes_per_launch': BYTES_UPDATE * n_valid,
-            'ms_per_launch': t_upd * 1e3,
-        },
-        'refresh_kernel': {
-            'what': 'low-precision refresh of the chunk padding left out of the update launch',
-            'ms_per_launch': t_refresh * 1e3,
-            'update_plus_refresh_ms': t_pair * 1e3,
-            'achieved_28B_over_both': BYTES_UPDATE * n_valid / t_pair / 1e9,
-        },
-        'stats_kernel': {
-            'kernel': 'grad_stats_kernel+stats_finish_kernel',
-            'achieved': BYTES_STATS * n_valid / t_stats / 1e9,
-            'unit': 'GB/s',
-            'frac': BYTES_STATS * n_valid / t_stats / 1e9 / HBM_PEAK_GBPS,
-            'ms_per_launch': t_stats * 1e3,
-        },
-        'build_s': t_build,
-    }
-    if args.landing_steps > 0:
-        out['fused_landing'] = fused_landing_leg(built, args.landing_steps)
+    out, built = chunk_set_line(args, args.workload, device, events_in_timed_steps=args.workload == 'c5')
     if args.cpu_sample > 0:
         out['cpu_baseline'] = cpu_baseline(built, args.cpu_sample)
+    del built
+    free_device_memory()
+
+    if args.workload == 'c5' and not args.no_configs:
+        # the other configurations in the same run (fewer steps each: a few hundred milliseconds of GPU time)
+        configs = {}
+        small = argparse.Namespace(**vars(args))
+        small.landing_steps = min(args.landing_steps, 3)
+        for name, steps in (('c4', 20), ('c2', 50)):
+            small.steps, small.warmup = steps, 5
+            line, b = chunk_set_line(small, name, device, events_in_timed_steps=False)
+            del b
+            free_device_memory()
+            configs[name] = summary_of(line)
+        small.steps, small.warmup = 50, 5
+        configs['c1'] = summary_of(config1_line(small, with_cpu=args.cpu_sample > 0))
+        free_device_memory()
+        small.steps, small.warmup = 10, 2
+        configs['velocity'] = summary_of(velocity_line(small))
+        free_device_memory()
+        configs['c3'] = 'the overflow path on the c2 layout is a correctness gate, not a throughput figure: ' \
+                        'tests/test_gpu_configs.py'
+        out['configs'] = configs
     print(json.dumps(out))
 
 

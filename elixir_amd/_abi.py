@@ -42,7 +42,7 @@ EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 
            'elx_decide', 'elx_adam_step_gated_mt', 'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_writeback',
            'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems',
            'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
-           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers')
+           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers')
 
 
 class ElxError(RuntimeError):
@@ -73,7 +73,7 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
                  'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
-           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers'):
+           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -85,6 +85,8 @@ def load() -> ctypes.CDLL:
     L.elx_grad_partials_mt.argtypes = [vp, u32, cint, u32, vp, cint, vp]
     L.elx_finish_decide.restype = cint
     L.elx_finish_decide.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp]
+    L.elx_put_hypers.restype = cint
+    L.elx_put_hypers.argtypes = [vp, u32, vp, vp]
     L.elx_grad_stats_mt_static.restype = cint
     L.elx_grad_stats_mt_static.argtypes = [vp, u32, cint, u32, vp, cint, vp]
     L.elx_adam_step_mt.restype = cint
@@ -191,6 +193,12 @@ def finish_decide(d_partials: int, n_chunks: int, blocks_per_chunk: int, d_stats
     check('elx_finish_decide',
           load().elx_finish_decide(d_partials, n_chunks, blocks_per_chunk, d_stats, ctl, d_hypers, max_hypers, d_decision,
                                    report or None, d_counter, stream))
+
+
+def put_hypers(hyper_host: np.ndarray, d_hypers: int, stream: int) -> None:
+    """Host hyper records -> device table, through the arguments of a tiny launch on ``stream``."""
+    assert hyper_host.dtype == HYPER_DTYPE
+    check('elx_put_hypers', load().elx_put_hypers(_np_ptr(hyper_host), len(hyper_host), d_hypers, stream))
 
 
 def max_ctl_hypers() -> int:

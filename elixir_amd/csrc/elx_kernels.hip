@@ -35,6 +35,7 @@
 // -ffp-contract=off.  The op order is torch.optim.Adam's single-tensor path
 // (torch/optim/adam.py:414-419, 457, 476, 528-545) with the fused forms its CPU kernels use.
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include <atomic>
@@ -998,6 +999,23 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Hyper records from the kernel arguments into the device table of an update launch: a handful of
+// records reach the device inside the launch packet itself, without a staging buffer and a copy to
+// order and to keep alive.
+constexpr uint32_t kMaxArgHypers = 32;
+struct HyperPack {
+    ElxHyper h[kMaxArgHypers];
+};
+
+__global__ __launch_bounds__(kWave) void put_hypers_kernel(HyperPack pack, uint32_t n_words, uint32_t *__restrict__ dst) {
+    // the pack is read where it lies, in the argument segment (indexing a by-value aggregate with the lane
+    // number would copy it to private memory first)
+    typedef const uint32_t __attribute__((address_space(4))) *kernarg_words;
+    kernarg_words src = (kernarg_words)__builtin_amdgcn_kernarg_segment_ptr();
+    for (uint32_t i = threadIdx.x; i < n_words; i += kWave) dst[i] = src[i];
+}
+static_assert(offsetof(HyperPack, h) == 0, "the records start at offset 0 of the argument segment");
+
 // ---------------------------------------------------------------------------------------------
 // host side of the ABI
 // ---------------------------------------------------------------------------------------------
@@ -1220,6 +1238,21 @@ int elx_finish_decide(const ElxStats *d_partials, uint32_t n_chunks, uint32_t bl
     hipLaunchKernelGGL(finish_decide_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, (hipStream_t)stream, d_partials,
                        blocks_per_chunk, d_stats, n_chunks, ctl, d_hypers, max_hypers, d_decision, report, d_counter);
     return (int)hipGetLastError();
+}
+
+int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream) {
+    if (!h_hypers || !d_hypers) return ELX_E_NULL;
+    if (n_hypers == 0) return ELX_E_SIZE;
+    if ((uintptr_t)d_hypers & 3u) return ELX_E_ALIGN;
+    for (uint32_t at = 0; at < n_hypers; at += kMaxArgHypers) {
+        const uint32_t n = n_hypers - at < kMaxArgHypers ? n_hypers - at : kMaxArgHypers;
+        HyperPack pack = {};
+        __builtin_memcpy(pack.h, h_hypers + at, n * sizeof(ElxHyper));
+        hipLaunchKernelGGL(put_hypers_kernel, dim3(1), dim3(kWave), 0, (hipStream_t)stream, pack,
+                           n * (uint32_t)(sizeof(ElxHyper) / 4u), reinterpret_cast<uint32_t *>(d_hypers + at));
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    }
+    return 0;
 }
 
 uint32_t elx_sizeof_step_ctl(void) { return (uint32_t)sizeof(ElxStepCtl); }

@@ -21,6 +21,7 @@ from typing import Dict, List, Optional, Tuple
 
 import numpy as np
 import torch
+from torch.optim import optimizer as _torch_optimizer
 
 from . import _abi
 from .chunk import gpu_device, Chunk, DeviceTable, dtype_code
@@ -73,35 +74,18 @@ class _CachedTable:
         return self.table
 
 
-class _HyperUploader:
-    """Per-step upload of the (tiny) hyper-parameter table without blocking the host: two pinned
-    staging buffers used in turn and an asynchronous copy on the launch stream.  A staging buffer
-    is rewritten two steps after its copy was enqueued; every step waits for the device at least
-    once in between (the readback of the gradient flags), so the copy has long completed."""
+class _HyperTable:
+    """The device table of the hyper records of a step.  The records change every step (bias
+    corrections); they reach the device in the arguments of a one-wavefront launch on the launch stream
+    (``elx_put_hypers``): nothing to stage, nothing to wait for, and the host array is free at once."""
 
     def __init__(self):
-        self.staging: List[torch.Tensor] = []
-        self.copied: List[Optional[torch.cuda.Event]] = [None, None]
         self.dev: Optional[torch.Tensor] = None
-        self.turn = 0
 
-    def upload(self, host: np.ndarray, device: torch.device) -> int:
-        nbytes = host.nbytes
-        if self.dev is None or self.dev.device != device or self.dev.numel() < nbytes:
-            cap = max(4096, nbytes)
-            self.dev = torch.empty(cap, dtype=torch.uint8, device=device)
-            self.staging = [torch.empty(cap, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
-            self.copied = [None, None]
-        turn = self.turn
-        stage = self.staging[turn]
-        self.turn ^= 1
-        if self.copied[turn] is None:
-            self.copied[turn] = torch.cuda.Event()    # created once per buffer, recorded again at every use
-        else:
-            self.copied[turn].synchronize()    # normally long past: the copy out of this buffer has run
-        stage[:nbytes].numpy()[:] = host.view(np.uint8).reshape(-1)
-        self.dev[:nbytes].copy_(stage[:nbytes], non_blocking=True)
-        self.copied[turn].record(torch.cuda.current_stream(device))
+    def put(self, host: np.ndarray, device: torch.device) -> int:
+        if self.dev is None or self.dev.device != device or self.dev.numel() < host.nbytes:
+            self.dev = torch.empty(max(4096, host.nbytes), dtype=torch.uint8, device=device)
+        _abi.put_hypers(host, self.dev.data_ptr(), torch.cuda.current_stream(device).cuda_stream)
         return self.dev.data_ptr()
 
 
@@ -212,10 +196,11 @@ class HybridAdam(torch.optim.Optimizer):
         self.blocks_per_cu = 0    # cap on resident update workgroups per compute unit; 0: library default
         self._binding: Optional[ChunkBinding] = None
         self._plans: Dict = {}                      # plan key -> _DevicePlan
-        self._hyper_uploader = _HyperUploader()
+        self._hyper_table_dev = _HyperTable()
         self._prepared: Optional[_Prepared] = None
         self._launched: Optional[_Prepared] = None   # launched with defer_commit, not yet committed or aborted
         self._bound_entries = None                  # cached walk over the bound fake parameters
+        self._standalone_cache = None               # cached walk over standalone parameters and their gradients
         # when set to a dict, step() records (begin, end) torch.cuda.Event pairs under 'adam_step' and 'refresh'
         self.kernel_events = None
 
@@ -277,7 +262,7 @@ class HybridAdam(torch.optim.Optimizer):
             if prep is not None:
                 prep.sig = sig
         if prep is not None and upload and not prep.d_hypers:
-            prep.d_hypers = self._hyper_uploader.upload(prep.hyper_host, prep.device)
+            prep.d_hypers = self._hyper_table_dev.put(prep.hyper_host, prep.device)
 
     def adopt_prepared(self) -> None:
         """The prepared step counts as launched without a launch from here: its launches were recorded
@@ -303,17 +288,36 @@ class HybridAdam(torch.optim.Optimizer):
             for (lr, b1, b2, eps, wd, step, bc) in hypers.keys()
         ])
 
-    @torch.no_grad()
     def step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
         """``gated``: the unscale parameters and the skip flag are read on the device from the gate
         words of the prepared hyper table, where ``elx_decide`` has put them (``div_scale`` is then
         ignored).  ``defer_commit``: launch only; the caller finishes with ``commit_step()`` once it
-        knows that the step happened, or ``abort_step()`` when the device decided to skip."""
-        return self.launch_step(closure, div_scale, gated=gated, defer_commit=defer_commit)
+        knows that the step happened, or ``abort_step()`` when the device decided to skip.
+
+        torch wraps every optimizer's ``step`` in a profiler scope and its hook dispatch, tens of
+        microseconds during which the device waits; this class opts out of that wrapper (the ``hooked``
+        mark below) and runs registered step hooks itself, in torch's order."""
+        pre = list(_torch_optimizer._global_optimizer_pre_hooks.values()) + list(self._optimizer_step_pre_hooks.values())
+        post = list(self._optimizer_step_post_hooks.values()) + list(_torch_optimizer._global_optimizer_post_hooks.values())
+        if not pre and not post:
+            return self.launch_step(closure, div_scale, gated=gated, defer_commit=defer_commit)
+        args, kwargs = (closure, div_scale), dict(gated=gated, defer_commit=defer_commit)
+        for hook in pre:
+            result = hook(self, args, kwargs)
+            if result is not None:
+                if not (isinstance(result, tuple) and len(result) == 2):
+                    raise RuntimeError(f'{hook} must return None or a tuple of (new_args, new_kwargs), but got {result}.')
+                args, kwargs = result
+        out = self.launch_step(*args, **kwargs)
+        for hook in post:
+            hook(self, args, kwargs)
+        return out
+
+    step.hooked = True    # torch.optim.Optimizer leaves a step marked like this unwrapped
 
     def launch_step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
-        """``step`` without the profiler scope and hook dispatch torch wraps around every optimizer's
-        ``step`` (tens of microseconds that the device would wait for)."""
+        """The launches of one step (``step`` without the hook dispatch).  Nothing here builds an autograd
+        graph, so no ``no_grad`` scope is entered either."""
         loss = None
         if closure is not None:
             with torch.enable_grad():
@@ -325,7 +329,7 @@ class HybridAdam(torch.optim.Optimizer):
             return loss
 
         if not prep.d_hypers:
-            prep.d_hypers = self._hyper_uploader.upload(prep.hyper_host, prep.device)
+            prep.d_hypers = self._hyper_table_dev.put(prep.hyper_host, prep.device)
         plan = prep.dplan.plan
         stream = torch.cuda.current_stream(prep.device).cuda_stream
         events = self.kernel_events
@@ -434,6 +438,7 @@ class HybridAdam(torch.optim.Optimizer):
             step = saved.get('step', 0)
             state['step'] = int(step.item()) if torch.is_tensor(step) else int(step)
         self._prepared = None
+        self._standalone_cache = None
 
     def _walk_bound(self):
         """(state dict, group index, chunk index, begin, end) per bound fake parameter, in group order."""
@@ -514,15 +519,31 @@ class HybridAdam(torch.optim.Optimizer):
 
     # ---- standalone, on ordinary parameters
 
-    def _prepare_standalone(self, hypers: Dict) -> Optional[_Prepared]:
-        items = []
+    def _standalone_items(self):
+        """(items, gradient dtype, device) of the parameters that carry a gradient: per parameter its state
+        dict, its group index and (gradient, parameter, exp_avg, exp_avg_sq addresses, element count).  The
+        walk with its checks is repeated only when a parameter, a gradient buffer or the group layout has
+        changed since the last step (every buffer is watched by address and dtype)."""
+        cache = self._standalone_cache
+        if cache is not None:
+            watch, layout, result = cache
+            if layout == tuple(len(g['params']) for g in self.param_groups):
+                for p, p_ptr, g_ptr, g_dtype in watch:
+                    g = p.grad
+                    if g is None:
+                        if g_ptr is not None:
+                            break
+                    elif g_ptr is None or g.data_ptr() != g_ptr or g.dtype != g_dtype or p.data_ptr() != p_ptr:
+                        break
+                else:
+                    return result
+        items, watch = [], []
         grad_dtype = None
         device = None
-        for group in self.param_groups:
+        for gi, group in enumerate(self.param_groups):
             for p in group['params']:
-                if p.grad is None:
-                    continue
-                if p.numel() == 0:
+                if p.grad is None or p.numel() == 0:
+                    watch.append((p, p.data_ptr(), None, None))
                     continue
                 if p.device.type != 'cuda':
                     raise RuntimeError('HybridAdam runs on the GPU: parameters must live in device memory')
@@ -540,17 +561,32 @@ class HybridAdam(torch.optim.Optimizer):
                     state['step'] = 0
                     state['exp_avg'] = torch.zeros_like(p, memory_format=torch.preserve_format)
                     state['exp_avg_sq'] = torch.zeros_like(p, memory_format=torch.preserve_format)
-                n = p.numel()
-                items.append((state, (p.grad.data_ptr(), 0, p.data.data_ptr(), state['exp_avg'].data_ptr(),
-                                      state['exp_avg_sq'].data_ptr(), n, self._hyper_index(hypers, group, state['step'] + 1))))
+                watch.append((p, p.data_ptr(), p.grad.data_ptr(), p.grad.dtype))
+                items.append((state, gi, (p.grad.data_ptr(), p.data.data_ptr(), state['exp_avg'].data_ptr(),
+                                          state['exp_avg_sq'].data_ptr(), p.numel())))
+        result = (items, grad_dtype, device)
+        self._standalone_cache = (watch, tuple(len(g['params']) for g in self.param_groups), result)
+        return result
+
+    def _prepare_standalone(self, hypers: Dict) -> Optional[_Prepared]:
+        items, grad_dtype, device = self._standalone_items()
         if not items:
             return None
+        groups = self.param_groups
+        seen: Dict = {}    # (group, step) -> hyper index
+        idx_of = []
+        for state, gi, _ in items:
+            k = (gi, state['step'])
+            h = seen.get(k)
+            if h is None:
+                h = seen[k] = self._hyper_index(hypers, groups[gi], k[1] + 1)
+            idx_of.append(h)
         grad_code = dtype_code(grad_dtype)
-        key = ('standalone', grad_code, tuple(it[1] for it in items))
+        key = ('standalone', grad_code, tuple(it[2] for it in items), tuple(idx_of))
 
         def buffers():
             return [FlatBuffer(grad=g, lowp_out=0, master=p, m=m, v=v, n_alloc=n, n_valid=n, segs=[(0, n, h)])
-                    for _, (g, _, p, m, v, n, h) in items]
+                    for (_, _, (g, p, m, v, n)), h in zip(items, idx_of)]
 
         dplan = self._device_plan(key, buffers, grad_dtype, grad_code, _abi.ELX_NONE, len(hypers), device)
         return _Prepared(dplan, self._hyper_table(hypers), grad_code, _abi.ELX_NONE, device, [it[0] for it in items])

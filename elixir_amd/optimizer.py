@@ -121,8 +121,7 @@ class _DeviceStep:
         head = self._ctl_head
         at = head.itemsize
         self._ctl_bytes[at:at + hyper_host.nbytes] = hyper_host.view(np.uint8).reshape(-1)
-        head['loss_scale'], head['max_norm'], head['clipping'], head['n_hypers'] = loss_scale, max_norm, int(clipping), n
-        head['seq'] = self.seq
+        head[0] = (loss_scale, max_norm, int(clipping), n, self.seq)
         return self.seq
 
     def partials_buffer(self, records: int) -> int:
@@ -532,8 +531,9 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 rows[i]['grad'] = c.shard.data_ptr()
                 rows[i]['n_alloc'] = c.shard_size
                 rows[i]['n_valid'] = c.n_valid
-            self._all_stats_table = ((ids, ptrs), rows, DeviceTable(rows, device))
-        return self._all_stats_table[1], self._all_stats_table[2]
+            self._all_stats_table = ((ids, ptrs), DeviceTable(rows, device),
+                                     stats_launch_blocks(int(rows['n_valid'].max())), bool(np.all(rows['grad'] % 16 == 0)))
+        return self._all_stats_table[1:]
 
     def _step_on_device(self, source) -> bool:
         """The step without a wait between the flags and the update: the decisions of
@@ -555,11 +555,9 @@ class ElixirOptimizer(torch.optim.Optimizer):
         main = torch.cuda.current_stream(prep.device)
         kind, first_slot = source
         if kind == 'launch':
-            rows, table = self._all_chunks_stats_table(prep.device)
-            bpc = stats_launch_blocks(int(rows['n_valid'].max()))
+            table, bpc, aligned = self._all_chunks_stats_table(prep.device)
             partials = eng.partials_buffer(n * bpc)
-            stats_args = (table.ptr, n, dtype_code(chunks[0].chunk_dtype), bpc, partials,
-                          not bool(np.all(rows['grad'] % 16 == 0)))
+            stats_args = (table.ptr, n, dtype_code(chunks[0].chunk_dtype), bpc, partials, not aligned)
             keep = (table, eng.partials)
         else:
             arena = StatsArena.get(chunks[0].shard_device)

@@ -279,6 +279,16 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
                      uint32_t flags, uint32_t blocks_per_cu, void *stream);
 
 /*
+ * Writes n_hypers records from HOST memory into the device table d_hypers, ordered on `stream`: the
+ * records travel in the arguments of a one-wavefront launch (32 per launch), so there is no staging
+ * buffer to keep alive and no host-to-device copy; h_hypers may be reused as soon as the call returns.
+ * This is how a host-decided or standalone step gets its per-step scalars (bias corrections, learning
+ * rate) to the device: the `lr`, `betas`, `step` ... arguments of the reference's
+ * fused_optim.multi_tensor_adam call (optimizer.py:216 -> HybridAdam.step).
+ */
+int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream);
+
+/*
  * The host decisions of optimizer.py:137-183 taken on the device, so that the update can be enqueued
  * without waiting for the flags to reach the host: one thread reads the n_chunks records of a stats or
  * landing launch (in the order given), ORs the overflow flags and, with `clipping`, forms the global
