@@ -842,6 +842,9 @@ __device__ __forceinline__ bool exact_reciprocal_dev(float s) {
 // norm exceeds max_norm).  Per chunk the squared norm passes through an fp32 norm
 // (chunk.py:218-221), the sum over chunks through an fp32 buffer (optimizer.py:158-162).  The
 // result goes into *out and into the gate words of every hyper record.
+__device__ __forceinline__ ElxDecision finish_decision(uint32_t found, double norm_sqr, double loss_scale, double max_norm,
+                                                       int clipping);
+
 // `stats` may have been written by other workgroups of the same launch: read through agent-scope loads.
 __device__ __forceinline__ ElxDecision decide_from_stats(const ElxStats *stats, uint32_t n, double loss_scale,
                                                          double max_norm, int clipping) {
@@ -854,6 +857,11 @@ __device__ __forceinline__ ElxDecision decide_from_stats(const ElxStats *stats, 
         const float nrm = (float)sqrt(__builtin_bit_cast(double, bits));
         norm_sqr += (double)nrm * (double)nrm;
     }
+    return finish_decision(found, norm_sqr, loss_scale, max_norm, clipping);
+}
+
+__device__ __forceinline__ ElxDecision finish_decision(uint32_t found, double norm_sqr, double loss_scale, double max_norm,
+                                                       int clipping) {
     ElxDecision d;
     d.skip = found ? 1u : 0u;
     d.total_norm = 0.0;
@@ -907,10 +915,29 @@ __global__ void decide_kernel(const ElxStats *__restrict__ stats, uint32_t n, do
 // follows is still running.
 constexpr uint32_t kMaxCtlHypers = 64;
 constexpr uint32_t kCtlWords = (uint32_t)(sizeof(ElxStepCtl) + kMaxCtlHypers * sizeof(ElxHyper)) / 4u;
+constexpr uint32_t kCtlEarlyHypers = 4;    // records fetched with the header, before anyone knows how many there are
+static_assert((sizeof(ElxStepCtl) + kCtlEarlyHypers * sizeof(ElxHyper)) / 4u <= kStatsThreads, "one early load per thread");
+constexpr uint32_t kDecideChunksInLds = 1024;    // per-chunk records staged in LDS for the decision loop
 
 template <typename T>
 __device__ __forceinline__ void store_system(T *p, T v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// The decision arithmetic of decide_from_stats over records staged in LDS.
+__device__ __forceinline__ void accumulate_decision(double sumsq, uint32_t overflow, uint32_t &found, double &norm_sqr) {
+    found |= overflow;
+    const float nrm = (float)sqrt(sumsq);
+    norm_sqr += (double)nrm * (double)nrm;
+}
+
+__device__ __forceinline__ double load_sumsq_agent(const ElxStats *r) {
+    return __builtin_bit_cast(double, __hip_atomic_load(reinterpret_cast<const uint64_t *>(&r->sumsq), __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT));
+}
+
+__device__ __forceinline__ uint32_t load_overflow_agent(const ElxStats *r) {
+    return __hip_atomic_load(&r->overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxStats *__restrict__ partials, uint32_t bpc,
@@ -921,6 +948,16 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
     __shared__ uint32_t s_last;
     __shared__ __align__(16) uint32_t s_ctl[kCtlWords];
     __shared__ ElxDecision s_decision;
+    __shared__ ElxStats s_stats[kDecideChunksInLds];
+    // Every workgroup asks for the head of the control block at once (it may sit in host memory, a long
+    // way off): the answer travels while the partials are folded, and the workgroup that ends up deciding
+    // has it at hand.  System-scope loads: the host rewrites the block between launches.
+    // Never beyond the max_hypers records the caller vouches for behind the header.
+    const uint32_t *cw = reinterpret_cast<const uint32_t *>(ctl);
+    const uint32_t early_words =
+        (uint32_t)(sizeof(ElxStepCtl) + (max_hypers < kCtlEarlyHypers ? max_hypers : kCtlEarlyHypers) * sizeof(ElxHyper)) / 4u;
+    uint32_t early = 0;
+    if (threadIdx.x < early_words) early = __hip_atomic_load(cw + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     {
         const ElxStats *row = partials + (uint64_t)blockIdx.x * bpc;
         double sum = 0.0;
@@ -940,24 +977,35 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
             s_last = done == n_chunks - 1 ? 1u : 0u;
         }
     }
+    if (threadIdx.x < early_words) s_ctl[threadIdx.x] = early;
     __syncthreads();
     if (!s_last) return;
 
-    // ---- the last workgroup: control block -> LDS (system-scope loads: it may live in host memory)
-    const uint32_t *cw = reinterpret_cast<const uint32_t *>(ctl);
-    for (uint32_t i = threadIdx.x; i < sizeof(ElxStepCtl) / 4u; i += kStatsThreads)
-        s_ctl[i] = __hip_atomic_load(cw + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __syncthreads();
+    // ---- the last workgroup decides
     const ElxStepCtl *c = reinterpret_cast<const ElxStepCtl *>(s_ctl);
     const uint32_t cap = max_hypers < kMaxCtlHypers ? max_hypers : kMaxCtlHypers;
     const bool valid = c->loss_scale > 0.0 && (!c->clipping || c->max_norm > 0.0) && c->n_hypers <= cap;
     const uint32_t n_hypers = valid ? c->n_hypers : 0u;
-    for (uint32_t i = sizeof(ElxStepCtl) / 4u + threadIdx.x; i < (sizeof(ElxStepCtl) + n_hypers * sizeof(ElxHyper)) / 4u;
+    // the hyper records behind the ones that came with the header, and every chunk's record, side by side
+    for (uint32_t i = early_words + threadIdx.x; i < (sizeof(ElxStepCtl) + n_hypers * sizeof(ElxHyper)) / 4u;
          i += kStatsThreads)
         s_ctl[i] = __hip_atomic_load(cw + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    const uint32_t staged = n_chunks < kDecideChunksInLds ? n_chunks : kDecideChunksInLds;
+    for (uint32_t i = threadIdx.x; i < staged; i += kStatsThreads) {
+        s_stats[i].sumsq = load_sumsq_agent(stats + i);
+        s_stats[i].overflow = load_overflow_agent(stats + i);
+        s_stats[i].reserved = 0;
+    }
+    __syncthreads();
     if (threadIdx.x == 0) {
-        ElxDecision d = decide_from_stats(stats, n_chunks, valid ? c->loss_scale : 1.0, valid ? c->max_norm : 1.0,
-                                          valid ? (int)c->clipping : 0);
+        // decide_from_stats, in the same order: over the staged records, then over whatever did not fit
+        uint32_t found = 0;
+        double norm_sqr = 0.0;
+        for (uint32_t i = 0; i < staged; ++i) accumulate_decision(s_stats[i].sumsq, s_stats[i].overflow, found, norm_sqr);
+        for (uint32_t i = staged; i < n_chunks; ++i)
+            accumulate_decision(load_sumsq_agent(stats + i), load_overflow_agent(stats + i), found, norm_sqr);
+        ElxDecision d = finish_decision(found, norm_sqr, valid ? c->loss_scale : 1.0, valid ? c->max_norm : 1.0,
+                                        valid ? (int)c->clipping : 0);
         if (!valid) d.skip = 1u;    // an unusable control block: nothing is updated, and the report says why
         s_decision = d;
         *out = d;
@@ -966,14 +1014,20 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
     const ElxDecision d = s_decision;
     // the hyper table of the update launch: the step's records with the gate words of this decision.  When
     // the control block is unusable every record the table can hold gets the skip gate.
-    const ElxHyper *src = reinterpret_cast<const ElxHyper *>(s_ctl + sizeof(ElxStepCtl) / 4u);
-    for (uint32_t i = threadIdx.x; i < (valid ? n_hypers : max_hypers); i += kStatsThreads) {
-        ElxHyper h = {};
-        if (valid) h = src[i];
-        h.gate_div_scale = d.div_scale;
-        h.gate_inv_scale = d.inv_scale;
-        h.gate = d.mode | (d.skip << 8);
-        hypers[i] = h;
+    // (word by word: nine words of the step's record, or zeros, then the three gate words)
+    constexpr uint32_t kHyperWords = sizeof(ElxHyper) / 4u, kGateWord = offsetof(ElxHyper, gate_div_scale) / 4u;
+    static_assert(kHyperWords == kGateWord + 3 && offsetof(ElxHyper, gate) / 4u == kGateWord + 2, "gate words come last");
+    const uint32_t *src = s_ctl + sizeof(ElxStepCtl) / 4u;
+    uint32_t *dst = reinterpret_cast<uint32_t *>(hypers);
+    const uint32_t gate_words[3] = {__builtin_bit_cast(uint32_t, d.div_scale), __builtin_bit_cast(uint32_t, d.inv_scale),
+                                    d.mode | (d.skip << 8)};
+    for (uint32_t i = threadIdx.x; i < (valid ? n_hypers : max_hypers) * kHyperWords; i += kStatsThreads) {
+        const uint32_t word = i % kHyperWords;
+        uint32_t value = valid ? src[i] : 0u;
+        if (word == kGateWord) value = gate_words[0];
+        if (word == kGateWord + 1) value = gate_words[1];
+        if (word == kGateWord + 2) value = gate_words[2];
+        dst[i] = value;
     }
     if (report) {
         const uint32_t *dw = reinterpret_cast<const uint32_t *>(&s_decision);
@@ -981,10 +1035,10 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
         for (uint32_t i = threadIdx.x; i < sizeof(ElxDecision) / 4u; i += kStatsThreads) store_system(rw + i, dw[i]);
         ElxStats *rs = reinterpret_cast<ElxStats *>(report + 1);
         for (uint32_t i = threadIdx.x; i < n_chunks; i += kStatsThreads) {
-            const uint64_t bits = __hip_atomic_load(reinterpret_cast<const uint64_t *>(&stats[i].sumsq), __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-            store_system(reinterpret_cast<uint64_t *>(&rs[i].sumsq), bits);
-            store_system(&rs[i].overflow, __hip_atomic_load(&stats[i].overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            const double sumsq = i < staged ? s_stats[i].sumsq : load_sumsq_agent(stats + i);
+            const uint32_t overflow = i < staged ? s_stats[i].overflow : load_overflow_agent(stats + i);
+            store_system(reinterpret_cast<uint64_t *>(&rs[i].sumsq), __builtin_bit_cast(uint64_t, sumsq));
+            store_system(&rs[i].overflow, overflow);
             store_system(&rs[i].reserved, 0u);
         }
         if (threadIdx.x == 0) {

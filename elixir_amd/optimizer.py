@@ -543,34 +543,43 @@ class ElixirOptimizer(torch.optim.Optimizer):
         host memory while the update runs, for the host's bookkeeping (scaler, step counts, chunk flags).
         Returns False when nothing was prepared to launch this way."""
         inner = self.optim
-        inner.prepare_step(upload=False)
-        prep = inner._prepared
-        if prep is None or prep.dplan.rows is None or len(prep.hyper_host) > _abi.max_ctl_hypers():
-            return False
         chunks = self._param_chunk_list
         n = len(chunks)
+        device = self._binding.launch_device()
         eng = self._device_step
-        if eng is None or eng.device != prep.device or eng.n_chunks != n:
-            eng = self._device_step = _DeviceStep(prep.device, n)
-        main = torch.cuda.current_stream(prep.device)
+        if eng is None or eng.device != device or eng.n_chunks != n:
+            eng = self._device_step = _DeviceStep(device, n)
+        main = torch.cuda.current_stream(device)
         kind, first_slot = source
+        early = False
         if kind == 'launch':
-            table, bpc, aligned = self._all_chunks_stats_table(prep.device)
+            table, bpc, aligned = self._all_chunks_stats_table(device)
             partials = eng.partials_buffer(n * bpc)
             stats_args = (table.ptr, n, dtype_code(chunks[0].chunk_dtype), bpc, partials, not aligned)
             keep = (table, eng.partials)
+            if not self.graph_step and self.kernel_events is None:
+                # the stats launch needs nothing of what follows: it goes out first, and the host prepares
+                # the rest of the step (tables, control block) while the device reads the gradients
+                _abi.grad_partials_mt(*stats_args, main.cuda_stream)
+                early = True
         else:
             arena = StatsArena.get(chunks[0].shard_device)
             for event in {c._stats_event for c in chunks if c._stats_event is not None}:
                 main.wait_event(event)    # the landings may have run on another stream
             bpc, partials, stats_args, keep = 1, arena.ptr(first_slot), None, (arena, )
+        inner.prepare_step(upload=False)
+        prep = inner._prepared
+        if prep is None or prep.dplan.rows is None or len(prep.hyper_host) > _abi.max_ctl_hypers():
+            return False    # (a stats launch that went out early is then simply repeated by the host-decided step)
+        assert prep.device == device
+        # the control block is complete before the launch that reads it is issued
         seq = eng.write_ctl(float(self.loss_scale), float(self.max_norm), self.clipping_flag, prep.hyper_host)
         prep.d_hypers = eng.d_hypers
 
         def enqueue():
-            stream = torch.cuda.current_stream(prep.device).cuda_stream
+            stream = torch.cuda.current_stream(device).cuda_stream
             with self._timed('stats' if stats_args is not None else 'decide'):
-                if stats_args is not None:
+                if stats_args is not None and not early:
                     _abi.grad_partials_mt(*stats_args, stream)
                 _abi.finish_decide(partials, n, bpc, eng.d_stats, eng.ctl.data_ptr(), eng.d_hypers, eng.max_hypers,
                                    eng.d_decision, eng.report.data_ptr(), eng.d_counter, stream)

@@ -220,7 +220,9 @@ int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_d
  * the ctl->n_hypers records behind *ctl are copied to d_hypers with their gate words filled in (the table
  * elx_adam_step_gated_mt reads next on the same stream), *d_decision is written and, when `report` is not
  * NULL, so is the report (see ElxStepReport; room for n_chunks ElxStats records behind the header).
- *   max_hypers  capacity of d_hypers in records, at most elx_max_ctl_hypers()
+ *   max_hypers  capacity of d_hypers in records, at most elx_max_ctl_hypers(); *ctl must be readable for
+ *               sizeof(ElxStepCtl) + max_hypers * sizeof(ElxHyper) bytes (the kernel fetches the first
+ *               records together with the header, before it knows n_hypers)
  *   d_counter   one uint32 of device memory, zero before the first call; the launch leaves it zero
  * An unusable control block (loss_scale <= 0, n_hypers > max_hypers ...) cannot be refused by the host
  * (it may be device memory): the kernel then sets the skip gate in all max_hypers records, so that the
