@@ -526,6 +526,9 @@ class ElixirOptimizer(torch.optim.Optimizer):
         ids = tuple(c.chunk_id for c in chunks)
         ptrs = tuple(c.shard.data_ptr() for c in chunks)
         if self._all_stats_table is None or self._all_stats_table[0] != (ids, ptrs):
+            # checked once per set of buffers, BEFORE anything is launched on them: a shard in pageable host
+            # memory is refused here (a launch over it would fault the device)
+            kernel_device(c.shard for c in chunks)
             rows = np.zeros(len(chunks), dtype=_abi.CHUNK_DTYPE)
             for i, c in enumerate(chunks):
                 rows[i]['grad'] = c.shard.data_ptr()

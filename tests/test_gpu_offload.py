@@ -174,8 +174,25 @@ def test_pageable_host_shards_are_refused():
     inner = ea.HybridAdam(list(module.parameters()), lr=1e-3)
     opt = ea.ElixirOptimizer(module, inner, initial_scale=2.0)
     opt.mark_gradients_scaled()
-    with pytest.raises(RuntimeError, match='pinned'):
-        opt.step()
+    # refused BEFORE anything is launched: a kernel over pageable host memory would fault the device (the
+    # stats launch of a step goes out ahead of the host's other preparations, so the check must come first)
+    from elixir_amd import _abi
+    launched = []
+    launchers = ('grad_partials_mt', 'grad_stats_mt', 'finish_decide', 'adam_step_mt', 'adam_step_gated_mt', 'writeback_mt',
+                 'put_hypers')
+    originals = {name: getattr(_abi, name) for name in launchers}
+    try:
+        for name in launchers:
+            setattr(_abi, name, lambda *a, _n=name, **k: launched.append(_n))
+        for gated in (True, False):
+            opt.gated_step = gated
+            with pytest.raises(RuntimeError, match='pinned'):
+                opt.step()
+    finally:
+        for name, fn in originals.items():
+            setattr(_abi, name, fn)
+    assert launched == []
+    torch.cuda.synchronize()
 
 
 def test_mixed_placement_steps_in_one_launch(oracle):
