@@ -42,7 +42,8 @@ EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 
            'elx_decide', 'elx_adam_step_gated_mt', 'elx_writeback_mt', 'elx_refresh_piece_elems', 'elx_writeback',
            'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems',
            'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
-           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers')
+           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers',
+           'elx_adam_step_put_mt')
 
 
 class ElxError(RuntimeError):
@@ -73,7 +74,8 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
                  'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
-           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers'):
+           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers',
+           'elx_adam_step_put_mt'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
     L.elx_check_tables.restype = cint
@@ -85,6 +87,8 @@ def load() -> ctypes.CDLL:
     L.elx_grad_partials_mt.argtypes = [vp, u32, cint, u32, vp, cint, vp]
     L.elx_finish_decide.restype = cint
     L.elx_finish_decide.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp]
+    L.elx_adam_step_put_mt.restype = cint
+    L.elx_adam_step_put_mt.argtypes = [vp, u32, vp, u32, vp, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_put_hypers.restype = cint
     L.elx_put_hypers.argtypes = [vp, u32, vp, vp]
     L.elx_grad_stats_mt_static.restype = cint
@@ -224,6 +228,17 @@ def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hyper
     check('elx_adam_step_mt',
           load().elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, info.total_tiles,
                                   info.max_tiles, div_scale, grad_dtype, lowp_dtype, info.flags, blocks_per_cu, stream))
+
+
+def adam_step_put_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, hyper_host: np.ndarray, d_hypers: int,
+                     info: TableInfo, div_scale: float, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int,
+                     stream: int) -> None:
+    """``put_hypers`` + ``adam_step_mt`` in one call: the two launches go out back to back."""
+    assert hyper_host.dtype == HYPER_DTYPE
+    check('elx_adam_step_put_mt',
+          load().elx_adam_step_put_mt(d_chunks, n_chunks, d_segs, n_segs, _np_ptr(hyper_host), d_hypers, len(hyper_host),
+                                      info.total_tiles, info.max_tiles, div_scale, grad_dtype, lowp_dtype, info.flags,
+                                      blocks_per_cu, stream))
 
 
 def decide(d_stats: int, n_chunks: int, loss_scale: float, max_norm: float, clipping: bool, d_hypers: int,

@@ -1358,6 +1358,28 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
                          grid_tiles_per_chunk, us, false, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
+int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream);
+
+int elx_adam_step_put_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
+                         const ElxHyper *h_hypers, ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,
+                         uint32_t grid_tiles_per_chunk, float div_scale, int grad_dtype, int lowp_dtype, uint32_t flags,
+                         uint32_t blocks_per_cu, void *stream) {
+    if (!h_hypers || !d_hypers) return ELX_E_NULL;
+    // every argument check of the update launch first: nothing goes out when the update would be refused
+    if (!d_chunks || (n_segs && !d_segs)) return ELX_E_NULL;
+    if (n_chunks == 0 || n_chunks > 65535u || total_tiles == 0 || total_tiles > 0x7FFFFFFFull || n_hypers == 0)
+        return ELX_E_SIZE;
+    if (grid_tiles_per_chunk == 0 || (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
+    if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
+    if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    uint32_t lds = 0;
+    if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
+        return rc;
+    if (int rc = elx_put_hypers(h_hypers, n_hypers, d_hypers, stream)) return rc;
+    return elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, total_tiles, grid_tiles_per_chunk,
+                            div_scale, grad_dtype, lowp_dtype, flags, blocks_per_cu, stream);
+}
+
 int elx_decide(const ElxStats *d_stats, uint32_t n_chunks, double loss_scale, double max_norm, int clipping,
                ElxHyper *d_hypers, uint32_t n_hypers, ElxDecision *d_decision, void *stream) {
     if (!d_stats || !d_decision || (n_hypers && !d_hypers)) return ELX_E_NULL;

@@ -61,6 +61,22 @@ def make_hyper_record(lr: float, beta1: float, beta2: float, eps: float, weight_
     return rec
 
 
+_HYPER_RECORDS: Dict = {}
+
+
+def hyper_record_cached(key: Tuple, adamw_mode: bool) -> np.ndarray:
+    """``make_hyper_record`` for ``key = (lr, beta1, beta2, eps, weight_decay, step, bias_correction)``, kept:
+    a step looks up the records the step before it has already computed while its launch was running."""
+    rec = _HYPER_RECORDS.get((key, adamw_mode))
+    if rec is None:
+        if len(_HYPER_RECORDS) > 4096:
+            _HYPER_RECORDS.clear()
+        lr, b1, b2, eps, wd, step, bc = key
+        rec = _HYPER_RECORDS[(key, adamw_mode)] = make_hyper_record(lr, b1, b2, eps, wd, step, bc, adamw_mode)
+        rec.flags.writeable = False    # shared between steps: nobody edits it
+    return rec
+
+
 class _CachedTable:
     """Device copy of a host table, re-uploaded only when the host contents change."""
 
@@ -82,11 +98,15 @@ class _HyperTable:
     def __init__(self):
         self.dev: Optional[torch.Tensor] = None
 
-    def put(self, host: np.ndarray, device: torch.device) -> int:
-        if self.dev is None or self.dev.device != device or self.dev.numel() < host.nbytes:
-            self.dev = torch.empty(max(4096, host.nbytes), dtype=torch.uint8, device=device)
-        _abi.put_hypers(host, self.dev.data_ptr(), torch.cuda.current_stream(device).cuda_stream)
+    def reserve(self, nbytes: int, device: torch.device) -> int:
+        if self.dev is None or self.dev.device != device or self.dev.numel() < nbytes:
+            self.dev = torch.empty(max(4096, nbytes), dtype=torch.uint8, device=device)
         return self.dev.data_ptr()
+
+    def put(self, host: np.ndarray, device: torch.device) -> int:
+        ptr = self.reserve(host.nbytes, device)
+        _abi.put_hypers(host, ptr, torch.cuda.current_stream(device).cuda_stream)
+        return ptr
 
 
 class _DevicePlan:
@@ -156,9 +176,10 @@ class _Prepared:
     """Everything a step needs that does not depend on the gradient flags: built while the stats
     launch is still running, consumed (and only then committed to the optimizer state) by step()."""
 
-    def __init__(self, dplan, hyper_host, grad_code, lowp_code, device, states):
+    def __init__(self, dplan, hyper_host, grad_code, lowp_code, device, states, hyper_keys=()):
         self.dplan: _DevicePlan = dplan
         self.hyper_host: np.ndarray = hyper_host
+        self.hyper_keys = tuple(hyper_keys)    # (lr, beta1, beta2, eps, weight_decay, step, bias_correction) per record
         self.grad_code, self.lowp_code, self.device = grad_code, lowp_code, device
         self.states: List[Dict] = states      # per-parameter state dicts whose 'step' advances on commit
         self.d_hypers: int = 0
@@ -283,10 +304,8 @@ class HybridAdam(torch.optim.Optimizer):
         self._prepared = None
 
     def _hyper_table(self, hypers: Dict) -> np.ndarray:
-        return np.concatenate([
-            make_hyper_record(lr, b1, b2, eps, wd, step, bc, self.adamw_mode)
-            for (lr, b1, b2, eps, wd, step, bc) in hypers.keys()
-        ])
+        records = [hyper_record_cached(key, self.adamw_mode) for key in hypers.keys()]
+        return records[0] if len(records) == 1 else np.concatenate(records)
 
     def step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
         """``gated``: the unscale parameters and the skip flag are read on the device from the gate
@@ -323,16 +342,21 @@ class HybridAdam(torch.optim.Optimizer):
             with torch.enable_grad():
                 loss = closure()
         if self._prepared is None:
-            self.prepare_step()
+            self.prepare_step(upload=False)    # the records go out with the launch below
         prep, self._prepared = self._prepared, None
         if prep is None:
             return loss
 
-        if not prep.d_hypers:
-            prep.d_hypers = self._hyper_table_dev.put(prep.hyper_host, prep.device)
         plan = prep.dplan.plan
         stream = torch.cuda.current_stream(prep.device).cuda_stream
         events = self.kernel_events
+        together = False    # hyper records and update in one call: the two launches go out back to back
+        if not prep.d_hypers:
+            if gated or events is not None or prep.dplan.rows is None:
+                prep.d_hypers = self._hyper_table_dev.put(prep.hyper_host, prep.device)
+            else:
+                prep.d_hypers = self._hyper_table_dev.reserve(prep.hyper_host.nbytes, prep.device)
+                together = True
         if prep.dplan.rows is not None:
             if events is not None:
                 if 'adam_step' not in events:    # created once, recorded again every step
@@ -342,6 +366,10 @@ class HybridAdam(torch.optim.Optimizer):
                 _abi.adam_step_gated_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs),
                                         prep.d_hypers, len(prep.hyper_host), plan.info, prep.grad_code,
                                         prep.lowp_code, self.blocks_per_cu, stream)
+            elif together:
+                _abi.adam_step_put_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs),
+                                      prep.hyper_host, prep.d_hypers, plan.info, float(div_scale), prep.grad_code,
+                                      prep.lowp_code, self.blocks_per_cu, stream)
             else:
                 _abi.adam_step_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs),
                                   prep.d_hypers, len(prep.hyper_host), plan.info, float(div_scale), prep.grad_code,
@@ -374,6 +402,9 @@ class HybridAdam(torch.optim.Optimizer):
             state['step'] += 1
         if self._binding is not None and prep.lowp_code != _abi.ELX_NONE:
             self._binding.fused_writeback = True
+        # the records of the next step, computed now, while the device is busy with this one
+        for (lr, b1, b2, eps, wd, step, bc) in prep.hyper_keys:
+            hyper_record_cached((lr, b1, b2, eps, wd, step + 1, bc), self.adamw_mode)
 
     def abort_step(self) -> None:
         """The launched step found the skip flag set on the device: nothing was updated and no step
@@ -515,7 +546,8 @@ class HybridAdam(torch.optim.Optimizer):
             return out
 
         dplan = self._device_plan(key, buffers, lowp_dtype, grad_code, lowp_code, len(hypers), device)
-        return _Prepared(dplan, self._hyper_table(hypers), grad_code, lowp_code, device, [e[0] for e in entries])
+        return _Prepared(dplan, self._hyper_table(hypers), grad_code, lowp_code, device, [e[0] for e in entries],
+                         hypers.keys())
 
     # ---- standalone, on ordinary parameters
 
@@ -589,4 +621,5 @@ class HybridAdam(torch.optim.Optimizer):
                     for (_, _, (g, p, m, v, n)), h in zip(items, idx_of)]
 
         dplan = self._device_plan(key, buffers, grad_dtype, grad_code, _abi.ELX_NONE, len(hypers), device)
-        return _Prepared(dplan, self._hyper_table(hypers), grad_code, _abi.ELX_NONE, device, [it[0] for it in items])
+        return _Prepared(dplan, self._hyper_table(hypers), grad_code, _abi.ELX_NONE, device, [it[0] for it in items],
+                         hypers.keys())

@@ -291,6 +291,17 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
 int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream);
 
 /*
+ * elx_put_hypers followed by elx_adam_step_mt on the same table, in one call (the two launches go out
+ * back to back, which matters for steps of a few tens of microseconds): the whole of
+ * `self.optim.step(div_scale=...)` (optimizer.py:216) for a host-decided or standalone step.  The
+ * arguments are those of the two functions; nothing is launched when the update would be refused.
+ */
+int elx_adam_step_put_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
+                         const ElxHyper *h_hypers, ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,
+                         uint32_t grid_tiles_per_chunk, float div_scale, int grad_dtype, int lowp_dtype, uint32_t flags,
+                         uint32_t blocks_per_cu, void *stream);
+
+/*
  * The host decisions of optimizer.py:137-183 taken on the device, so that the update can be enqueued
  * without waiting for the flags to reach the host: one thread reads the n_chunks records of a stats or
  * landing launch (in the order given), ORs the overflow flags and, with `clipping`, forms the global
