@@ -35,6 +35,8 @@ BYTES_STATS = 2                 # per valid element: the compulsory second read 
 # first 16 hex digits), and the line names the summary it comes from.
 RECORDED_TRAFFIC = {
     # workload: (bytes per launch, summary under profiles/, kernel source the counters were read on)
+    'c5': (94.411e9 + 94.364e9, 'profiles/adam_step_kernel_c5_llama7b.md', 'ac9e8c28e0a64fa1'),
+    'c4': (18.4445e9 + 18.4305e9, 'profiles/all_kernels_c4_opt1b3_c2_gpt2_c1.md', 'ac9e8c28e0a64fa1'),
 }
 KERNEL_SOURCE = os.path.join(ROOT, 'elixir_amd', 'csrc', 'elx_kernels.hip')
 
@@ -549,7 +551,9 @@ def summary_of(line):
             'metric': line['metric'], 'value': line['value'], 'unit': line['unit'], 'steps': line['steps'],
             'ms_per_step': line['ms_per_step'], 'ms_min': line['step']['ms_min'],
             'roofline_frac_update_launch': line['roofline']['frac'],
-            'update_launch_ms': line['roofline']['ms_per_launch'], 'update_launch_timed_in': line['roofline'].get('timed_in')}
+            'update_launch_ms': line['roofline']['ms_per_launch'], 'update_launch_timed_in': line['roofline'].get('timed_in'),
+            'update_launch_bytes': line['roofline']['bytes_per_launch'], 'update_launch_traffic': line['roofline'].get('traffic'),
+            'update_launch_traffic_source': line['roofline'].get('traffic_source')}
     for k in ('frac_30B', 'frac_touch_once_28B', 'frac_28B'):
         if k in line['step']:
             keep['step_' + k] = line['step'][k]
