@@ -130,6 +130,32 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_NONE, 4, 0, None) == -2
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_F16, 0, 0, None) == -7
     assert lib.elx_refresh_piece_elems() == 1024
+    # the stats launch alone, the fold-and-decide launch, the hyper records through launch arguments
+    assert lib.elx_grad_partials_mt(None, 1, _abi.ELX_F16, 1, 1, 0, None) == -1
+    assert lib.elx_grad_partials_mt(1, 1, _abi.ELX_F16, 1025, 1, 0, None) == -7
+    assert lib.elx_grad_partials_mt(1, 1, 9, 1, 1, 0, None) == -2
+    assert lib.elx_max_ctl_hypers() == 64
+    assert lib.elx_finish_decide(None, 1, 1, 8, 8, 8, 1, 8, None, 8, None) == -1
+    assert lib.elx_finish_decide(8, 1, 1, 8, None, 8, 1, 8, None, 8, None) == -1            # no control block
+    assert lib.elx_finish_decide(8, 1, 1, 8, 8, 8, 1, 8, None, None, None) == -1            # no counter
+    assert lib.elx_finish_decide(8, 0, 1, 8, 8, 8, 1, 8, None, 8, None) == -7
+    assert lib.elx_finish_decide(8, 1, 0, 8, 8, 8, 1, 8, None, 8, None) == -7
+    assert lib.elx_finish_decide(8, 1, 1, 8, 8, 8, 65, 8, None, 8, None) == -7             # more records than the block can carry
+    assert lib.elx_finish_decide(8, 1, 1, 8, 12, 8, 1, 8, None, 8, None) == -3             # control block not 8-byte aligned
+    assert lib.elx_put_hypers(None, 1, 8, None) == -1
+    assert lib.elx_put_hypers(8, 0, 8, None) == -7
+    assert lib.elx_put_hypers(8, 1, 6, None) == -3
+    for args, code in (((8, 1, None, 0, None, 8, 1, 4, 4, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None), -1),
+                       ((8, 1, None, 0, 8, 8, 0, 4, 4, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None), -7),
+                       ((8, 1, None, 0, 8, 8, 1, 4, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None), -6),
+                       ((8, 1, None, 0, 8, 8, 1, 4, 4, -1.0, 9, _abi.ELX_NONE, 0, 0, None), -2),
+                       ((8, 1, None, 0, 8, 8, 1, 4, 4, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 2, None), -7)):
+        assert lib.elx_adam_step_put_mt(*args) == code, args    # refused before the records are even read
+    # the variant without a workspace refuses what its fixed array cannot hold, before it looks anything up
+    assert lib.elx_static_partials() == 65536
+    assert lib.elx_grad_stats_mt_static(8, 65, _abi.ELX_F16, 1024, 8, 0, None) == -7
+    assert lib.elx_grad_stats_mt_static(8, 1, 9, 1, 8, 0, None) == -2
+    assert lib.elx_grad_stats_mt_static(None, 1, _abi.ELX_F16, 1, 8, 0, None) == -1
 
 
 def test_check_land_rows_accepts_and_rejects():
