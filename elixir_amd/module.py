@@ -161,8 +161,12 @@ class ElixirModule(nn.Module):
                  reserve_memory: bool = True) -> None:
         super().__init__()
         assert dtype in {torch.float, torch.float16, torch.bfloat16}
-        if prefetch or use_fused_kernels:
-            raise NotImplementedError('prefetch and fused forward kernels belong to the forward/backward pass')
+        # Both are speed settings of the reference's forward/backward pass (module.py:51-75: overlapped chunk
+        # prefetch, fused LayerNorm / attention); neither changes a result.  That pass is not part of this
+        # build, so they are accepted -- the reference's own callers pass them (example/common/elx.py:37)
+        # -- and have no effect here.
+        self.prefetch_flag = bool(prefetch)
+        self.use_fused_kernels = bool(use_fused_kernels)
 
         self.synthetic = not isinstance(module, nn.Module)
         self.module = module if not self.synthetic else None

@@ -401,3 +401,70 @@ def test_tables_prepared_at_backward_follow_late_hyperparameter_changes():
         for name, want in ref.state_dict().items():
             torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
         del ahead
+
+
+def test_fine_tune_loop_of_the_reference_with_torch_adam_and_a_warmup_schedule():
+    """The shape of example/fine-tune/elixir_mini.py:70-110 and func_module.py:46-66: an fp32 module, a plain
+    ``torch.optim.Adam`` with a decay group and a no-decay group as the inner optimizer,
+    ``ElixirOptimizer(model, optimizer, init_step=True)``, a linear warm-up / decay schedule built ON THE
+    WRAPPER, and the loop zero_grad -> forward -> optimizer.backward -> optimizer.step -> lr_scheduler.step.
+    Against the same loop on a plain copy (which takes the allocation step's zero-gradient update by hand):
+    the same weights to the reference's own tolerance, the same learning rates."""
+
+    def schedule(opt, warm=3, total=10):    # transformers' get_linear_schedule_with_warmup
+        return torch.optim.lr_scheduler.LambdaLR(
+            opt, lambda s: s / max(1, warm) if s < warm else max(0.0, (total - s) / max(1, total - warm)))
+
+    def groups(model):
+        decay = [p for n, p in model.named_parameters() if 'norm' not in n and 'bias' not in n]
+        rest = [p for n, p in model.named_parameters() if 'norm' in n or 'bias' in n]
+        return [dict(params=decay, weight_decay=0.01), dict(params=rest, weight_decay=0.0)]
+
+    torch.manual_seed(0)
+    ref = Net().to(DEV)
+    model = copy.deepcopy(ref)
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    x0 = batch(gen)
+    # What init_step does (optimizer.py:94-113): one step with zero gradients, at the constructor's
+    # learning rate, on the master weights only -- the parameters the first forward pass sees are not
+    # refreshed (optimizer.py:113 passes update_flag=False).  On the plain copy: take the first batch's
+    # gradients on the untouched weights, then the zero-gradient step, then the first real step.
+    ropt = torch.optim.Adam(groups(ref), lr=2e-3, eps=1e-8)
+    ref(x0).backward()
+    first_grads = [p.grad.clone() for p in ref.parameters()]
+    for p in ref.parameters():
+        p.grad = torch.zeros_like(p)
+    ropt.step()
+    rsched = schedule(ropt)
+
+    optimizer = torch.optim.Adam(groups(model), lr=2e-3, eps=1e-8)
+    named = [(n, p.numel()) for n, p in model.named_parameters()]
+    module = ea.ElixirModule(model, ea.greedy_search(named, 4096, torch.float32), None, dtype=torch.float32,
+                             use_fused_kernels=True)
+    optimizer = ea.ElixirOptimizer(module, optimizer, init_step=True)
+    assert isinstance(optimizer, torch.optim.Optimizer) and not optimizer.scaled_optimizer
+    lr_scheduler = schedule(optimizer)
+
+    for step in range(6):
+        x = x0 if step == 0 else batch(gen)
+        if step == 0:
+            for p, g in zip(ref.parameters(), first_grads):
+                p.grad = g
+        else:
+            ropt.zero_grad()
+            ref(x).backward()
+        ropt.step()
+        rsched.step()
+
+        optimizer.zero_grad()
+        loss = module(x)
+        optimizer.backward(loss)
+        optimizer.step()
+        lr_scheduler.step()
+
+        assert [g['lr'] for g in optimizer.param_groups] == [g['lr'] for g in ropt.param_groups]
+        module.materialize_params()
+        sd = module.state_dict()
+        for name, want in ref.state_dict().items():
+            torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
+    assert lr_scheduler.last_epoch == 6 and optimizer.param_groups[0]['lr'] == pytest.approx(2e-3 * 4 / 7)

@@ -216,6 +216,18 @@ def test_module_builds_paired_chunks(dtype):
     assert module.state_dict(from_param=True)['fc.weight'].dtype == dtype
 
 
+def test_module_accepts_the_forward_pass_settings_of_the_reference_callers():
+    """example/common/elx.py:37 builds ElixirModule(model, sr, group, prefetch=True, dtype=torch.float16,
+    use_fused_kernels=True): both are speed settings of the forward pass, accepted and without effect here."""
+    net = TinyNet()
+    named = [(n, p.numel()) for n, p in net.named_parameters()]
+    sr = ea.greedy_search(named, 1024, torch.float16, shard_device=torch.device('cpu'))
+    module = ea.ElixirModule(net, sr, None, prefetch=True, dtype=torch.float16, use_fused_kernels=True)
+    assert module.use_amp and module.prefetch_flag and module.use_fused_kernels
+    opt = ea.ElixirOptimizer(module, ea.HybridAdam(net.parameters(), lr=1e-3), initial_scale=64, hysteresis=1)
+    assert opt.loss_scale == 64.0
+
+
 def test_optimizer_ranges_groups_and_refusal_to_run_on_cpu():
     torch.manual_seed(0)
     net = TinyNet()
