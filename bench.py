@@ -191,7 +191,7 @@ def fused_landing_leg(built, steps):
         'step_gbps_28B': BYTES_UPDATE * n_valid / t_step / 1e9,
         'step_frac_28B': BYTES_UPDATE * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
         'land_kernel': {
-            'kernel': 'land_grads_kernel+stats_finish_kernel',
+            'kernel': 'land_grads_kernel+stats_fold_kernel+stats_finish_kernel',
             'ms_per_launch': t_land * 1e3,
             'bytes_per_launch': 2 * esize * n_alloc,
             'achieved': 2 * esize * n_alloc / t_land / 1e9,

@@ -309,7 +309,7 @@ class HybridAdam(torch.optim.Optimizer):
 
     def step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
         """``gated``: the unscale parameters and the skip flag are read on the device from the gate
-        words of the prepared hyper table, where ``elx_decide`` has put them (``div_scale`` is then
+        words of the prepared hyper table, where ``elx_finish_decide`` has put them (``div_scale`` is then
         ignored).  ``defer_commit``: launch only; the caller finishes with ``commit_step()`` once it
         knows that the step happened, or ``abort_step()`` when the device decided to skip.
 

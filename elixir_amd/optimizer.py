@@ -3,15 +3,21 @@ constructor, methods and control flow, driving the HIP kernels.
 
 One step is:
 
-  1. one stats launch over every parameter chunk that has no flags yet (overflow flag and sum of
-     squares of the still-scaled gradients) -- none at all when the gradients arrived through the
-     fused landing, which leaves the flags on the device -- and ONE device-to-host copy of 16 bytes
-     per chunk (the reference pays two ``.item()`` per chunk at gradient-landing time, plus one for
-     the loss scale, plus one for the norm);
-  2. the host decisions of optimizer.py:192-209 in Python floats: overflow -> skip and back off,
-     otherwise combined scale = loss scale (x clip coefficient);
-  3. one fused launch: unscale + Adam/AdamW on master/m/v + low-precision writeback
-     (optimizer.py:216-219), or the writeback alone on a skipped step (optimizer.py:196-203).
+  1. one stats launch over every parameter chunk (overflow flag and sum of squares of the
+     still-scaled gradients) -- none at all when the gradients arrived through the fused landing,
+     which leaves the flags on the device;
+  2. the decisions of optimizer.py:192-209 -- overflow -> skip and back off, otherwise combined scale
+     = loss scale (x clip coefficient) -- taken ON THE DEVICE by the launch that folds the flags, in
+     the float64 arithmetic of the reference's Python, and left where the update launch reads them;
+     the decision and the 16 bytes of flags per chunk come back through pinned host memory for the
+     host's bookkeeping (the reference pays two ``.item()`` per chunk at gradient-landing time, plus
+     one for the loss scale, plus one for the norm);
+  3. one fused launch, enqueued without waiting for 2.: unscale + Adam/AdamW on master/m/v +
+     low-precision writeback (optimizer.py:216-219), which turns into the writeback alone when the
+     decision says skip (optimizer.py:196-203).
+
+With ``gated_step`` off, or when the flags of some chunks are already on the host, the host fetches the
+flags, decides in Python floats and only then launches 3. (or the writeback alone).
 
 Differences from the reference, all on purpose:
   * clipping works: ``max_norm > 0`` switches ``l2_norm_flag`` on for every parameter chunk (the
