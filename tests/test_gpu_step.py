@@ -1013,7 +1013,8 @@ def DeviceTableOf(rows):
 @pytest.mark.parametrize('fused_landing', [False, True])
 def test_recorded_step_replays_like_the_eager_one(oracle, fused_landing):
     """A seven-step trajectory -- clean steps, an overflow that only arms the back-off (hysteresis 2),
-    one that backs off, clean steps until the scale grows again -- three times: decided on the host,
+    one that backs off, clean steps until the scale grows again, the learning rate changing at every
+    step -- three times: decided on the host,
     decided on the device with eager launches, and with the launches of the step recorded as a HIP
     graph and replayed (the first step runs eagerly, the second records, all later ones replay -- the
     overflows among them).  Identical bits in every buffer after every step, identical scale, reports and step counts;
@@ -1032,6 +1033,12 @@ def test_recorded_step_replays_like_the_eager_one(oracle, fused_landing):
         gen = torch.Generator(device=DEV).manual_seed(23)
         trace = []
         for step in range(7):
+            # a learning rate that changes every step: a replayed step must pick up the new hyper records
+            for group in opt.param_groups:
+                group['lr'] = 1e-3 * (1 + step % 3)
+            for oc in ochunks:
+                for seg in oc.segments:
+                    seg.lr = 1e-3 * (1 + step % 3)
             payloads = []
             for pc in module.param_chunks:
                 g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (2e-2 * opt.loss_scale)
