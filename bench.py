@@ -545,6 +545,36 @@ def chunk_set_line(args, workload: str, device, events_in_timed_steps: bool):
     return out, built
 
 
+def skip_step_leg(built, steps=20):
+    """Configuration 3's timed part: the step that finds an overflow (on the c2 layout: one +inf planted in
+    the gradients of the last chunk) -- stats launch, decision, and the update launch turned into the
+    low-precision refresh of every shard; master / exp_avg / exp_avg_sq untouched, loss scale backed off.
+    Bytes: 2 B per valid element (the flags) + 6 B per allocated element (4 B of master read, 2 B written).
+    Runs last on its chunk set: it leaves the loss scale at its floor."""
+    opt = built.optimizer
+    pc = built.module.param_chunks[-1]
+    keep = built.grads[-1][pc.utilized_size // 2].clone()
+    built.grads[-1][pc.utilized_size // 2] = float('inf')
+    master0 = pc.paired_chunk.shard[:4096].clone()
+    ts = []
+    for i in range(steps + 3):
+        built.land_gradients()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        ts.append(time.perf_counter() - t0)
+        assert opt.last_step_info['found_inf'] is True
+    built.grads[-1][pc.utilized_size // 2] = keep
+    assert torch.equal(master0, pc.paired_chunk.shard[:4096])
+    t = float(np.mean(ts[3:]))
+    nbytes = BYTES_STATS * built.n_valid + 6 * built.n_alloc
+    return {'what': 'c3: the step that finds an overflow on the c2 layout (flags, decision, refresh of every shard; '
+                    'nothing updated); the parity of the whole scenario is tests/test_gpu_configs.py',
+            'steps': steps, 'ms_per_step': t * 1e3, 'ms_min': float(np.min(ts[3:])) * 1e3, 'bytes_per_step': nbytes,
+            'gbps': nbytes / t / 1e9, 'frac': nbytes / t / 1e9 / HBM_PEAK_GBPS, 'loss_scale_after': opt.loss_scale}
+
+
 def summary_of(line):
     """What the `configs` object keeps of a workload's line."""
     keep = {'workload': line['config']['workload'], 'valid_elements': line['config']['valid_elements'],
@@ -640,6 +670,8 @@ def main():
     out, built = chunk_set_line(args, args.workload, device, events_in_timed_steps=args.workload == 'c5')
     if args.cpu_sample > 0:
         out['cpu_baseline'] = cpu_baseline(built, args.cpu_sample)
+    if args.workload == 'c2':
+        out['skip_step'] = skip_step_leg(built, steps=max(3, args.steps))
     del built
     free_device_memory()
 
@@ -651,6 +683,8 @@ def main():
         for name, steps in (('c4', 20), ('c2', 50)):
             small.steps, small.warmup = steps, 5
             line, b = chunk_set_line(small, name, device, events_in_timed_steps=False)
+            if name == 'c2':
+                configs['c3'] = skip_step_leg(b)
             del b
             free_device_memory()
             configs[name] = summary_of(line)
@@ -660,8 +694,6 @@ def main():
         small.steps, small.warmup = 10, 2
         configs['velocity'] = summary_of(velocity_line(small))
         free_device_memory()
-        configs['c3'] = 'the overflow path on the c2 layout is a correctness gate, not a throughput figure: ' \
-                        'tests/test_gpu_configs.py'
         out['configs'] = configs
     print(json.dumps(out))
 

@@ -32,6 +32,10 @@ def test_bench_json_line():
     c = out['cpu_baseline']
     assert c['kind'] == 'port' and c['cores'] >= 1 and c['value'] > 0 and c['unit'] == 'elements/s'
     assert out['fused_landing']['ms_per_step'] > 0
+    # configuration 3's timed part rides the c2 line: the step that finds an overflow
+    skip = out['skip_step']
+    assert skip['bytes_per_step'] == 2 * 124_439_808 + 6 * 134_217_728 and 0 < skip['frac'] < 1
+    assert skip['loss_scale_after'] == 64.0 / 2**6    # 3 warm-up + 3 timed skipped steps, each halves the scale
 
 
 def test_velocity_line():
