@@ -13,6 +13,7 @@ import numpy as np
 ELX_ABI_VERSION = 2
 ELX_F32, ELX_F16, ELX_BF16, ELX_NONE = 0, 1, 2, -1
 ELX_FLAG_SCALAR_ONLY = 1
+ELX_FLAG_KEEP_CACHED = 2
 ELX_E_NULL, ELX_E_DTYPE, ELX_E_ALIGN, ELX_E_RANGE, ELX_E_ORDER, ELX_E_TILES, ELX_E_SIZE = -1, -2, -3, -4, -5, -6, -7
 ELX_HYPER_L2 = 1
 ELX_HYPER_LERP_FROM_G = 2
@@ -176,19 +177,25 @@ def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, 
     return TableInfo((int(tiles.value), int(max_tiles.value), bool(aligned.value)))
 
 
+def stats_flags(scalar_only: bool, keep_cached: bool) -> int:
+    return (ELX_FLAG_SCALAR_ONLY if scalar_only else 0) | (ELX_FLAG_KEEP_CACHED if keep_cached else 0)
+
+
 def grad_stats_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_partials: int, d_stats: int,
-                  scalar_only: bool, stream: int) -> None:
+                  scalar_only: bool, stream: int, keep_cached: bool = False) -> None:
+    """``keep_cached``: ordinary instead of non-temporal loads, for a gradient set that fits the
+    memory-side cache and is read again by the update launch right behind."""
     check('elx_grad_stats_mt',
           load().elx_grad_stats_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, d_stats,
-                                   int(scalar_only), stream))
+                                   stats_flags(scalar_only, keep_cached), stream))
 
 
 def grad_partials_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_partials: int,
-                     scalar_only: bool, stream: int) -> None:
+                     scalar_only: bool, stream: int, keep_cached: bool = False) -> None:
     """The first launch of ``grad_stats_mt`` alone: the partials are left for ``finish_decide``."""
     check('elx_grad_partials_mt',
-          load().elx_grad_partials_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, int(scalar_only),
-                                      stream))
+          load().elx_grad_partials_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials,
+                                      stats_flags(scalar_only, keep_cached), stream))
 
 
 def finish_decide(d_partials: int, n_chunks: int, blocks_per_chunk: int, d_stats: int, ctl: int, d_hypers: int,
@@ -214,12 +221,12 @@ def static_partials() -> int:
 
 
 def grad_stats_mt_static(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_chunk: int, d_stats: int,
-                         scalar_only: bool, stream: int) -> None:
+                         scalar_only: bool, stream: int, keep_cached: bool = False) -> None:
     """``grad_stats_mt`` with the partials in the library's fixed device array: allocates nothing.  The
     stream's device must be the current one; overlapping calls on one GPU race."""
     check('elx_grad_stats_mt_static',
-          load().elx_grad_stats_mt_static(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_stats, int(scalar_only),
-                                          stream))
+          load().elx_grad_stats_mt_static(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_stats,
+                                          stats_flags(scalar_only, keep_cached), stream))
 
 
 def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hypers: int, n_hypers: int, info: TableInfo,

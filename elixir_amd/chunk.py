@@ -94,6 +94,19 @@ def stats_launch_blocks(n_valid_max: int) -> int:
     return int(max(1, min(1024, math.ceil(n_valid_max / 16384))))
 
 
+# The memory-side cache of the GPU holds 256 MiB.  A gradient set below this size is read by the stats pass
+# with ordinary loads, so that the update launch right behind it finds the gradients there (step time
+# -2 % to -5 % between 64 and 256 MiB of gradients); larger sets are read with non-temporal loads, which
+# stream faster (a 2.6 GB set: 0.39 against 0.45 ms).
+KEEP_GRADS_CACHED_BELOW = 256 << 20
+
+
+def keep_grads_cached(chunk_rows: np.ndarray, grad_dtype: int) -> bool:
+    """Whether the gradients the stats launch over ``chunk_rows`` reads fit the memory-side cache."""
+    esize = 4 if grad_dtype == _abi.ELX_F32 else 2
+    return int(chunk_rows['n_valid'].sum()) * esize <= KEEP_GRADS_CACHED_BELOW
+
+
 def launch_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.device,
                       table: Optional[DeviceTable] = None, workspace: Optional[Dict] = None) -> torch.Tensor:
     """Enqueues the stats pass for the chunks described by ``chunk_rows`` (host table, only grad /
@@ -115,7 +128,8 @@ def launch_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.dev
     d_partials = buf.data_ptr()
     d_stats = d_partials + n * bpc * _abi.STATS_DTYPE.itemsize
     stream = torch.cuda.current_stream(device).cuda_stream
-    _abi.grad_stats_mt(table.ptr, n, grad_dtype, bpc, d_partials, d_stats, not aligned, stream)
+    _abi.grad_stats_mt(table.ptr, n, grad_dtype, bpc, d_partials, d_stats, not aligned, stream,
+                       keep_cached=keep_grads_cached(chunk_rows, grad_dtype))
     return buf[n * bpc * _abi.STATS_DTYPE.itemsize:need]
 
 

@@ -109,9 +109,14 @@ struct Elem<ELX_BF16> {
     static __device__ __forceinline__ uint16_t from_f32(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }
 };
 
-template <typename V>
+// KEEP: an ordinary load, which leaves the line in the memory-side cache for a launch that reads it
+// again soon; otherwise non-temporal (read once, do not displace anything).
+template <bool KEEP, typename V>
 __device__ __forceinline__ V ld_stream(const V *p) {
-    return __builtin_nontemporal_load(p);
+    if constexpr (KEEP)
+        return *p;
+    else
+        return __builtin_nontemporal_load(p);
 }
 
 // Tile-local buffer addressing for the update launch: each stream of a tile is described by a
@@ -572,7 +577,7 @@ __device__ __forceinline__ void stats_elem(float x, float &acc, float &poison) {
     poison = fmaf(x, 0.0f, poison);
 }
 
-template <int GD>
+template <int GD, bool KEEP>
 __device__ __forceinline__ void grad_stats_body(const ElxChunk &c, uint32_t bpc, ElxStats *__restrict__ partials,
                                                 uint32_t scalar_only) {
     typedef typename Elem<GD>::scalar gscalar;
@@ -594,7 +599,7 @@ __device__ __forceinline__ void grad_stats_body(const ElxChunk &c, uint32_t bpc,
             const gvec *gp = reinterpret_cast<const gvec *>(g + base) + threadIdx.x;
             gvec G[kStatsUnroll];
 #pragma unroll
-            for (int u = 0; u < kStatsUnroll; ++u) G[u] = ld_stream(gp + u * kStatsThreads);
+            for (int u = 0; u < kStatsUnroll; ++u) G[u] = ld_stream<KEEP>(gp + u * kStatsThreads);
 #pragma unroll
             for (int u = 0; u < kStatsUnroll; ++u)
 #pragma unroll
@@ -618,12 +623,12 @@ __device__ __forceinline__ void grad_stats_body(const ElxChunk &c, uint32_t bpc,
     }
 }
 
-template <int GD>
+template <int GD, bool KEEP>
 __global__ __launch_bounds__(kStatsThreads) void grad_stats_kernel(const ElxChunk *__restrict__ chunks, uint32_t bpc,
                                                                    ElxStats *__restrict__ partials,
                                                                    uint32_t scalar_only) {
     const ElxChunk c = chunks[blockIdx.y];
-    grad_stats_body<GD>(c, bpc, partials, scalar_only);
+    grad_stats_body<GD, KEEP>(c, bpc, partials, scalar_only);
 }
 
 // One buffer, described in the kernel arguments.
@@ -631,7 +636,7 @@ template <int GD>
 __global__ __launch_bounds__(kStatsThreads) void grad_stats_one_kernel(ElxChunk c, uint32_t bpc,
                                                                        ElxStats *__restrict__ partials,
                                                                        uint32_t scalar_only) {
-    grad_stats_body<GD>(c, bpc, partials, scalar_only);
+    grad_stats_body<GD, false>(c, bpc, partials, scalar_only);
 }
 
 __global__ __launch_bounds__(kStatsThreads) void stats_finish_kernel(const ElxStats *__restrict__ partials,
@@ -1146,6 +1151,17 @@ int scratch_of_current_device(void **out) {
 
 }    // namespace
 
+template <int GD>
+static void launch_grad_stats(bool keep, dim3 grid, hipStream_t st, const ElxChunk *d_chunks, uint32_t bpc,
+                              ElxStats *d_partials, uint32_t scalar_only) {
+    if (keep)
+        hipLaunchKernelGGL((grad_stats_kernel<GD, true>), grid, dim3(kStatsThreads), 0, st, d_chunks, bpc, d_partials,
+                           scalar_only);
+    else
+        hipLaunchKernelGGL((grad_stats_kernel<GD, false>), grid, dim3(kStatsThreads), 0, st, d_chunks, bpc, d_partials,
+                           scalar_only);
+}
+
 extern "C" {
 
 int elx_version(void) { return ELX_ABI_VERSION; }
@@ -1246,12 +1262,12 @@ int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t 
 }
 
 int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
-                         ElxStats *d_partials, int scalar_only, void *stream);
+                         ElxStats *d_partials, int flags, void *stream);
 
 int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
-                      ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream) {
+                      ElxStats *d_partials, ElxStats *d_stats, int flags, void *stream) {
     if (!d_stats) return ELX_E_NULL;
-    if (int rc = elx_grad_partials_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, scalar_only, stream))
+    if (int rc = elx_grad_partials_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, d_partials, flags, stream))
         return rc;
     hipLaunchKernelGGL(stats_finish_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, (hipStream_t)stream, d_partials,
                        blocks_per_chunk, d_stats);
@@ -1259,23 +1275,19 @@ int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtyp
 }
 
 int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
-                         ElxStats *d_partials, int scalar_only, void *stream) {
+                         ElxStats *d_partials, int flags, void *stream) {
     if (!d_chunks || !d_partials) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxStatsBlocks)
         return ELX_E_SIZE;
+    if ((uint32_t)flags & ~(uint32_t)(ELX_FLAG_SCALAR_ONLY | ELX_FLAG_KEEP_CACHED)) return ELX_E_RANGE;
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid(blocks_per_chunk, n_chunks);
-    const uint32_t so = scalar_only ? 1u : 0u;
+    const uint32_t so = ((uint32_t)flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u;
+    const bool keep = ((uint32_t)flags & ELX_FLAG_KEEP_CACHED) != 0;
     switch (grad_dtype) {
-        case ELX_F32:
-            hipLaunchKernelGGL((grad_stats_kernel<ELX_F32>), grid, dim3(kStatsThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
-            break;
-        case ELX_F16:
-            hipLaunchKernelGGL((grad_stats_kernel<ELX_F16>), grid, dim3(kStatsThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
-            break;
-        case ELX_BF16:
-            hipLaunchKernelGGL((grad_stats_kernel<ELX_BF16>), grid, dim3(kStatsThreads), 0, st, d_chunks, blocks_per_chunk, d_partials, so);
-            break;
+        case ELX_F32: launch_grad_stats<ELX_F32>(keep, grid, st, d_chunks, blocks_per_chunk, d_partials, so); break;
+        case ELX_F16: launch_grad_stats<ELX_F16>(keep, grid, st, d_chunks, blocks_per_chunk, d_partials, so); break;
+        case ELX_BF16: launch_grad_stats<ELX_BF16>(keep, grid, st, d_chunks, blocks_per_chunk, d_partials, so); break;
         default: return ELX_E_DTYPE;
     }
     return (int)hipGetLastError();
@@ -1316,17 +1328,18 @@ uint32_t elx_max_ctl_hypers(void) { return kMaxCtlHypers; }
 uint32_t elx_static_partials(void) { return kStaticPartials; }
 
 int elx_grad_stats_mt_static(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
-                             ElxStats *d_stats, int scalar_only, void *stream) {
+                             ElxStats *d_stats, int flags, void *stream) {
     if (!d_chunks || !d_stats) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxStatsBlocks)
         return ELX_E_SIZE;
     if ((uint64_t)n_chunks * blocks_per_chunk > kStaticPartials) return ELX_E_SIZE;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
+    if ((uint32_t)flags & ~(uint32_t)(ELX_FLAG_SCALAR_ONLY | ELX_FLAG_KEEP_CACHED)) return ELX_E_RANGE;
     void *partials = nullptr;
     if (int rc = scratch_of_current_device(&partials)) return rc;
     // every partial the finish launch reads is written by the stats launch first: nothing to clear
     return elx_grad_stats_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, reinterpret_cast<ElxStats *>(partials),
-                             d_stats, scalar_only, stream);
+                             d_stats, flags, stream);
 }
 
 int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,

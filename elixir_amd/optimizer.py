@@ -40,8 +40,8 @@ import torch
 from torch.nn import Parameter
 
 from . import _abi
-from .chunk import (Chunk, DeviceTable, StatsArena, dtype_code, kernel_device, launch_grad_stats, read_grad_stats,
-                    resolve_pending_stats, stats_launch_blocks)
+from .chunk import (Chunk, DeviceTable, StatsArena, dtype_code, keep_grads_cached, kernel_device, launch_grad_stats,
+                    read_grad_stats, resolve_pending_stats, stats_launch_blocks)
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
 from .hybrid_adam import HybridAdam
 
@@ -541,7 +541,9 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 rows[i]['n_alloc'] = c.shard_size
                 rows[i]['n_valid'] = c.n_valid
             self._all_stats_table = ((ids, ptrs), DeviceTable(rows, device),
-                                     stats_launch_blocks(int(rows['n_valid'].max())), bool(np.all(rows['grad'] % 16 == 0)))
+                                     stats_launch_blocks(int(rows['n_valid'].max())), bool(np.all(rows['grad'] % 16 == 0)),
+                                     all(c.shard.is_cuda for c in chunks)
+                                     and keep_grads_cached(rows, dtype_code(chunks[0].chunk_dtype)))
         return self._all_stats_table[1:]
 
     def _step_on_device(self, source) -> bool:
@@ -562,20 +564,20 @@ class ElixirOptimizer(torch.optim.Optimizer):
         kind, first_slot = source
         early = False
         if kind == 'launch':
-            table, bpc, aligned = self._all_chunks_stats_table(device)
+            table, bpc, aligned, cached = self._all_chunks_stats_table(device)
             partials = eng.partials_buffer(n * bpc)
             stats_args = (table.ptr, n, dtype_code(chunks[0].chunk_dtype), bpc, partials, not aligned)
             keep = (table, eng.partials)
             if not self.graph_step and self.kernel_events is None:
                 # the stats launch needs nothing of what follows: it goes out first, and the host prepares
                 # the rest of the step (tables, control block) while the device reads the gradients
-                _abi.grad_partials_mt(*stats_args, main.cuda_stream)
+                _abi.grad_partials_mt(*stats_args, main.cuda_stream, keep_cached=cached)
                 early = True
         else:
             arena = StatsArena.get(chunks[0].shard_device)
             for event in {c._stats_event for c in chunks if c._stats_event is not None}:
                 main.wait_event(event)    # the landings may have run on another stream
-            bpc, partials, stats_args, keep = 1, arena.ptr(first_slot), None, (arena, )
+            bpc, partials, stats_args, keep, cached = 1, arena.ptr(first_slot), None, (arena, ), False
         inner.prepare_step(upload=False)
         prep = inner._prepared
         if prep is None or prep.dplan.rows is None or len(prep.hyper_host) > _abi.max_ctl_hypers():
@@ -589,7 +591,7 @@ class ElixirOptimizer(torch.optim.Optimizer):
             stream = torch.cuda.current_stream(device).cuda_stream
             with self._timed('stats' if stats_args is not None else 'decide'):
                 if stats_args is not None and not early:
-                    _abi.grad_partials_mt(*stats_args, stream)
+                    _abi.grad_partials_mt(*stats_args, stream, keep_cached=cached)
                 _abi.finish_decide(partials, n, bpc, eng.d_stats, eng.ctl.data_ptr(), eng.d_hypers, eng.max_hypers,
                                    eng.d_decision, eng.report.data_ptr(), eng.d_counter, stream)
             with self._timed('update'):

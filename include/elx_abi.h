@@ -47,10 +47,16 @@ enum {
     ELX_E_SIZE = -7      /* a count is zero, out of its allowed range, or exceeds what a launch can address */
 };
 
-/* flags of elx_adam_step_mt and elx_writeback_mt */
+/* flags of the update, writeback and stats launches */
 enum {
-    ELX_FLAG_SCALAR_ONLY = 1u    /* take the element-by-element path for every tile (set by the host when
+    ELX_FLAG_SCALAR_ONLY = 1u,   /* take the element-by-element path for every tile (set by the host when
                                     elx_check_tables reports base pointers that are not 16-byte aligned) */
+    ELX_FLAG_KEEP_CACHED = 2u    /* stats launches only: read the gradients with ordinary loads instead of
+                                    non-temporal ones, so that they stay in the memory-side cache (256 MiB)
+                                    for the update launch that reads them next.  Pays when all gradients of
+                                    the launch fit that cache (2-5 % of the step at 64-256 MiB); a larger
+                                    set is read faster without it (the stats pass of a 2.6 GB set is 16 %
+                                    slower with it).  Results do not depend on it */
 };
 
 /*
@@ -200,16 +206,18 @@ int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *
  *   d_partials  workspace of n_chunks * blocks_per_chunk ElxStats records (contents ignored)
  *   d_stats     n_chunks results; the reduction order is fixed, so results are reproducible
  *   blocks_per_chunk  1..1024
+ *   flags       0, ELX_FLAG_SCALAR_ONLY (gradient bases not 16-byte aligned), ELX_FLAG_KEEP_CACHED, or both;
+ *               any other bit: ELX_E_RANGE
  */
 int elx_grad_stats_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
-                      ElxStats *d_partials, ElxStats *d_stats, int scalar_only, void *stream);
+                      ElxStats *d_partials, ElxStats *d_stats, int flags, void *stream);
 
 /*
  * The first launch of elx_grad_stats_mt alone: n_chunks * blocks_per_chunk partials, chunk by chunk, left
  * for elx_finish_decide (or any fold of the caller's) to reduce.
  */
 int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
-                         ElxStats *d_partials, int scalar_only, void *stream);
+                         ElxStats *d_partials, int flags, void *stream);
 
 /*
  * The fold of the partials and elx_decide in one launch whose arguments do not change from step to step:
@@ -249,7 +257,7 @@ uint32_t elx_max_ctl_hypers(void);
  *     the last call's partials, and every record a call reads it has written first.
  */
 int elx_grad_stats_mt_static(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
-                             ElxStats *d_stats, int scalar_only, void *stream);
+                             ElxStats *d_stats, int flags, void *stream);
 
 /* Capacity, in ElxStats records, of the fixed partials array of elx_grad_stats_mt_static. */
 uint32_t elx_static_partials(void);

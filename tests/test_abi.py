@@ -134,6 +134,11 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_grad_partials_mt(None, 1, _abi.ELX_F16, 1, 1, 0, None) == -1
     assert lib.elx_grad_partials_mt(1, 1, _abi.ELX_F16, 1025, 1, 0, None) == -7
     assert lib.elx_grad_partials_mt(1, 1, 9, 1, 1, 0, None) == -2
+    # flags of the stats launches: scalar-only (1), keep-cached (2) or both; anything else is refused
+    assert lib.elx_grad_partials_mt(1, 1, _abi.ELX_F16, 1, 1, 4, None) == -4
+    assert lib.elx_grad_stats_mt(1, 1, _abi.ELX_F16, 1, 1, 1, 8, None) == -4
+    assert lib.elx_grad_stats_mt_static(8, 1, _abi.ELX_F16, 1, 8, 4, None) == -4
+    assert _abi.stats_flags(True, True) == 3 and _abi.stats_flags(False, True) == _abi.ELX_FLAG_KEEP_CACHED == 2
     assert lib.elx_max_ctl_hypers() == 64
     assert lib.elx_finish_decide(None, 1, 1, 8, 8, 8, 1, 8, None, 8, None) == -1
     assert lib.elx_finish_decide(8, 1, 1, 8, None, 8, 1, 8, None, 8, None) == -1            # no control block

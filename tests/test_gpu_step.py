@@ -15,7 +15,7 @@ import torch
 import elixir_amd as ea
 from elixir_amd import _abi
 from elixir_amd import shapes as S
-from elixir_amd.chunk import run_grad_stats
+from elixir_amd.chunk import DeviceTable, run_grad_stats
 from oracle import oracle as O
 
 from helpers import (CODE, assert_close_f32, build_workload, compare_state, from_bits, refresh_oracle_grads, seeds, to_np,
@@ -62,6 +62,50 @@ def test_stats_matches_oracle(oracle, dtype, n):
     assert flag == oracle.overflow(xn, CODE[dtype]) == False
     want = oracle.sumsq(xn, CODE[dtype])
     assert abs(sumsq - want) <= 1e-6 * want, (sumsq, want)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+def test_stats_load_policy_does_not_change_the_records(oracle, dtype):
+    """The stats launches read with non-temporal loads or, for a set that fits the memory-side cache
+    (ELX_FLAG_KEEP_CACHED), with ordinary ones: the same records bit for bit, for the two-launch entry
+    point, the partials-only one and the one with the library's own workspace, aligned or not."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(17)
+    sizes = [1 << 20, 70001, 5, 300000]
+    bufs = [(torch.randn(n + 8, generator=g, device=DEV) * 2.0).to(dtype) for n in sizes]
+    bufs[2][1] = float('inf')    # inside the valid part of the third buffer at either shift
+    stream = torch.cuda.current_stream().cuda_stream
+    item = _abi.STATS_DTYPE.itemsize
+    for shift in (0, 1):    # 1: bases off the 16-byte grid -> element-by-element path
+        rows = np.zeros(len(sizes), dtype=_abi.CHUNK_DTYPE)
+        for i, (b, n) in enumerate(zip(bufs, sizes)):
+            rows[i]['grad'] = b.data_ptr() + shift * b.element_size()
+            rows[i]['n_alloc'] = n
+            rows[i]['n_valid'] = n - 3
+        table = DeviceTable(rows, torch.device(DEV))
+        bpc = 64
+        got = {}
+        for keep in (False, True):
+            partials = torch.zeros(len(sizes) * bpc * item, dtype=torch.uint8, device=DEV)
+            stats = torch.zeros(len(sizes) * item, dtype=torch.uint8, device=DEV)
+            _abi.grad_stats_mt(table.ptr, len(sizes), CODE[dtype], bpc, partials.data_ptr(), stats.data_ptr(), bool(shift),
+                               stream, keep_cached=keep)
+            only = torch.zeros_like(partials)
+            _abi.grad_partials_mt(table.ptr, len(sizes), CODE[dtype], bpc, only.data_ptr(), bool(shift), stream,
+                                  keep_cached=keep)
+            fixed = torch.zeros_like(stats)
+            _abi.grad_stats_mt_static(table.ptr, len(sizes), CODE[dtype], bpc, fixed.data_ptr(), bool(shift), stream,
+                                      keep_cached=keep)
+            torch.cuda.synchronize()
+            assert torch.equal(partials, only) and torch.equal(stats, fixed)
+            got[keep] = (partials.cpu().numpy().copy(), stats.cpu().numpy().view(_abi.STATS_DTYPE).copy())
+        assert np.array_equal(got[False][0], got[True][0])
+        assert np.array_equal(got[False][1].view(np.uint8), got[True][1].view(np.uint8))
+        rec = got[True][1]
+        assert list(rec['overflow']) == [0, 0, 1, 0]
+        for i in (0, 1, 3):
+            want = oracle.sumsq(to_np(bufs[i])[shift:shift + sizes[i] - 3], CODE[dtype])
+            assert abs(float(rec['sumsq'][i]) - want) <= 1e-6 * want
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
