@@ -401,7 +401,8 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 c.optim_update()
         if not gpu_chunks:
             return
-        if self._wb_table is None:
+        key = tuple((c.shard.data_ptr(), c.paired_chunk.shard.data_ptr()) for c in gpu_chunks)
+        if self._wb_table is None or self._wb_table[0] != key:
             tile = _abi.tile_elems()
             rows = np.zeros(len(gpu_chunks), dtype=_abi.CHUNK_DTYPE)
             tiles = 0
@@ -419,9 +420,9 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 tiles += (c.shard_size + tile - 1) // tile
             code = dtype_code(gpu_chunks[0].chunk_dtype)
             info = _abi.check_tables(rows, None, 0, code, code)
-            self._wb_table = (DeviceTable(rows, gpu_chunks[0].shard_device), info, code,
+            self._wb_table = (key, DeviceTable(rows, gpu_chunks[0].shard_device), info, code,
                               max(c.shard_size for c in gpu_chunks))
-        table, info, code, max_elems = self._wb_table
+        _, table, info, code, max_elems = self._wb_table
         stream = torch.cuda.current_stream(table.dev.device).cuda_stream
         _abi.writeback_mt(table.ptr, len(table), code, max_elems, info.aligned, stream)
         for c in gpu_chunks:
@@ -434,7 +435,7 @@ class ElixirOptimizer(torch.optim.Optimizer):
         if not pending:
             return None
         device = kernel_device(c.shard for c in pending)
-        ids = tuple(c.chunk_id for c in pending)
+        ids = tuple((c.chunk_id, c.shard.data_ptr()) for c in pending)    # the table holds addresses
         if self._stats_table is None or self._stats_table[0] != ids:
             rows = np.zeros(len(pending), dtype=_abi.CHUNK_DTYPE)
             for i, c in enumerate(pending):
