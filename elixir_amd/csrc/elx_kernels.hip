@@ -372,10 +372,8 @@ static_assert(sizeof(ElxChunk) == 72, "load_chunk_row reads nine 64-bit words");
 // enqueued before the host knows whether the step happens.  They arrive with the hyper record the
 // tile loads anyway; on a skip the tile only refreshes its low-precision copy.
 template <int GD, int LD, bool GATED>
-__global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks,
-                                                          const ElxSeg *__restrict__ segs,
-                                                          const ElxHyper *__restrict__ hypers, Unscale us,
-                                                          uint32_t scalar_only) {
+__device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chunks, const ElxSeg *__restrict__ segs,
+                                               const ElxHyper *__restrict__ hypers, Unscale us, uint32_t scalar_only) {
     // 2-D grid (tiles, records): blockIdx.y names the record, blockIdx.x the tile; nothing is looked
     // up, and workgroups beyond a record's last tile exit
     const uint32_t ci = blockIdx.y, local_tile = blockIdx.x;
@@ -474,6 +472,34 @@ __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__rest
             s = mid + 1;
     }
     tile_scalar<GD, LD, GATED>(c, base, tile_n, s, segs, hypers, us, false);
+}
+
+template <int GD, int LD, bool GATED>
+__global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks,
+                                                          const ElxSeg *__restrict__ segs,
+                                                          const ElxHyper *__restrict__ hypers, Unscale us,
+                                                          uint32_t scalar_only) {
+    adam_step_tile<GD, LD, GATED>(chunks, segs, hypers, us, scalar_only);
+}
+
+// A handful of hyper records travel in the arguments of the launch that uses them.
+constexpr uint32_t kMaxArgHypers = 32;
+struct HyperPack {
+    ElxHyper h[kMaxArgHypers];
+};
+static_assert(offsetof(HyperPack, h) == 0, "the records start at offset 0 of the argument segment");
+
+// The update launch of a host-decided or standalone step whose hyper records fit its own arguments:
+// the table the tiles read is the argument segment itself, so no launch has to fill a table first.
+template <int GD, int LD>
+__global__ __launch_bounds__(kWave) void adam_step_args_kernel(HyperPack pack, const ElxChunk *__restrict__ chunks,
+                                                               const ElxSeg *__restrict__ segs, Unscale us,
+                                                               uint32_t scalar_only) {
+    // `pack` is the first argument: the records are read where they lie (indexing the by-value
+    // aggregate would copy it to private memory first)
+    typedef const ElxHyper __attribute__((address_space(4))) *kernarg_hypers;
+    const ElxHyper *hypers = (const ElxHyper *)(kernarg_hypers)__builtin_amdgcn_kernarg_segment_ptr();
+    adam_step_tile<GD, LD, false>(chunks, segs, hypers, us, scalar_only);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1061,11 +1087,6 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
 // Hyper records from the kernel arguments into the device table of an update launch: a handful of
 // records reach the device inside the launch packet itself, without a staging buffer and a copy to
 // order and to keep alive.
-constexpr uint32_t kMaxArgHypers = 32;
-struct HyperPack {
-    ElxHyper h[kMaxArgHypers];
-};
-
 __global__ __launch_bounds__(kWave) void put_hypers_kernel(HyperPack pack, uint32_t n_words, uint32_t *__restrict__ dst) {
     // the pack is read where it lies, in the argument segment (indexing a by-value aggregate with the lane
     // number would copy it to private memory first)
@@ -1073,7 +1094,6 @@ __global__ __launch_bounds__(kWave) void put_hypers_kernel(HyperPack pack, uint3
     kernarg_words src = (kernarg_words)__builtin_amdgcn_kernarg_segment_ptr();
     for (uint32_t i = threadIdx.x; i < n_words; i += kWave) dst[i] = src[i];
 }
-static_assert(offsetof(HyperPack, h) == 0, "the records start at offset 0 of the argument segment");
 
 // ---------------------------------------------------------------------------------------------
 // host side of the ABI
@@ -1089,6 +1109,23 @@ bool exact_reciprocal(float s) {
     __builtin_memcpy(&u, &s, 4);
     const uint32_t exp = (u >> 23) & 0xFFu, man = u & 0x7FFFFFu;
     return (u >> 31) == 0 && man == 0 && exp >= 1 && exp <= 252;
+}
+
+// How the update launch divides by div_scale (the div_scale of optimizer.py:216; <= 0: not at all).
+Unscale unscale_of(float div_scale) {
+    Unscale us;
+    us.div_scale = div_scale;
+    us.inv_scale = 1.0f;
+    us.mode = kDivNone;
+    if (div_scale > 0.0f) {
+        if (exact_reciprocal(div_scale)) {
+            us.mode = kDivMulInv;
+            us.inv_scale = 1.0f / div_scale;
+        } else {
+            us.mode = kDivTrue;
+        }
+    }
+    return us;
 }
 
 // dynamic LDS bytes that let exactly `blocks_per_cu` update workgroups share a compute unit
@@ -1118,6 +1155,29 @@ int dispatch_step(int gd, int ld, uint32_t lds, hipStream_t st, const ElxChunk *
 #define ELX_CASE(G, L)                                                                                   \
     if (gd == G && ld == L)                                                                              \
         return launch_step<G, L>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, scalar_only);
+    ELX_CASE(ELX_F32, ELX_NONE)
+    ELX_CASE(ELX_F32, ELX_F32)
+    ELX_CASE(ELX_F16, ELX_NONE)
+    ELX_CASE(ELX_F16, ELX_F16)
+    ELX_CASE(ELX_BF16, ELX_NONE)
+    ELX_CASE(ELX_BF16, ELX_BF16)
+#undef ELX_CASE
+    return ELX_E_DTYPE;
+}
+
+template <int GD, int LD>
+int launch_step_args(uint32_t lds, hipStream_t st, const HyperPack &pack, const ElxChunk *chunks, uint32_t n_chunks,
+                     const ElxSeg *segs, uint32_t grid_tiles, Unscale us, uint32_t scalar_only) {
+    hipLaunchKernelGGL((adam_step_args_kernel<GD, LD>), dim3(grid_tiles, n_chunks), dim3(kWave), lds, st, pack, chunks,
+                       segs, us, scalar_only);
+    return (int)hipGetLastError();
+}
+
+int dispatch_step_args(int gd, int ld, uint32_t lds, hipStream_t st, const HyperPack &pack, const ElxChunk *chunks,
+                       uint32_t n_chunks, const ElxSeg *segs, uint32_t grid_tiles, Unscale us, uint32_t scalar_only) {
+#define ELX_CASE(G, L)                                                                                   \
+    if (gd == G && ld == L)                                                                              \
+        return launch_step_args<G, L>(lds, st, pack, chunks, n_chunks, segs, grid_tiles, us, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -1355,20 +1415,8 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
     uint32_t lds = 0;
     if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
         return rc;
-    Unscale us;
-    us.div_scale = div_scale;
-    us.inv_scale = 1.0f;
-    us.mode = kDivNone;
-    if (div_scale > 0.0f) {
-        if (exact_reciprocal(div_scale)) {
-            us.mode = kDivMulInv;
-            us.inv_scale = 1.0f / div_scale;
-        } else {
-            us.mode = kDivTrue;
-        }
-    }
     return dispatch_step(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, d_chunks, n_chunks, d_segs, d_hypers,
-                         grid_tiles_per_chunk, us, false, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+                         grid_tiles_per_chunk, unscale_of(div_scale), false, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
 int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream);
@@ -1388,6 +1436,12 @@ int elx_adam_step_put_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxS
     uint32_t lds = 0;
     if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
         return rc;
+    if (n_hypers <= kMaxArgHypers) {    // the records ride the update launch itself; d_hypers is not written
+        HyperPack pack = {};
+        __builtin_memcpy(pack.h, h_hypers, n_hypers * sizeof(ElxHyper));
+        return dispatch_step_args(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, pack, d_chunks, n_chunks, d_segs,
+                                  grid_tiles_per_chunk, unscale_of(div_scale), (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+    }
     if (int rc = elx_put_hypers(h_hypers, n_hypers, d_hypers, stream)) return rc;
     return elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, total_tiles, grid_tiles_per_chunk,
                             div_scale, grad_dtype, lowp_dtype, flags, blocks_per_cu, stream);

@@ -299,10 +299,12 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
 int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream);
 
 /*
- * elx_put_hypers followed by elx_adam_step_mt on the same table, in one call (the two launches go out
- * back to back, which matters for steps of a few tens of microseconds): the whole of
- * `self.optim.step(div_scale=...)` (optimizer.py:216) for a host-decided or standalone step.  The
- * arguments are those of the two functions; nothing is launched when the update would be refused.
+ * The whole of `self.optim.step(div_scale=...)` (optimizer.py:216) for a host-decided or standalone step,
+ * in one call: the hyper records come from HOST memory (h_hypers, reusable as soon as the call returns).
+ * Up to 32 records travel in the arguments of the update launch itself, which reads them there: one
+ * launch, and d_hypers is NOT written.  More than 32: elx_put_hypers into d_hypers followed by
+ * elx_adam_step_mt on that table, the launches going out back to back.  The other arguments are those
+ * of elx_adam_step_mt; nothing is launched when the update would be refused.
  */
 int elx_adam_step_put_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *d_segs, uint32_t n_segs,
                          const ElxHyper *h_hypers, ElxHyper *d_hypers, uint32_t n_hypers, uint64_t total_tiles,

@@ -209,6 +209,37 @@ def test_reduce_chunk_lands_and_flags(oracle, dtype, sync):
         assert pc.overflow is (i == 1)
 
 
+def test_reduce_chunk_norm_identity_of_the_reference_test():
+    """test/chunk/test_chunk.py:14-73 on one process: four tensors (2x64, 2x2x128, 128, 4x32) packed into
+    a 1024-element fp32 chunk keep their values; after ``reduce_chunk`` of the payload the chunk's
+    ``l2_norm`` is ``payload.float().norm(2)**2`` (the reference's assertion, ``torch.allclose`` defaults)."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(3)
+    tensors = [torch.randn(*shape, generator=g, device=DEV) for shape in ((2, 64), (2, 2, 128), (128, ), (4, 32))]
+    copies = [t.clone() for t in tensors]
+    chunk = ea.Chunk(None, 1024, torch.float, None)
+    chunk.l2_norm_flag = True
+    assert chunk.chunk_size == 1024 and chunk.chunk_dtype == torch.float and chunk.shard_size == 1024
+    for t in tensors:
+        chunk.append_tensor(t)
+    for t, c in zip(tensors, copies):    # packed into the chunk, values and shapes kept
+        assert torch.equal(t, c)
+    chunk.close_chunk()
+    assert chunk.is_replica is False and chunk.utilized_size == 128 + 512 + 128 + 128
+    for on_gpu, on_cpu in zip(copies, chunk.get_cpu_copy()):
+        assert on_cpu.device.type == 'cpu' and torch.equal(on_gpu.cpu(), on_cpu)
+    payload = chunk.shard.clone()    # what a gather hands out and backward fills: here the values themselves
+    norm = payload.float().norm(2)**2
+    chunk.reduce_chunk(payload)
+    assert chunk.is_replica is False and chunk.overflow is False
+    assert torch.allclose(norm, torch.tensor([chunk.l2_norm], device=DEV))
+    # the flag follows the payload: one inf among the valid elements
+    payload[300] = float('inf')
+    chunk.invalidate_stats()
+    chunk.reduce_chunk(payload)
+    assert chunk.overflow is True
+
+
 def test_fused_landing_then_step_equals_plain_landing_then_step(oracle):
     """The step after a fused landing launches no stats pass and gives the same bits."""
     dtype = torch.float16
