@@ -240,7 +240,8 @@ def adam_step_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, d_hyper
 def adam_step_put_mt(d_chunks: int, n_chunks: int, d_segs: int, n_segs: int, hyper_host: np.ndarray, d_hypers: int,
                      info: TableInfo, div_scale: float, grad_dtype: int, lowp_dtype: int, blocks_per_cu: int,
                      stream: int) -> None:
-    """``put_hypers`` + ``adam_step_mt`` in one call: the two launches go out back to back."""
+    """The update with its hyper records taken from host memory: up to 32 ride in the arguments of the
+    update launch itself (``d_hypers`` is then not written), more go through ``put_hypers`` into ``d_hypers``."""
     assert hyper_host.dtype == HYPER_DTYPE
     check('elx_adam_step_put_mt',
           load().elx_adam_step_put_mt(d_chunks, n_chunks, d_segs, n_segs, _np_ptr(hyper_host), d_hypers, len(hyper_host),

@@ -807,7 +807,7 @@ def _offset_view(data: torch.Tensor, offset: int) -> torch.Tensor:
 
 
 @pytest.mark.parametrize('gdtype', [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize('how', ['host', 'gated', 'gated_skip'])
+@pytest.mark.parametrize('how', ['host', 'host_args', 'host_put', 'gated', 'gated_skip'])
 def test_update_on_misaligned_buffers(oracle, gdtype, how):
     """One misaligned base pointer makes the host pass ELX_FLAG_SCALAR_ONLY and every tile of the
     update launch takes the element-by-element path (optimizer.py:115-124 hands the inner optimizer
@@ -815,7 +815,9 @@ def test_update_on_misaligned_buffers(oracle, gdtype, how):
     element offsets, with a segment boundary inside a tile, a gap no segment covers, a padding tail
     that starts inside a tile, two hyper records (decoupled decay and L2) and a divisor that is not a
     power of two: identical bits to the oracle and to the same launch on aligned copies; decided by
-    the host, decided on the device, and skipped on the device."""
+    the host (hyper records in a device table; in the arguments of the update launch, which leaves the
+    table untouched; 40 records, which go through the table after all), decided on the device, and
+    skipped on the device."""
     from elixir_amd.chunk import DeviceTable
     from elixir_amd.hybrid_adam import make_hyper_record
     code = CODE[gdtype]
@@ -863,6 +865,16 @@ def test_update_on_misaligned_buffers(oracle, gdtype, how):
         if how == 'host':
             _abi.adam_step_mt(d_rows.ptr, len(rows), d_segs.ptr, len(segs), d_hyp.ptr, len(hyper_host), info, div, code,
                               code, 0, stream)
+        elif how in ('host_args', 'host_put'):
+            records = hyper_host if how == 'host_args' else np.concatenate([hyper_host] + [hyper_host[:1]] * 38)
+            table = torch.full((records.nbytes, ), 0xA5, dtype=torch.uint8, device=DEV)
+            _abi.adam_step_put_mt(d_rows.ptr, len(rows), d_segs.ptr, len(segs), records, table.data_ptr(), info, div,
+                                  code, code, 0, stream)
+            torch.cuda.synchronize()
+            if how == 'host_args':    # the records rode in the launch arguments
+                assert bool((table == 0xA5).all())
+            else:
+                assert np.array_equal(table.cpu().numpy(), records.view(np.uint8).reshape(-1))
         else:
             stats = np.zeros(1, dtype=_abi.STATS_DTYPE)
             stats['overflow'] = 1 if how == 'gated_skip' else 0
