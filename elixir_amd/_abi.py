@@ -294,8 +294,10 @@ def land_workspace_records(n_rows: int, blocks_per_row: int, n_slots: int = 0) -
 
 def land_grads_mt(d_rows: int, n_rows: int, src_dtype: int, dst_dtype: int, mul: float, blocks_per_row: int,
                   d_partials: int, d_stats: int, aligned: bool, stream: int, blocks_per_cu: int = 0,
-                  d_slot_offsets: int = 0, n_slots: int = 0) -> None:
-    flags = (0 if aligned else ELX_FLAG_SCALAR_ONLY) | ((blocks_per_cu & 0xFF) << 8)
+                  d_slot_offsets: int = 0, n_slots: int = 0, keep_cached: bool = False) -> None:
+    """``keep_cached``: ordinary instead of non-temporal stores, for a destination that fits the
+    memory-side cache and is read by the optimizer step soon after."""
+    flags = stats_flags(not aligned, keep_cached) | ((blocks_per_cu & 0xFF) << 8)
     check('elx_land_grads_mt',
           load().elx_land_grads_mt(d_rows, n_rows, d_slot_offsets or None, n_slots, src_dtype, dst_dtype, mul,
                                    blocks_per_row, d_partials, d_stats, flags, stream))

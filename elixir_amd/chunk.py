@@ -97,7 +97,9 @@ def stats_launch_blocks(n_valid_max: int) -> int:
 # The memory-side cache of the GPU holds 256 MiB.  A gradient set below this size is read by the stats pass
 # with ordinary loads, so that the update launch right behind it finds the gradients there (step time
 # -2 % to -5 % between 64 and 256 MiB of gradients); larger sets are read with non-temporal loads, which
-# stream faster (a 2.6 GB set: 0.39 against 0.45 ms).
+# stream faster (a 2.6 GB set: 0.39 against 0.45 ms).  A landing launch follows the same rule with its
+# stores (GPT-2 small: landing 0.145 -> 0.139 ms, the step behind it 0.573 -> 0.556 ms; the 2.95 GB of
+# OPT-1.3B: landing 0.97 -> 1.00 ms with ordinary stores, so they stay non-temporal).
 KEEP_GRADS_CACHED_BELOW = 256 << 20
 
 
@@ -256,7 +258,8 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
         cached = ws['land_table'] = DeviceTable(rows, device)
     stream = torch.cuda.current_stream(device).cuda_stream
     _abi.land_grads_mt(cached.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
-                       arena.ptr(chunks[0]._stats_slot), aligned, stream, LAND_BLOCKS_PER_CU)
+                       arena.ptr(chunks[0]._stats_slot), aligned, stream, LAND_BLOCKS_PER_CU,
+                       keep_cached=keep_grads_cached(rows, dst_code))
     landed = torch.cuda.Event()
     landed.record(torch.cuda.current_stream(device))
     for c in chunks:
@@ -361,7 +364,8 @@ def land_tensors(chunks: List['Chunk'], grad_of, mul: float = 1.0) -> None:
     stream = torch.cuda.current_stream(device).cuda_stream
     _abi.land_grads_mt(table.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
                        arena.ptr(chunks[0]._stats_slot), True, stream, LAND_BLOCKS_PER_CU,
-                       d_slot_offsets=offsets.data_ptr(), n_slots=len(chunks))
+                       d_slot_offsets=offsets.data_ptr(), n_slots=len(chunks),
+                       keep_cached=sum(c.n_valid for c in chunks) * dsize <= KEEP_GRADS_CACHED_BELOW)
     landed = torch.cuda.Event()
     landed.record(torch.cuda.current_stream(device))
     for c in chunks:

@@ -735,8 +735,10 @@ struct LaneIo<16> {
     static __device__ __forceinline__ raw load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
         return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxLoad);
     }
+    // KEEP: an ordinary store, which leaves the line in the memory-side cache for a launch that reads it soon
+    template <bool KEEP>
     static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, raw x) {
-        __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)off, 0, kAuxStore);
+        __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)off, 0, KEEP ? 0 : kAuxStore);
     }
 };
 template <>
@@ -745,12 +747,13 @@ struct LaneIo<8> {
     static __device__ __forceinline__ raw load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
         return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kAuxLoad);
     }
+    template <bool KEEP>
     static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, raw x) {
-        __builtin_amdgcn_raw_buffer_store_b64(x, r, (int)off, 0, kAuxStore);
+        __builtin_amdgcn_raw_buffer_store_b64(x, r, (int)off, 0, KEEP ? 0 : kAuxStore);
     }
 };
 
-template <int SD, int DD, bool MUL>
+template <int SD, int DD, bool MUL, bool KEEP>
 __global__ __launch_bounds__(kWave) void land_grads_kernel(const ElxChunk *__restrict__ rows, float mul,
                                                            ElxStats *__restrict__ partials, uint32_t scalar_only) {
     typedef typename Elem<SD>::scalar sscalar;
@@ -787,8 +790,8 @@ __global__ __launch_bounds__(kWave) void land_grads_kernel(const ElxChunk *__res
                 dvec D;
 #pragma unroll
                 for (uint32_t k = 0; k < kEpl; ++k) D[k] = land_elem<SD, DD, MUL>(S[u][k], mul, F[u][k]);
-                LaneIo<kDstBytes>::store(dr, (threadIdx.x + u * kWave) * (uint32_t)kDstBytes,
-                                         __builtin_bit_cast(typename LaneIo<kDstBytes>::raw, D));
+                LaneIo<kDstBytes>::template store<KEEP>(dr, (threadIdx.x + u * kWave) * (uint32_t)kDstBytes,
+                                                        __builtin_bit_cast(typename LaneIo<kDstBytes>::raw, D));
             }
             if (base < nv) {    // wave-uniform: the tile lies inside the valid head
 #pragma unroll
@@ -1211,6 +1214,21 @@ int scratch_of_current_device(void **out) {
 
 }    // namespace
 
+template <int S, int D>
+static int launch_land(bool scaled, bool keep, dim3 grid, uint32_t lds, hipStream_t st, const ElxChunk *d_rows, float mul,
+                       ElxStats *d_partials, uint32_t scalar_only) {
+    const dim3 block(kWave);
+    if (scaled && keep)
+        hipLaunchKernelGGL((land_grads_kernel<S, D, true, true>), grid, block, lds, st, d_rows, mul, d_partials, scalar_only);
+    else if (scaled)
+        hipLaunchKernelGGL((land_grads_kernel<S, D, true, false>), grid, block, lds, st, d_rows, mul, d_partials, scalar_only);
+    else if (keep)
+        hipLaunchKernelGGL((land_grads_kernel<S, D, false, true>), grid, block, lds, st, d_rows, mul, d_partials, scalar_only);
+    else
+        hipLaunchKernelGGL((land_grads_kernel<S, D, false, false>), grid, block, lds, st, d_rows, mul, d_partials, scalar_only);
+    return (int)hipGetLastError();
+}
+
 template <int GD>
 static void launch_grad_stats(bool keep, dim3 grid, hipStream_t st, const ElxChunk *d_chunks, uint32_t bpc,
                               ElxStats *d_partials, uint32_t scalar_only) {
@@ -1556,7 +1574,7 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d
     if (n_slots == 0 || n_slots > n_rows) return ELX_E_SIZE;
     if (!(mul == mul) || mul <= 0.0f || mul > 3.0e38f) return ELX_E_RANGE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const dim3 grid(blocks_per_row, n_rows), block(kWave);
+    const dim3 grid(blocks_per_row, n_rows);
     const uint32_t so = (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u;
     uint32_t lds = 0;
     const uint32_t land_default = (src_dtype == ELX_F32 && dst_dtype != ELX_F32) ? kDefaultLandBlocksPerCuNarrowing
@@ -1565,13 +1583,9 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d
     if (rc) return rc;
     rc = ELX_E_DTYPE;
 #define ELX_LAND(S, D)                                                                                       \
-    if (src_dtype == S && dst_dtype == D) {                                                                  \
-        if (mul == 1.0f)                                                                                     \
-            hipLaunchKernelGGL((land_grads_kernel<S, D, false>), grid, block, lds, st, d_rows, mul, d_partials, so); \
-        else                                                                                                 \
-            hipLaunchKernelGGL((land_grads_kernel<S, D, true>), grid, block, lds, st, d_rows, mul, d_partials, so);  \
-        rc = (int)hipGetLastError();                                                                         \
-    }
+    if (src_dtype == S && dst_dtype == D)                                                                    \
+        rc = launch_land<S, D>(mul != 1.0f, (flags & ELX_FLAG_KEEP_CACHED) != 0, grid, lds, st, d_rows, mul,    \
+                               d_partials, so);
     ELX_LAND(ELX_F32, ELX_F32)
     ELX_LAND(ELX_F16, ELX_F16)
     ELX_LAND(ELX_BF16, ELX_BF16)

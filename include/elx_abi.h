@@ -51,12 +51,12 @@ enum {
 enum {
     ELX_FLAG_SCALAR_ONLY = 1u,   /* take the element-by-element path for every tile (set by the host when
                                     elx_check_tables reports base pointers that are not 16-byte aligned) */
-    ELX_FLAG_KEEP_CACHED = 2u    /* stats launches only: read the gradients with ordinary loads instead of
-                                    non-temporal ones, so that they stay in the memory-side cache (256 MiB)
-                                    for the update launch that reads them next.  Pays when all gradients of
-                                    the launch fit that cache (2-5 % of the step at 64-256 MiB); a larger
-                                    set is read faster without it (the stats pass of a 2.6 GB set is 16 %
-                                    slower with it).  Results do not depend on it */
+    ELX_FLAG_KEEP_CACHED = 2u    /* stats and landing launches: touch the gradients with ordinary loads / stores
+                                    instead of non-temporal ones, so that they stay in the memory-side cache
+                                    (256 MiB) for the update launch that reads them next.  Pays when all
+                                    gradients of the launch fit that cache (2-5 % of the step at 64-256 MiB);
+                                    a larger set streams faster without it (the stats pass of a 2.6 GB set is
+                                    16 % slower with it).  Results do not depend on it */
 };
 
 /*
@@ -392,7 +392,10 @@ int elx_grad_stats(const void *grad, int grad_dtype, uint64_t n, uint32_t blocks
  *              records (contents ignored)
  *   d_stats    n_slots results; fixed reduction order
  *   flags      ELX_FLAG_SCALAR_ONLY forces the element-by-element path (rows whose ends are not both
- *              16-byte aligned take it by themselves); bits 8..15: cap on resident workgroups per
+ *              16-byte aligned take it by themselves); ELX_FLAG_KEEP_CACHED writes the destination with
+ *              ordinary instead of non-temporal stores, so that a destination of at most 256 MiB is still
+ *              in the memory-side cache when the optimizer step reads it (a loss on larger ones);
+ *              bits 8..15: cap on resident workgroups per
  *              compute unit, 3..32 (0 = the library default: 10, or 13 when an fp32 payload lands in a
  *              16-bit shard)
  */

@@ -23,8 +23,9 @@ PAIRS = [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16), (torc
          (torch.float32, torch.float16), (torch.float32, torch.bfloat16)]
 
 
-def _land(src: torch.Tensor, dst: torch.Tensor, n_valid: int, mul: float = 1.0, blocks: int = 0):
-    """One row through the C ABI; returns (overflow, sumsq)."""
+def _land(src: torch.Tensor, dst: torch.Tensor, n_valid: int, mul: float = 1.0, blocks: int = 0, keep: bool = False):
+    """One row through the C ABI; returns (overflow, sumsq).  ``keep``: ordinary instead of non-temporal
+    stores (ELX_FLAG_KEEP_CACHED), which must not change anything but the speed."""
     n = dst.numel()
     assert src.numel() == n
     row = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
@@ -37,7 +38,7 @@ def _land(src: torch.Tensor, dst: torch.Tensor, n_valid: int, mul: float = 1.0, 
     aligned = src.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0
     _abi.land_grads_mt(table.ptr, 1, CODE[src.dtype], CODE[dst.dtype], mul, bpr, ws.data_ptr(),
                        ws.data_ptr() + recs * _abi.STATS_DTYPE.itemsize, aligned,
-                       torch.cuda.current_stream().cuda_stream)
+                       torch.cuda.current_stream().cuda_stream, keep_cached=keep)
     rec = ws[recs * _abi.STATS_DTYPE.itemsize:].cpu().numpy().view(_abi.STATS_DTYPE)
     return bool(rec['overflow'][0]), float(rec['sumsq'][0])
 
@@ -50,13 +51,14 @@ def _payload(n, dtype, seed, scale=3.0):
 
 @pytest.mark.parametrize('sd,dd', PAIRS)
 @pytest.mark.parametrize('n', [1, 7, 4095, 4096, 8192 * 4 + 5, (1 << 20) + 3, (1 << 22) + 12345])
-def test_landing_matches_oracle(oracle, sd, dd, n):
+@pytest.mark.parametrize('keep', [False, True])
+def test_landing_matches_oracle(oracle, sd, dd, n, keep):
     src = _payload(n, sd, n)
     nv = max(1, n - n // 5)                       # a padded tail
     if nv < n:
         src[nv:] = float('inf')                   # garbage in the padding: copied, never counted
     dst = torch.full((n,), 7.0, dtype=dd, device=DEV)
-    flag, sumsq = _land(src, dst, nv)
+    flag, sumsq = _land(src, dst, nv, keep=keep)
     want = oracle.land(to_np(src), CODE[sd], CODE[dd])
     got = to_np(dst)
     assert np.array_equal(got.view(np.uint32 if dd == torch.float32 else np.uint16),
@@ -120,7 +122,7 @@ def test_landing_scaled_like_torchs_device_division(oracle, sd, dd, pg):
     want /= pg
     want = want.to(dd)
     dst = torch.zeros(n, dtype=dd, device=DEV)
-    flag, sumsq = _land(src, dst, n, mul=float(np.float32(1.0) / np.float32(pg)))
+    flag, sumsq = _land(src, dst, n, mul=float(np.float32(1.0) / np.float32(pg)), keep=pg % 3 == 0)
     view = torch.int32 if dd == torch.float32 else torch.int16
     assert torch.equal(dst.view(view), want.view(view))
     assert flag is False
