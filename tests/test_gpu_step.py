@@ -680,6 +680,58 @@ def test_random_trajectories_match_oracle(oracle, seed):
             oc.master[:], oc.m[:], oc.v[:], oc.lowp[:] = to_np(fc.shard), to_np(m), to_np(v), to_np(pc.shard)
 
 
+def test_three_hundred_steps_stay_on_the_oracle(oracle):
+    """A long run on a small layout: 300 steps with a learning rate that changes at every step (a
+    warm-up and decay schedule written into the groups, as a scheduler does), the dynamic scaler
+    growing every 25 clean steps and backing off after two overflows in a row (hysteresis 2),
+    overflows injected at steps 40, 41 and 120, the step decided on the device or on the host and
+    the gradients written into the shards or landed by the fused launch in turn.  Scale, skips and
+    step counts are compared at every step, the whole state bit for bit every 20 steps and at the end:
+    nothing that is cached from one step to the next (tables, hyper records, control block) may go stale."""
+    from elixir_amd.chunk import land_chunks
+    dtype = torch.float16
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=91, loss_scale=64.0, weight_decay=0.05,
+                                          initial_scale=64.0, hysteresis=2, growth_interval=25, max_scale=2.0**12)
+    scaler = O.DynamicGradScalerOracle(initial_scale=64.0, min_scale=1, max_scale=2.0**12, hysteresis=2, growth_interval=25)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(92)
+    base_lr = [g['lr'] for g in opt.param_groups]
+    skipped = 0
+    for step in range(300):
+        factor = min(1.0, (step + 1) / 30.0) * (1.0 - step / 400.0)
+        for g, lr0 in zip(opt.param_groups, base_lr):
+            g['lr'] = lr0 * factor
+        for oc in ochunks:
+            for seg in oc.segments:
+                seg.lr = base_lr[0] * factor    # both groups start from the same rate
+        ls = opt.loss_scale
+        payloads = []
+        for pc in module.param_chunks:
+            g = (torch.randn(pc.shard_size, generator=gen, device=DEV) * (1e-3 * ls)).to(dtype)
+            g[pc.utilized_size:] = 0
+            payloads.append(g)
+        if step in (40, 41, 120):
+            payloads[step % len(payloads)][7] = float('inf')
+        opt.gated_step = step % 2 == 0
+        if step % 3 == 0:
+            land_chunks(list(module.param_chunks), payloads)
+        else:
+            for pc, g in zip(module.param_chunks, payloads):
+                pc.shard.copy_(g)
+                pc.invalidate_stats()
+        refresh_oracle_grads(module, ochunks)
+        info = _run_and_compare(module, opt, ochunks, dtype, scaler, tag=f'step {step}')
+        assert info['found_inf'] is (step in (40, 41, 120))
+        skipped += int(info['found_inf'])
+        if step % 20 == 19 or step == 299 or info['found_inf']:
+            assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'step {step}') == 0
+    assert skipped == 3
+    steps_taken = {int(st['step']) for st in opt.optim.state.values()}
+    assert steps_taken == {297}
+    # 64 -> x2 after 25 clean steps, two overflows in a row -> one back-off, later growth capped at 2^12
+    assert opt.loss_scale == float(scaler.scale) and opt.loss_scale <= 2.0**12
+
+
 @pytest.mark.parametrize('beta1', [0.9, 0.5, 0.0])
 @pytest.mark.parametrize('div_scale', [-1.0, 64.0, 48.0])
 @pytest.mark.parametrize('gdtype', [torch.float32, torch.float16, torch.bfloat16])
