@@ -279,6 +279,39 @@ def test_flat_random_hypers_match_oracle(oracle, seed):
                     f'seed {seed} step {step} {name} {gdtype} adamw {adamw} group {grp} div {div}'
 
 
+def test_two_hundred_flat_steps_with_a_schedule_stay_on_the_oracle(oracle):
+    """Standalone HybridAdam over two groups for 200 steps, torch's LambdaLR changing both learning
+    rates at every step, gradients re-allocated at every step (new addresses): the bits of master and
+    moments equal the oracle's after every 25th step and at the end, so neither the cached walk over
+    the parameters nor the records computed one step ahead may lag behind."""
+    sizes, lrs, wds = [40_000, 3_001], [1e-3, 5e-3], [0.1, 0.0]
+    torch.manual_seed(5)
+    params = [torch.nn.Parameter((torch.randn(n) * 0.02).to(DEV)) for n in sizes]
+    host = [(to_np(p.data).copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)) for p, n in zip(params, sizes)]
+    opt = ea.HybridAdam([dict(params=[p], lr=lr, weight_decay=wd) for p, lr, wd in zip(params, lrs, wds)])
+    schedule = lambda k: min(1.0, (k + 1) / 20.0) * 0.995**k
+    sched = torch.optim.lr_scheduler.LambdaLR(opt, schedule)
+    gen = torch.Generator().manual_seed(6)
+    for step in range(1, 201):
+        grads = [(torch.randn(n, generator=gen) * 1e-2 * 8.0).half() for n in sizes]
+        for p, g in zip(params, grads):
+            p.grad_dtype = None
+            p.grad = g.to(DEV)
+        now = [grp['lr'] for grp in opt.param_groups]
+        assert now == [lr * schedule(step - 1) for lr in lrs]
+        opt.step(div_scale=8.0)
+        sched.step()
+        for p, g, lr, wd, (pn, mn, vn) in zip(params, grads, now, wds, host):
+            oracle.adam(to_np(g), O.F16, pn, mn, vn, lr=lr, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=wd, step=step,
+                        adamw_mode=True, div_scale=8.0)
+        if step % 25 == 0:
+            for p, (pn, mn, vn) in zip(params, host):
+                st = opt.state[p]
+                assert st['step'] == step
+                for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
+                    assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32)), f'step {step} {name}'
+
+
 def test_first_step_is_sign_descent():
     """Closed form: with m = v = 0 and step 1, p moves by -lr * g / (|g| + eps) ~ -lr * sign(g)."""
     n = 10000
