@@ -64,6 +64,7 @@ constexpr uint32_t kDefaultBlocksPerCu = 12;           // fp32 gradients (4 KiB 
 constexpr uint32_t kDefaultBlocksPerCuLowp = 13;       // 16-bit gradients (3.5 KiB): one more workgroup pays
 constexpr uint32_t kMinBlocksPerCu = 3;                // keeps the reservation below 64 KiB
 constexpr uint32_t kMaxBlocksPerCu = 32;
+constexpr uint32_t kStatsStreamBlocksPerCu = 3;        // stats workgroups (256 threads) per CU when the set streams from HBM
 
 constexpr int kStatsThreads = 256;
 constexpr int kStatsUnroll = 4;
@@ -1232,12 +1233,20 @@ static int launch_land(bool scaled, bool keep, dim3 grid, uint32_t lds, hipStrea
 template <int GD>
 static void launch_grad_stats(bool keep, dim3 grid, hipStream_t st, const ElxChunk *d_chunks, uint32_t bpc,
                               ElxStats *d_partials, uint32_t scalar_only) {
-    if (keep)
+    if (keep) {
         hipLaunchKernelGGL((grad_stats_kernel<GD, true>), grid, dim3(kStatsThreads), 0, st, d_chunks, bpc, d_partials,
                            scalar_only);
-    else
-        hipLaunchKernelGGL((grad_stats_kernel<GD, false>), grid, dim3(kStatsThreads), 0, st, d_chunks, bpc, d_partials,
+    } else {
+        // A set that streams from HBM is read fastest with a shallow queue, like the update's streams: three
+        // workgroups (twelve wavefronts, 48 KiB of loads in flight) per compute unit instead of the eight that
+        // fit, held there by an LDS reservation no thread touches (-3.5 % on 2.6 and 13.5 GB of gradients;
+        // a set served from the cache wants all eight).
+        // (the kernel's own few bytes of static LDS come on top of the reservation: leave room for them, or
+        // only two workgroups fit and the pass slows down by a fifth)
+        const uint32_t lds = (kLdsPerCu / kStatsStreamBlocksPerCu - 1024u) & ~255u;
+        hipLaunchKernelGGL((grad_stats_kernel<GD, false>), grid, dim3(kStatsThreads), lds, st, d_chunks, bpc, d_partials,
                            scalar_only);
+    }
 }
 
 extern "C" {
