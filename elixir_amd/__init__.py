@@ -7,13 +7,13 @@ ABI declared in ``include/elx_abi.h``; there is no CPU or eager-PyTorch fallback
 """
 from .chunk import Chunk, ChunkFullError, ChunkGroup, TensorInfo, TensorState
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
-from .hybrid_adam import HybridAdam
+from .hybrid_adam import CPUAdam, FusedAdam, HybridAdam
 from .module import (ChunkPlan, ElixirModule, SearchResult, greedy_groups, greedy_search, simple_groups,
                      simple_search)
 from .optimizer import ElixirOptimizer, OptimState, calc_combined_scale
 
 __all__ = [
     'Chunk', 'ChunkFullError', 'ChunkGroup', 'TensorInfo', 'TensorState', 'BaseGradScaler', 'ConstantGradScaler',
-    'DynamicGradScaler', 'HybridAdam', 'ChunkPlan', 'ElixirModule', 'SearchResult', 'greedy_groups', 'greedy_search',
-    'simple_groups', 'simple_search',    'ElixirOptimizer', 'OptimState', 'calc_combined_scale'
+    'DynamicGradScaler', 'HybridAdam', 'FusedAdam', 'CPUAdam', 'ChunkPlan', 'ElixirModule', 'SearchResult', 'greedy_groups', 'greedy_search',
+    'simple_groups', 'simple_search', 'ElixirOptimizer', 'OptimState', 'calc_combined_scale'
 ]

@@ -623,3 +623,48 @@ class HybridAdam(torch.optim.Optimizer):
         dplan = self._device_plan(key, buffers, grad_dtype, grad_code, _abi.ELX_NONE, len(hypers), device)
         return _Prepared(dplan, self._hyper_table(hypers), grad_code, _abi.ELX_NONE, device, [it[0] for it in items],
                          hypers.keys())
+
+
+class FusedAdam(HybridAdam):
+    """The device-only member of the reference's list of optimizers that take ``div_scale``
+    (elixir/wrapper/optimizer.py:19: ``{FusedAdam, CPUAdam, HybridAdam}``).  Constructor and ``step``
+    follow ColossalAI's ``FusedAdam`` as published (its source is not in the reference's tree):
+    ``adamw_mode`` comes before ``weight_decay``, ``amsgrad`` is refused, ``set_grad_none`` is the
+    default of ``zero_grad``; the legacy ``grads`` / ``output_params`` / ``scale`` / ``grad_norms``
+    arguments of ``step`` are refused as they are there.  Same launches as ``HybridAdam``."""
+
+    def __init__(self,
+                 params,
+                 lr: float = 1e-3,
+                 bias_correction: bool = True,
+                 betas: Tuple[float, float] = (0.9, 0.999),
+                 eps: float = 1e-8,
+                 adamw_mode: bool = True,
+                 weight_decay: float = 0.,
+                 amsgrad: bool = False,
+                 set_grad_none: bool = True):
+        if amsgrad:
+            raise RuntimeError('FusedAdam does not support the AMSGrad variant.')
+        super().__init__(params, lr=lr, bias_correction=bias_correction, betas=betas, eps=eps, weight_decay=weight_decay,
+                         adamw_mode=adamw_mode)
+        self.set_grad_none = set_grad_none
+
+    def zero_grad(self, set_to_none: Optional[bool] = None):
+        return super().zero_grad(set_to_none=self.set_grad_none if set_to_none is None else set_to_none)
+
+    def step(self, closure=None, grads=None, output_params=None, scale=None, grad_norms=None, div_scale: float = -1,
+             **kwargs):
+        if any(p is not None for p in (grads, output_params, scale, grad_norms)):
+            raise RuntimeError('FusedAdam has been updated.  Simply initialize it identically to torch.optim.Adam, and '
+                               'call step() with no arguments.')
+        return HybridAdam.step(self, closure, div_scale, **kwargs)
+
+    step.hooked = True    # see HybridAdam.step
+
+
+class CPUAdam(HybridAdam):
+    """The host-side member of the same list: ColossalAI's ``CPUAdam(model_params, lr, bias_correction,
+    betas, eps, weight_decay, adamw_mode, nvme_offload_fraction, nvme_offload_dir)`` with
+    ``step(closure=None, div_scale=-1)`` -- the signature ``HybridAdam`` inherits there.  There is no CPU
+    arithmetic in this package: chunk shards in pinned host memory are updated in place by the same
+    launches over the host link, pageable host memory is refused."""

@@ -43,9 +43,9 @@ from . import _abi
 from .chunk import (Chunk, DeviceTable, StatsArena, dtype_code, keep_grads_cached, kernel_device, launch_grad_stats,
                     read_grad_stats, resolve_pending_stats, stats_launch_blocks)
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
-from .hybrid_adam import HybridAdam
+from .hybrid_adam import CPUAdam, FusedAdam, HybridAdam
 
-_AVAIL_OPTIM_LIST = {HybridAdam}
+_AVAIL_OPTIM_LIST = {FusedAdam, CPUAdam, HybridAdam}
 
 
 class OptimState(Enum):

@@ -1387,6 +1387,34 @@ def test_lr_scheduler_drives_the_wrapped_optimizer(oracle):
     assert opt._opt_called and sched.last_epoch == 3
 
 
+@pytest.mark.parametrize('gated', [True, False])
+@pytest.mark.parametrize('inner_cls', [ea.FusedAdam, ea.CPUAdam])
+def test_the_other_scaled_optimizers_take_the_fused_path(oracle, inner_cls, gated):
+    """optimizer.py:19,211-216: FusedAdam and CPUAdam are handed ``div_scale`` like HybridAdam.  Inside
+    the wrapper they run the same launches: two steps (L2 decay, a loss scale that is not a power of
+    two, decided on the device and on the host), identical bits to the oracle."""
+    dtype = torch.bfloat16
+    module, opt, ochunks = build_workload(tiny_gpt2(), 1 << 16, dtype, seed=51, loss_scale=3.0, weight_decay=0.02,
+                                          adamw_mode=False, inner_cls=inner_cls)
+    assert type(opt.optim) is inner_cls and opt.scaled_optimizer
+    opt.gated_step = gated
+    opt.grad_scaler._scale = np.float32(3.0)    # bf16 modules get the constant scaler: keep 3.0 for both steps
+    gen = torch.Generator(device=DEV).manual_seed(52)
+    for step in range(2):
+        if step:
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * 3e-3
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+                pc.invalidate_stats()
+            refresh_oracle_grads(module, ochunks)
+        info = _run_and_compare(module, opt, ochunks, dtype, O.ConstantGradScalerOracle(3.0), adamw_mode=False,
+                                tag=f'step {step}')
+        assert info['combined_scale'] == 3.0
+        assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'step {step}') == 0
+    assert sorted(set(st['step'] for st in opt.state.values())) == [2]
+
+
 def test_step_over_simple_search_plans(oracle):
     """The chunk plans of the reference's own planner fixture (test/search/test_simple.py:29-42: a
     private, fused chunk of 320 for the tied embedding and five public chunks of 1088): the wrapper

@@ -513,6 +513,47 @@ def test_hybrid_adam_dispatches_step_hooks_itself():
     assert seen == [('pre', (None, 4.0), dict(gated=False, defer_commit=False))]
 
 
+def test_every_optimizer_of_the_references_scaled_list_is_here():
+    """optimizer.py:19 lists the optimizers that may be handed a ``div_scale``: FusedAdam, CPUAdam and
+    HybridAdam.  All three exist with ColossalAI's argument order, count as scaled optimizers inside the
+    wrapper, and keep their step out of torch's profiling wrapper."""
+    import inspect
+    from elixir_amd.optimizer import _AVAIL_OPTIM_LIST
+    assert _AVAIL_OPTIM_LIST == {ea.FusedAdam, ea.CPUAdam, ea.HybridAdam}
+    assert list(inspect.signature(ea.FusedAdam.__init__).parameters)[1:] == [
+        'params', 'lr', 'bias_correction', 'betas', 'eps', 'adamw_mode', 'weight_decay', 'amsgrad', 'set_grad_none']
+    assert list(inspect.signature(ea.FusedAdam.step).parameters)[1:7] == [
+        'closure', 'grads', 'output_params', 'scale', 'grad_norms', 'div_scale']
+    assert list(inspect.signature(ea.CPUAdam.__init__).parameters)[1:10] == [
+        'model_params', 'lr', 'bias_correction', 'betas', 'eps', 'weight_decay', 'adamw_mode', 'nvme_offload_fraction',
+        'nvme_offload_dir']
+    assert list(inspect.signature(ea.CPUAdam.step).parameters)[1:3] == ['closure', 'div_scale']
+    p = nn.Parameter(torch.zeros(4))
+    p.grad = torch.ones(4)
+    # positional use as in ColossalAI: the sixth argument of FusedAdam is adamw_mode, of CPUAdam weight_decay
+    fused = ea.FusedAdam([p], 1e-3, True, (0.9, 0.999), 1e-8, False, 0.1)
+    assert fused.adamw_mode is False and fused.param_groups[0]['weight_decay'] == 0.1
+    cpu = ea.CPUAdam([p], 1e-3, True, (0.9, 0.999), 1e-8, 0.1, False)
+    assert cpu.adamw_mode is False and cpu.param_groups[0]['weight_decay'] == 0.1
+    with pytest.raises(RuntimeError, match='AMSGrad'):
+        ea.FusedAdam([p], amsgrad=True)
+    with pytest.raises(RuntimeError, match='no arguments'):
+        fused.step(grads=[p.grad])
+    for opt in (fused, cpu):
+        assert getattr(type(opt).step, 'hooked', False) and not hasattr(type(opt).step, '__wrapped__')
+        with pytest.raises(RuntimeError, match='GPU'):    # no device here, and no other way to step
+            opt.step(div_scale=2.0)
+    fused.zero_grad()
+    assert p.grad is None
+    p.grad = torch.ones(4)
+    ea.FusedAdam([p], set_grad_none=False).zero_grad()
+    assert p.grad is not None and float(p.grad.sum()) == 0.0
+    for cls in (ea.FusedAdam, ea.CPUAdam):
+        module, _ = _cpu_optimizer(3)
+        wrapped = ea.ElixirOptimizer(module, cls(module.parameters(), lr=1e-3), initial_scale=64)
+        assert wrapped.scaled_optimizer and wrapped._binding is not None
+
+
 def test_chunk_cpu_copy_and_load_tensors():
     a, b = torch.randn(3, 5), torch.randn(7)
     chunk = ea.Chunk(None, 32, torch.float, None, shard_device='cpu', temp_device='cpu')
