@@ -141,7 +141,8 @@ def _np_ptr(a: Optional[np.ndarray]):
 
 
 class TableInfo(tuple):
-    """(total_tiles, max_tiles_per_chunk, all_aligned16) as reported by elx_check_tables."""
+    """(total_tiles, max_tiles_per_chunk, all_aligned16) as reported by elx_check_tables, optionally followed
+    by the caller's choice of store policy for the low-precision copy (``keep_lowp_cached``)."""
     __slots__ = ()
 
     @property
@@ -157,8 +158,16 @@ class TableInfo(tuple):
         return self[2]
 
     @property
+    def keep_lowp_cached(self) -> bool:
+        return len(self) > 3 and bool(self[3])
+
+    def with_keep_lowp_cached(self, keep: bool) -> 'TableInfo':
+        return TableInfo(tuple(self[:3]) + (bool(keep), ))
+
+    @property
     def flags(self) -> int:
-        return 0 if self[2] else ELX_FLAG_SCALAR_ONLY
+        """The ``flags`` argument of the update launches for these tables."""
+        return (0 if self[2] else ELX_FLAG_SCALAR_ONLY) | (ELX_FLAG_KEEP_CACHED if self.keep_lowp_cached else 0)
 
 
 def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, grad_dtype: int,

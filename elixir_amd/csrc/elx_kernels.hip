@@ -129,6 +129,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kAuxLoad = 2;          // nt
 constexpr int kAuxStore = 2 | 16;    // nt | sc1
+constexpr int kAuxStoreKeep = 16;    // sc1
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const void *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
@@ -156,6 +157,17 @@ struct TileIo<u16x4> {
         __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, x), r, (int)off, 0, kAuxStore);
     }
 };
+
+// The low-precision copy of a tile goes out with the streaming policy of the other stores, or (KEEP) at
+// agent scope without the non-temporal hint: such a store is taken in by the memory-side cache, over the
+// gradient it replaces when that is still there, and written back from there later.
+template <bool KEEP, typename V>
+__device__ __forceinline__ void store_lowp_tile(__amdgpu_buffer_rsrc_t r, uint32_t off, V x) {
+    if constexpr (sizeof(V) == 16)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, (int)off, 0, KEEP ? kAuxStoreKeep : kAuxStore);
+    else
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, x), r, (int)off, 0, KEEP ? kAuxStoreKeep : kAuxStore);
+}
 
 // ---------------------------------------------------------------------------------------------
 // the update of one element
@@ -272,7 +284,7 @@ __device__ __forceinline__ void tile_math_flags(const typename Elem<GD>::vec4 (&
 // fused update + writeback
 // ---------------------------------------------------------------------------------------------
 
-template <int LD>
+template <int LD, bool KEEPL>
 __device__ __forceinline__ void store_lowp_vec(const ElxChunk &c, uint64_t base, const f32x4 (&P)[kUnroll]) {
     if constexpr (LD != ELX_NONE) {
         if (!c.lowp_out) return;
@@ -284,13 +296,13 @@ __device__ __forceinline__ void store_lowp_vec(const ElxChunk &c, uint64_t base,
             lvec L;
 #pragma unroll
             for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
-            TileIo<lvec>::store(lr, (threadIdx.x + u * kWave) * sizeof(lvec), L);
+            store_lowp_tile<KEEPL>(lr, (threadIdx.x + u * kWave) * sizeof(lvec), L);
         }
     }
 }
 
 // Whole tile outside the valid head of the shard (padding), or the writeback-only launch.
-template <int LD>
+template <int LD, bool KEEPL>
 __device__ __forceinline__ void tile_refresh_vec(const ElxChunk &c, uint64_t base) {
     if constexpr (LD != ELX_NONE) {
         if (!c.lowp_out) return;
@@ -298,7 +310,7 @@ __device__ __forceinline__ void tile_refresh_vec(const ElxChunk &c, uint64_t bas
         f32x4 P[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) P[u] = TileIo<f32x4>::load(pr, (threadIdx.x + u * kWave) * sizeof(f32x4));
-        store_lowp_vec<LD>(c, base, P);
+        store_lowp_vec<LD, KEEPL>(c, base, P);
     }
 }
 
@@ -372,7 +384,7 @@ static_assert(sizeof(ElxChunk) == 72, "load_chunk_row reads nine 64-bit words");
 // has put them earlier on the same stream) instead of the kernel arguments, so that the launch can be
 // enqueued before the host knows whether the step happens.  They arrive with the hyper record the
 // tile loads anyway; on a skip the tile only refreshes its low-precision copy.
-template <int GD, int LD, bool GATED>
+template <int GD, int LD, bool GATED, bool KEEPL>
 __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chunks, const ElxSeg *__restrict__ segs,
                                                const ElxHyper *__restrict__ hypers, Unscale us, uint32_t scalar_only) {
     // 2-D grid (tiles, records): blockIdx.y names the record, blockIdx.x the tile; nothing is looked
@@ -427,7 +439,7 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
                 us.inv_scale = h.gate_inv;
                 us.mode = (int)(h.gate & 0xFFu);
                 if (h.gate >> 8) {    // the step is skipped: refresh the low-precision copy only
-                    store_lowp_vec<LD>(c, base, P);
+                    store_lowp_vec<LD, KEEPL>(c, base, P);
                     return;
                 }
             }
@@ -444,11 +456,11 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
                 TileIo<f32x4>::store(mr, off, M[u]);
                 TileIo<f32x4>::store(vr, off, V[u]);
             }
-            store_lowp_vec<LD>(c, base, P);
+            store_lowp_vec<LD, KEEPL>(c, base, P);
             return;
         }
         if (!has || sb >= base + kTile) {    // inside the valid head but owned by no segment
-            store_lowp_vec<LD>(c, base, P);
+            store_lowp_vec<LD, KEEPL>(c, base, P);
             return;
         }
         // the tile straddles a segment boundary: redo it element by element below
@@ -459,7 +471,7 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
     const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
     if (base >= c.n_valid) {    // padding inside an update chunk: refresh only
         if (tile_n == kTile && !scalar_only)
-            tile_refresh_vec<LD>(c, base);
+            tile_refresh_vec<LD, KEEPL>(c, base);
         else
             tile_scalar<GD, LD, GATED>(c, base, tile_n, 0, segs, hypers, us, true);
         return;
@@ -475,12 +487,12 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
     tile_scalar<GD, LD, GATED>(c, base, tile_n, s, segs, hypers, us, false);
 }
 
-template <int GD, int LD, bool GATED>
+template <int GD, int LD, bool GATED, bool KEEPL>
 __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks,
                                                           const ElxSeg *__restrict__ segs,
                                                           const ElxHyper *__restrict__ hypers, Unscale us,
                                                           uint32_t scalar_only) {
-    adam_step_tile<GD, LD, GATED>(chunks, segs, hypers, us, scalar_only);
+    adam_step_tile<GD, LD, GATED, KEEPL>(chunks, segs, hypers, us, scalar_only);
 }
 
 // A handful of hyper records travel in the arguments of the launch that uses them.
@@ -492,7 +504,7 @@ static_assert(offsetof(HyperPack, h) == 0, "the records start at offset 0 of the
 
 // The update launch of a host-decided or standalone step whose hyper records fit its own arguments:
 // the table the tiles read is the argument segment itself, so no launch has to fill a table first.
-template <int GD, int LD>
+template <int GD, int LD, bool KEEPL>
 __global__ __launch_bounds__(kWave) void adam_step_args_kernel(HyperPack pack, const ElxChunk *__restrict__ chunks,
                                                                const ElxSeg *__restrict__ segs, Unscale us,
                                                                uint32_t scalar_only) {
@@ -500,7 +512,7 @@ __global__ __launch_bounds__(kWave) void adam_step_args_kernel(HyperPack pack, c
     // aggregate would copy it to private memory first)
     typedef const ElxHyper __attribute__((address_space(4))) *kernarg_hypers;
     const ElxHyper *hypers = (const ElxHyper *)(kernarg_hypers)__builtin_amdgcn_kernarg_segment_ptr();
-    adam_step_tile<GD, LD, false>(chunks, segs, hypers, us, scalar_only);
+    adam_step_tile<GD, LD, false, KEEPL>(chunks, segs, hypers, us, scalar_only);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1142,23 +1154,30 @@ int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes, uint32_t 
 
 template <int GD, int LD>
 int launch_step(uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks, const ElxSeg *segs,
-                const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, uint32_t scalar_only) {
+                const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, bool keep, uint32_t scalar_only) {
     const dim3 grid(grid_tiles, n_chunks);
-    if (gated)
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+    constexpr bool kHasLowp = LD != ELX_NONE;    // without a low-precision copy there is no policy to choose
+    if (gated && keep && kHasLowp)
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true, kHasLowp>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+                           scalar_only);
+    else if (gated)
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true, false>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+                           scalar_only);
+    else if (keep && kHasLowp)
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false, kHasLowp>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
                            scalar_only);
     else
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false, false>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
                            scalar_only);
     return (int)hipGetLastError();
 }
 
 int dispatch_step(int gd, int ld, uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
-                  const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated,
+                  const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, bool keep,
                   uint32_t scalar_only) {
 #define ELX_CASE(G, L)                                                                                   \
     if (gd == G && ld == L)                                                                              \
-        return launch_step<G, L>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, scalar_only);
+        return launch_step<G, L>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, keep, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -1171,17 +1190,23 @@ int dispatch_step(int gd, int ld, uint32_t lds, hipStream_t st, const ElxChunk *
 
 template <int GD, int LD>
 int launch_step_args(uint32_t lds, hipStream_t st, const HyperPack &pack, const ElxChunk *chunks, uint32_t n_chunks,
-                     const ElxSeg *segs, uint32_t grid_tiles, Unscale us, uint32_t scalar_only) {
-    hipLaunchKernelGGL((adam_step_args_kernel<GD, LD>), dim3(grid_tiles, n_chunks), dim3(kWave), lds, st, pack, chunks,
-                       segs, us, scalar_only);
+                     const ElxSeg *segs, uint32_t grid_tiles, Unscale us, bool keep, uint32_t scalar_only) {
+    constexpr bool kHasLowp = LD != ELX_NONE;
+    if (keep && kHasLowp)
+        hipLaunchKernelGGL((adam_step_args_kernel<GD, LD, kHasLowp>), dim3(grid_tiles, n_chunks), dim3(kWave), lds, st, pack,
+                           chunks, segs, us, scalar_only);
+    else
+        hipLaunchKernelGGL((adam_step_args_kernel<GD, LD, false>), dim3(grid_tiles, n_chunks), dim3(kWave), lds, st, pack,
+                           chunks, segs, us, scalar_only);
     return (int)hipGetLastError();
 }
 
 int dispatch_step_args(int gd, int ld, uint32_t lds, hipStream_t st, const HyperPack &pack, const ElxChunk *chunks,
-                       uint32_t n_chunks, const ElxSeg *segs, uint32_t grid_tiles, Unscale us, uint32_t scalar_only) {
+                       uint32_t n_chunks, const ElxSeg *segs, uint32_t grid_tiles, Unscale us, bool keep,
+                       uint32_t scalar_only) {
 #define ELX_CASE(G, L)                                                                                   \
     if (gd == G && ld == L)                                                                              \
-        return launch_step_args<G, L>(lds, st, pack, chunks, n_chunks, segs, grid_tiles, us, scalar_only);
+        return launch_step_args<G, L>(lds, st, pack, chunks, n_chunks, segs, grid_tiles, us, keep, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -1443,7 +1468,8 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
     if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
         return rc;
     return dispatch_step(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, d_chunks, n_chunks, d_segs, d_hypers,
-                         grid_tiles_per_chunk, unscale_of(div_scale), false, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+                         grid_tiles_per_chunk, unscale_of(div_scale), false, (flags & ELX_FLAG_KEEP_CACHED) != 0,
+                         (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
 int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream);
@@ -1467,7 +1493,8 @@ int elx_adam_step_put_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxS
         HyperPack pack = {};
         __builtin_memcpy(pack.h, h_hypers, n_hypers * sizeof(ElxHyper));
         return dispatch_step_args(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, pack, d_chunks, n_chunks, d_segs,
-                                  grid_tiles_per_chunk, unscale_of(div_scale), (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+                                  grid_tiles_per_chunk, unscale_of(div_scale), (flags & ELX_FLAG_KEEP_CACHED) != 0,
+                                  (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
     }
     if (int rc = elx_put_hypers(h_hypers, n_hypers, d_hypers, stream)) return rc;
     return elx_adam_step_mt(d_chunks, n_chunks, d_segs, n_segs, d_hypers, n_hypers, total_tiles, grid_tiles_per_chunk,
@@ -1502,7 +1529,8 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
     us.inv_scale = 1.0f;
     us.mode = kDivNone;
     return dispatch_step(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, d_chunks, n_chunks, d_segs, d_hypers,
-                         grid_tiles_per_chunk, us, true, (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
+                         grid_tiles_per_chunk, us, true, (flags & ELX_FLAG_KEEP_CACHED) != 0,
+                         (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
 int elx_writeback_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int lowp_dtype, uint32_t blocks_per_chunk,

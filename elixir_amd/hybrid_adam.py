@@ -253,13 +253,15 @@ class HybridAdam(torch.optim.Optimizer):
             hypers[key] = idx
         return idx
 
-    def _device_plan(self, key, buffers_fn, grad_dtype, grad_code, lowp_code, n_hypers, device) -> _DevicePlan:
+    def _device_plan(self, key, buffers_fn, grad_dtype, grad_code, lowp_code, n_hypers, device,
+                     device_resident: bool = True) -> _DevicePlan:
         dplan = self._plans.get(key)
         if dplan is None:
             if len(self._plans) > 8:
                 self._plans.clear()
             esize = 4 if grad_dtype == torch.float32 else 2
-            dplan = _DevicePlan(build_plan(buffers_fn(), esize, esize, n_hypers, grad_code, lowp_code), device)
+            dplan = _DevicePlan(build_plan(buffers_fn(), esize, esize, n_hypers, grad_code, lowp_code,
+                                           device_resident=device_resident), device)
             self._plans[key] = dplan
         return dplan
 
@@ -545,7 +547,8 @@ class HybridAdam(torch.optim.Optimizer):
                                       segs=sorted(per_chunk[i])))
             return out
 
-        dplan = self._device_plan(key, buffers, lowp_dtype, grad_code, lowp_code, len(hypers), device)
+        dplan = self._device_plan(key, buffers, lowp_dtype, grad_code, lowp_code, len(hypers), device,
+                                  device_resident=all(c.shard.is_cuda and c.paired_chunk.shard.is_cuda for c in b.chunks))
         return _Prepared(dplan, self._hyper_table(hypers), grad_code, lowp_code, device, [e[0] for e in entries],
                          hypers.keys())
 

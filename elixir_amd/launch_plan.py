@@ -64,14 +64,23 @@ def choose_block_elems(buffers: Sequence[FlatBuffer], tile: int) -> int:
     return max(16 * tile, min(block, _pow2_at_least(longest)))
 
 
+# The update launch writes the low-precision copy with stores that the memory-side cache (256 MiB) takes in
+# when all low-precision shards of the launch together are no larger than this many bytes.  Measured on sets
+# of equal tensors, step time with against without: -2.5 % at 128 MB, -3 to -5 % at 512 MB, -1.5 % at 1 GB,
+# -1.1 % at 2 GB, -0.5 % at 2.9 GB (the same whether the gradients are re-landed between the steps or the
+# steps follow each other back to back); on the OPT-1.3B set (2.95 GB) +0.2 %, on LLaMA-7B (14.5 GB) +1 %:
+# there the streaming stores are the better ones.
+KEEP_LOWP_CACHED_BELOW = 2 << 30
+
 FOLD_PADDING_BELOW = 24 << 20    # elements: about 20 us of refresh, less than what a launch of its own costs a small set
 
 
 def build_plan(buffers: Sequence[FlatBuffer], grad_esize: int, lowp_esize: int, n_hypers: int, grad_dtype: int,
-               lowp_dtype: int, fold_padding_below: int = FOLD_PADDING_BELOW) -> LaunchPlan:
+               lowp_dtype: int, fold_padding_below: int = FOLD_PADDING_BELOW, device_resident: bool = True) -> LaunchPlan:
     """``fold_padding_below``: when the runs of pure padding hold fewer elements than this in total they
     are listed as rows of the update launch (n_valid = 0: refreshed tile by tile there) instead of going
-    to a refresh launch of their own."""
+    to a refresh launch of their own.  ``device_resident``: every buffer lies in device memory (the
+    memory-side cache only fronts that)."""
     tile = _abi.tile_elems()
     block = choose_block_elems(buffers, tile)
     rows, segs, refresh = [], [], []
@@ -110,6 +119,9 @@ def build_plan(buffers: Sequence[FlatBuffer], grad_esize: int, lowp_esize: int, 
     rows_np = np.array(rows, dtype=_abi.CHUNK_DTYPE) if rows else np.zeros(0, dtype=_abi.CHUNK_DTYPE)
     segs_np = np.array(segs, dtype=_abi.SEG_DTYPE) if segs else np.zeros(0, dtype=_abi.SEG_DTYPE)
     info = _abi.check_tables(rows_np, segs_np, n_hypers, grad_dtype, lowp_dtype) if len(rows_np) else None
+    if info is not None:
+        lowp_bytes = sum(b.n_alloc for b in buffers if b.lowp_out) * lowp_esize
+        info = info.with_keep_lowp_cached(device_resident and 0 < lowp_bytes <= KEEP_LOWP_CACHED_BELOW)
     refresh_np, refresh_max = None, 0
     if refresh:
         refresh_np = np.array(refresh, dtype=_abi.CHUNK_DTYPE)

@@ -56,7 +56,13 @@ enum {
                                     (256 MiB) for the update launch that reads them next.  Pays when all
                                     gradients of the launch fit that cache (2-5 % of the step at 64-256 MiB);
                                     a larger set streams faster without it (the stats pass of a 2.6 GB set is
-                                    16 % slower with it).  Results do not depend on it */
+                                    16 % slower with it).
+                                    Update launches: the low-precision copy is written with stores that the
+                                    memory-side cache takes in (over the gradients it replaces, when they are
+                                    still there) and writes back later, instead of streaming stores.  Pays up
+                                    to about 2 GB of low-precision shards (3 % of the step at 0.25-0.5 GB, 1 %
+                                    at 1-2 GB); larger sets lose up to 1 % with it.
+                                    Results never depend on it */
 };
 
 /*
@@ -279,6 +285,8 @@ uint32_t elx_static_partials(void);
  *                          tile x, nothing is looked up.  At least the max_tiles_per_chunk that
  *                          elx_check_tables reported; 0, or a grid that cannot hold total_tiles, is
  *                          ELX_E_TILES.  n_chunks <= 65535: list a long shard as several records
+ *   flags          0, ELX_FLAG_SCALAR_ONLY (elx_check_tables found a base pointer that is not 16-byte
+ *                  aligned), ELX_FLAG_KEEP_CACHED (store policy of the low-precision copy, above), or both
  *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (13 for
  *                  16-bit gradients, 12 for fp32 gradients).
  *                  The update streams best with a shallow, orderly queue of memory requests.

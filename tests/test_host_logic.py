@@ -357,6 +357,35 @@ def test_launch_plan_blocks_segments_and_padding():
     assert plan.refresh_rows is not None and int(plan.rows['n_alloc'].sum()) + int(plan.refresh_rows['n_alloc'].sum()) == 1 << 26
 
 
+def test_launch_plan_chooses_the_store_policy_of_the_low_precision_copy_by_size():
+    """Low-precision shards of up to 2 GiB in all, in device memory: the update launch is told to write them
+    with the stores the memory-side cache takes in (ELX_FLAG_KEEP_CACHED); larger sets, host-resident ones
+    and launches without a low-precision copy keep the streaming stores."""
+    from elixir_amd.launch_plan import KEEP_LOWP_CACHED_BELOW, FlatBuffer, build_plan
+    base = 0x40000000
+    assert KEEP_LOWP_CACHED_BELOW == 2 << 30
+
+    def plan_of(n_buffers, n_alloc, lowp=True, **kw):
+        bufs = [FlatBuffer(grad=base + (i << 34), lowp_out=(base + (i << 34)) if lowp else 0, master=base + (i << 34) + (1 << 32),
+                           m=base + (i << 34) + (2 << 32), v=base + (i << 34) + (3 << 32), n_alloc=n_alloc, n_valid=n_alloc,
+                           segs=[(0, n_alloc, 0)]) for i in range(n_buffers)]
+        esize = 2 if lowp else 4
+        return build_plan(bufs, esize, esize, 1, _abi.ELX_F16 if lowp else _abi.ELX_F32,
+                          _abi.ELX_F16 if lowp else _abi.ELX_NONE, **kw)
+
+    small = plan_of(2, 64 << 20)                     # 256 MiB of fp16
+    assert small.info.keep_lowp_cached and small.info.flags == _abi.ELX_FLAG_KEEP_CACHED
+    assert plan_of(8, 128 << 20).info.keep_lowp_cached              # exactly 2 GiB
+    large = plan_of(9, 128 << 20)                                   # 2.25 GiB
+    assert not large.info.keep_lowp_cached and large.info.flags == 0
+    assert not plan_of(2, 64 << 20, device_resident=False).info.keep_lowp_cached
+    assert not plan_of(1, 1 << 20, lowp=False).info.keep_lowp_cached
+    # what elx_check_tables reports carries no choice
+    info = _abi.check_tables(small.rows, small.segs, 1, _abi.ELX_F16, _abi.ELX_F16)
+    assert not info.keep_lowp_cached and info.with_keep_lowp_cached(True).flags == _abi.ELX_FLAG_KEEP_CACHED
+    assert info.with_keep_lowp_cached(True)[:3] == tuple(info)
+
+
 def test_launch_plan_keeps_rows_bounded_for_the_large_workloads():
     from elixir_amd.launch_plan import FlatBuffer, build_plan
     from elixir_amd.module import greedy_groups
