@@ -14,6 +14,7 @@ ELX_ABI_VERSION = 2
 ELX_F32, ELX_F16, ELX_BF16, ELX_NONE = 0, 1, 2, -1
 ELX_FLAG_SCALAR_ONLY = 1
 ELX_FLAG_KEEP_CACHED = 2
+ELX_FLAG_KEEP_STATE_CACHED = 4
 ELX_E_NULL, ELX_E_DTYPE, ELX_E_ALIGN, ELX_E_RANGE, ELX_E_ORDER, ELX_E_TILES, ELX_E_SIZE = -1, -2, -3, -4, -5, -6, -7
 ELX_HYPER_L2 = 1
 ELX_HYPER_LERP_FROM_G = 2
@@ -142,7 +143,9 @@ def _np_ptr(a: Optional[np.ndarray]):
 
 class TableInfo(tuple):
     """(total_tiles, max_tiles_per_chunk, all_aligned16) as reported by elx_check_tables, optionally followed
-    by the caller's choice of store policy for the low-precision copy (``keep_lowp_cached``)."""
+    by the caller's choice of cache policy for the update launch: 0 every access streams, 1 the low-precision
+    copy is stored through the memory-side cache (``ELX_FLAG_KEEP_CACHED``), 2 the whole state of the launch
+    fits that cache and stays there (``ELX_FLAG_KEEP_STATE_CACHED``)."""
     __slots__ = ()
 
     @property
@@ -158,16 +161,29 @@ class TableInfo(tuple):
         return self[2]
 
     @property
+    def cache_policy(self) -> int:
+        return int(self[3]) if len(self) > 3 else 0
+
+    @property
     def keep_lowp_cached(self) -> bool:
-        return len(self) > 3 and bool(self[3])
+        return self.cache_policy >= 1
+
+    @property
+    def keep_state_cached(self) -> bool:
+        return self.cache_policy >= 2
+
+    def with_cache_policy(self, policy: int) -> 'TableInfo':
+        assert policy in (0, 1, 2)
+        return TableInfo(tuple(self[:3]) + (int(policy), ))
 
     def with_keep_lowp_cached(self, keep: bool) -> 'TableInfo':
-        return TableInfo(tuple(self[:3]) + (bool(keep), ))
+        return self.with_cache_policy(1 if keep else 0)
 
     @property
     def flags(self) -> int:
         """The ``flags`` argument of the update launches for these tables."""
-        return (0 if self[2] else ELX_FLAG_SCALAR_ONLY) | (ELX_FLAG_KEEP_CACHED if self.keep_lowp_cached else 0)
+        return ((0 if self[2] else ELX_FLAG_SCALAR_ONLY) | (ELX_FLAG_KEEP_CACHED if self.cache_policy >= 1 else 0)
+                | (ELX_FLAG_KEEP_STATE_CACHED if self.cache_policy >= 2 else 0))
 
 
 def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, grad_dtype: int,

@@ -140,34 +140,42 @@ struct TileIo;
 
 template <>
 struct TileIo<f32x4> {
+    template <int AUX = kAuxLoad>
     static __device__ __forceinline__ f32x4 load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
-        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxLoad));
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, AUX));
     }
+    template <int AUX = kAuxStore>
     static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, f32x4 x) {
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, (int)off, 0, kAuxStore);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, (int)off, 0, AUX);
     }
 };
 
 template <>
 struct TileIo<u16x4> {
+    template <int AUX = kAuxLoad>
     static __device__ __forceinline__ u16x4 load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
-        return __builtin_bit_cast(u16x4, __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kAuxLoad));
+        return __builtin_bit_cast(u16x4, __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, AUX));
     }
+    template <int AUX = kAuxStore>
     static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, uint32_t off, u16x4 x) {
-        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, x), r, (int)off, 0, kAuxStore);
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, x), r, (int)off, 0, AUX);
     }
 };
 
-// The low-precision copy of a tile goes out with the streaming policy of the other stores, or (KEEP) at
-// agent scope without the non-temporal hint: such a store is taken in by the memory-side cache, over the
-// gradient it replaces when that is still there, and written back from there later.
-template <bool KEEP, typename V>
-__device__ __forceinline__ void store_lowp_tile(__amdgpu_buffer_rsrc_t r, uint32_t off, V x) {
-    if constexpr (sizeof(V) == 16)
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, (int)off, 0, KEEP ? kAuxStoreKeep : kAuxStore);
-    else
-        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, x), r, (int)off, 0, KEEP ? kAuxStoreKeep : kAuxStore);
-}
+// Cache policy of an update launch (ELX_FLAG_KEEP_CACHED, ELX_FLAG_KEEP_STATE_CACHED).
+//   kStream     every access streams: non-temporal loads, non-temporal stores at agent scope;
+//   kKeepLowp   the low-precision copy alone is stored at agent scope without the non-temporal hint: such a
+//               store is taken in by the memory-side cache, over the gradient it replaces when that is still
+//               there, and written back from there later;
+//   kKeepState  everything the launch touches fits that cache: ordinary loads, and all stores as above, so
+//               that the next step finds the state there.
+enum { kStream = 0, kKeepLowp = 1, kKeepState = 2 };
+template <int POLICY>
+struct Aux {
+    static constexpr int load = POLICY == kKeepState ? 0 : kAuxLoad;
+    static constexpr int store = POLICY == kKeepState ? kAuxStoreKeep : kAuxStore;
+    static constexpr int store_lowp = POLICY == kStream ? kAuxStore : kAuxStoreKeep;
+};
 
 // ---------------------------------------------------------------------------------------------
 // the update of one element
@@ -284,7 +292,7 @@ __device__ __forceinline__ void tile_math_flags(const typename Elem<GD>::vec4 (&
 // fused update + writeback
 // ---------------------------------------------------------------------------------------------
 
-template <int LD, bool KEEPL>
+template <int LD, int POLICY>
 __device__ __forceinline__ void store_lowp_vec(const ElxChunk &c, uint64_t base, const f32x4 (&P)[kUnroll]) {
     if constexpr (LD != ELX_NONE) {
         if (!c.lowp_out) return;
@@ -296,21 +304,22 @@ __device__ __forceinline__ void store_lowp_vec(const ElxChunk &c, uint64_t base,
             lvec L;
 #pragma unroll
             for (int k = 0; k < kVec; ++k) L[k] = Elem<LD>::from_f32(P[u][k]);
-            store_lowp_tile<KEEPL>(lr, (threadIdx.x + u * kWave) * sizeof(lvec), L);
+            TileIo<lvec>::template store<Aux<POLICY>::store_lowp>(lr, (threadIdx.x + u * kWave) * sizeof(lvec), L);
         }
     }
 }
 
 // Whole tile outside the valid head of the shard (padding), or the writeback-only launch.
-template <int LD, bool KEEPL>
+template <int LD, int POLICY>
 __device__ __forceinline__ void tile_refresh_vec(const ElxChunk &c, uint64_t base) {
     if constexpr (LD != ELX_NONE) {
         if (!c.lowp_out) return;
         const __amdgpu_buffer_rsrc_t pr = tile_rsrc(c.master + base, kTile * sizeof(float));
         f32x4 P[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) P[u] = TileIo<f32x4>::load(pr, (threadIdx.x + u * kWave) * sizeof(f32x4));
-        store_lowp_vec<LD, KEEPL>(c, base, P);
+        for (int u = 0; u < kUnroll; ++u)
+            P[u] = TileIo<f32x4>::template load<Aux<POLICY>::load>(pr, (threadIdx.x + u * kWave) * sizeof(f32x4));
+        store_lowp_vec<LD, POLICY>(c, base, P);
     }
 }
 
@@ -384,7 +393,7 @@ static_assert(sizeof(ElxChunk) == 72, "load_chunk_row reads nine 64-bit words");
 // has put them earlier on the same stream) instead of the kernel arguments, so that the launch can be
 // enqueued before the host knows whether the step happens.  They arrive with the hyper record the
 // tile loads anyway; on a skip the tile only refreshes its low-precision copy.
-template <int GD, int LD, bool GATED, bool KEEPL>
+template <int GD, int LD, bool GATED, int POLICY>
 __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chunks, const ElxSeg *__restrict__ segs,
                                                const ElxHyper *__restrict__ hypers, Unscale us, uint32_t scalar_only) {
     // 2-D grid (tiles, records): blockIdx.y names the record, blockIdx.x the tile; nothing is looked
@@ -414,11 +423,11 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
         // below then overlap the memory latency
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            G[u] = TileIo<gvec>::load(gr, (threadIdx.x + u * kWave) * sizeof(gvec));
+            G[u] = TileIo<gvec>::template load<Aux<POLICY>::load>(gr, (threadIdx.x + u * kWave) * sizeof(gvec));
             const uint32_t off = (threadIdx.x + u * kWave) * sizeof(f32x4);
-            P[u] = TileIo<f32x4>::load(pr, off);
-            M[u] = TileIo<f32x4>::load(mr, off);
-            V[u] = TileIo<f32x4>::load(vr, off);
+            P[u] = TileIo<f32x4>::template load<Aux<POLICY>::load>(pr, off);
+            M[u] = TileIo<f32x4>::template load<Aux<POLICY>::load>(mr, off);
+            V[u] = TileIo<f32x4>::template load<Aux<POLICY>::load>(vr, off);
         }
         // first segment of the chunk that ends after the start of the tile
         uint32_t s = c.seg_begin, s_hi = c.seg_end;
@@ -439,7 +448,7 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
                 us.inv_scale = h.gate_inv;
                 us.mode = (int)(h.gate & 0xFFu);
                 if (h.gate >> 8) {    // the step is skipped: refresh the low-precision copy only
-                    store_lowp_vec<LD, KEEPL>(c, base, P);
+                    store_lowp_vec<LD, POLICY>(c, base, P);
                     return;
                 }
             }
@@ -452,15 +461,15 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
                 const uint32_t off = (threadIdx.x + u * kWave) * sizeof(f32x4);
-                TileIo<f32x4>::store(pr, off, P[u]);
-                TileIo<f32x4>::store(mr, off, M[u]);
-                TileIo<f32x4>::store(vr, off, V[u]);
+                TileIo<f32x4>::template store<Aux<POLICY>::store>(pr, off, P[u]);
+                TileIo<f32x4>::template store<Aux<POLICY>::store>(mr, off, M[u]);
+                TileIo<f32x4>::template store<Aux<POLICY>::store>(vr, off, V[u]);
             }
-            store_lowp_vec<LD, KEEPL>(c, base, P);
+            store_lowp_vec<LD, POLICY>(c, base, P);
             return;
         }
         if (!has || sb >= base + kTile) {    // inside the valid head but owned by no segment
-            store_lowp_vec<LD, KEEPL>(c, base, P);
+            store_lowp_vec<LD, POLICY>(c, base, P);
             return;
         }
         // the tile straddles a segment boundary: redo it element by element below
@@ -471,7 +480,7 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
     const uint32_t tile_n = left < kTile ? (uint32_t)left : kTile;
     if (base >= c.n_valid) {    // padding inside an update chunk: refresh only
         if (tile_n == kTile && !scalar_only)
-            tile_refresh_vec<LD, KEEPL>(c, base);
+            tile_refresh_vec<LD, POLICY>(c, base);
         else
             tile_scalar<GD, LD, GATED>(c, base, tile_n, 0, segs, hypers, us, true);
         return;
@@ -487,12 +496,12 @@ __device__ __forceinline__ void adam_step_tile(const ElxChunk *__restrict__ chun
     tile_scalar<GD, LD, GATED>(c, base, tile_n, s, segs, hypers, us, false);
 }
 
-template <int GD, int LD, bool GATED, bool KEEPL>
+template <int GD, int LD, bool GATED, int POLICY>
 __global__ __launch_bounds__(kWave) void adam_step_kernel(const ElxChunk *__restrict__ chunks,
                                                           const ElxSeg *__restrict__ segs,
                                                           const ElxHyper *__restrict__ hypers, Unscale us,
                                                           uint32_t scalar_only) {
-    adam_step_tile<GD, LD, GATED, KEEPL>(chunks, segs, hypers, us, scalar_only);
+    adam_step_tile<GD, LD, GATED, POLICY>(chunks, segs, hypers, us, scalar_only);
 }
 
 // A handful of hyper records travel in the arguments of the launch that uses them.
@@ -504,7 +513,7 @@ static_assert(offsetof(HyperPack, h) == 0, "the records start at offset 0 of the
 
 // The update launch of a host-decided or standalone step whose hyper records fit its own arguments:
 // the table the tiles read is the argument segment itself, so no launch has to fill a table first.
-template <int GD, int LD, bool KEEPL>
+template <int GD, int LD, int POLICY>
 __global__ __launch_bounds__(kWave) void adam_step_args_kernel(HyperPack pack, const ElxChunk *__restrict__ chunks,
                                                                const ElxSeg *__restrict__ segs, Unscale us,
                                                                uint32_t scalar_only) {
@@ -512,7 +521,7 @@ __global__ __launch_bounds__(kWave) void adam_step_args_kernel(HyperPack pack, c
     // aggregate would copy it to private memory first)
     typedef const ElxHyper __attribute__((address_space(4))) *kernarg_hypers;
     const ElxHyper *hypers = (const ElxHyper *)(kernarg_hypers)__builtin_amdgcn_kernarg_segment_ptr();
-    adam_step_tile<GD, LD, false, KEEPL>(chunks, segs, hypers, us, scalar_only);
+    adam_step_tile<GD, LD, false, POLICY>(chunks, segs, hypers, us, scalar_only);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1152,32 +1161,50 @@ int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes, uint32_t 
     return 0;
 }
 
-template <int GD, int LD>
-int launch_step(uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks, const ElxSeg *segs,
-                const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, bool keep, uint32_t scalar_only) {
+// The cache policy the flags of an update launch ask for.  Without a low-precision copy kKeepLowp has nothing
+// to act on and is the streaming launch.
+template <int LD>
+int policy_of(uint32_t flags) {
+    if (flags & ELX_FLAG_KEEP_STATE_CACHED) return kKeepState;
+    if ((flags & ELX_FLAG_KEEP_CACHED) && LD != ELX_NONE) return kKeepLowp;
+    return kStream;
+}
+
+template <int GD, int LD, bool GATED>
+int launch_step_policy(uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks, const ElxSeg *segs,
+                       const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, uint32_t flags, uint32_t scalar_only) {
     const dim3 grid(grid_tiles, n_chunks);
-    constexpr bool kHasLowp = LD != ELX_NONE;    // without a low-precision copy there is no policy to choose
-    if (gated && keep && kHasLowp)
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true, kHasLowp>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
-                           scalar_only);
-    else if (gated)
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, true, false>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
-                           scalar_only);
-    else if (keep && kHasLowp)
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false, kHasLowp>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
-                           scalar_only);
-    else
-        hipLaunchKernelGGL((adam_step_kernel<GD, LD, false, false>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
-                           scalar_only);
+    constexpr int kLowp = LD != ELX_NONE ? kKeepLowp : kStream;    // no third instantiation without a low-precision copy
+    switch (policy_of<LD>(flags)) {
+        case kKeepState:
+            hipLaunchKernelGGL((adam_step_kernel<GD, LD, GATED, kKeepState>), grid, dim3(kWave), lds, st, chunks, segs, hypers,
+                               us, scalar_only);
+            break;
+        case kKeepLowp:
+            hipLaunchKernelGGL((adam_step_kernel<GD, LD, GATED, kLowp>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+                               scalar_only);
+            break;
+        default:
+            hipLaunchKernelGGL((adam_step_kernel<GD, LD, GATED, kStream>), grid, dim3(kWave), lds, st, chunks, segs, hypers, us,
+                               scalar_only);
+    }
     return (int)hipGetLastError();
 }
 
+template <int GD, int LD>
+int launch_step(uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks, const ElxSeg *segs,
+                const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, uint32_t flags, uint32_t scalar_only) {
+    if (gated)
+        return launch_step_policy<GD, LD, true>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, flags, scalar_only);
+    return launch_step_policy<GD, LD, false>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, flags, scalar_only);
+}
+
 int dispatch_step(int gd, int ld, uint32_t lds, hipStream_t st, const ElxChunk *chunks, uint32_t n_chunks,
-                  const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, bool keep,
+                  const ElxSeg *segs, const ElxHyper *hypers, uint32_t grid_tiles, Unscale us, bool gated, uint32_t flags,
                   uint32_t scalar_only) {
 #define ELX_CASE(G, L)                                                                                   \
     if (gd == G && ld == L)                                                                              \
-        return launch_step<G, L>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, keep, scalar_only);
+        return launch_step<G, L>(lds, st, chunks, n_chunks, segs, hypers, grid_tiles, us, gated, flags, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -1190,23 +1217,31 @@ int dispatch_step(int gd, int ld, uint32_t lds, hipStream_t st, const ElxChunk *
 
 template <int GD, int LD>
 int launch_step_args(uint32_t lds, hipStream_t st, const HyperPack &pack, const ElxChunk *chunks, uint32_t n_chunks,
-                     const ElxSeg *segs, uint32_t grid_tiles, Unscale us, bool keep, uint32_t scalar_only) {
-    constexpr bool kHasLowp = LD != ELX_NONE;
-    if (keep && kHasLowp)
-        hipLaunchKernelGGL((adam_step_args_kernel<GD, LD, kHasLowp>), dim3(grid_tiles, n_chunks), dim3(kWave), lds, st, pack,
-                           chunks, segs, us, scalar_only);
-    else
-        hipLaunchKernelGGL((adam_step_args_kernel<GD, LD, false>), dim3(grid_tiles, n_chunks), dim3(kWave), lds, st, pack,
-                           chunks, segs, us, scalar_only);
+                     const ElxSeg *segs, uint32_t grid_tiles, Unscale us, uint32_t flags, uint32_t scalar_only) {
+    const dim3 grid(grid_tiles, n_chunks);
+    constexpr int kLowp = LD != ELX_NONE ? kKeepLowp : kStream;
+    switch (policy_of<LD>(flags)) {
+        case kKeepState:
+            hipLaunchKernelGGL((adam_step_args_kernel<GD, LD, kKeepState>), grid, dim3(kWave), lds, st, pack, chunks, segs, us,
+                               scalar_only);
+            break;
+        case kKeepLowp:
+            hipLaunchKernelGGL((adam_step_args_kernel<GD, LD, kLowp>), grid, dim3(kWave), lds, st, pack, chunks, segs, us,
+                               scalar_only);
+            break;
+        default:
+            hipLaunchKernelGGL((adam_step_args_kernel<GD, LD, kStream>), grid, dim3(kWave), lds, st, pack, chunks, segs, us,
+                               scalar_only);
+    }
     return (int)hipGetLastError();
 }
 
 int dispatch_step_args(int gd, int ld, uint32_t lds, hipStream_t st, const HyperPack &pack, const ElxChunk *chunks,
-                       uint32_t n_chunks, const ElxSeg *segs, uint32_t grid_tiles, Unscale us, bool keep,
+                       uint32_t n_chunks, const ElxSeg *segs, uint32_t grid_tiles, Unscale us, uint32_t flags,
                        uint32_t scalar_only) {
 #define ELX_CASE(G, L)                                                                                   \
     if (gd == G && ld == L)                                                                              \
-        return launch_step_args<G, L>(lds, st, pack, chunks, n_chunks, segs, grid_tiles, us, keep, scalar_only);
+        return launch_step_args<G, L>(lds, st, pack, chunks, n_chunks, segs, grid_tiles, us, flags, scalar_only);
     ELX_CASE(ELX_F32, ELX_NONE)
     ELX_CASE(ELX_F32, ELX_F32)
     ELX_CASE(ELX_F16, ELX_NONE)
@@ -1468,7 +1503,7 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
     if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
         return rc;
     return dispatch_step(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, d_chunks, n_chunks, d_segs, d_hypers,
-                         grid_tiles_per_chunk, unscale_of(div_scale), false, (flags & ELX_FLAG_KEEP_CACHED) != 0,
+                         grid_tiles_per_chunk, unscale_of(div_scale), false, flags,
                          (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 
@@ -1493,7 +1528,7 @@ int elx_adam_step_put_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxS
         HyperPack pack = {};
         __builtin_memcpy(pack.h, h_hypers, n_hypers * sizeof(ElxHyper));
         return dispatch_step_args(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, pack, d_chunks, n_chunks, d_segs,
-                                  grid_tiles_per_chunk, unscale_of(div_scale), (flags & ELX_FLAG_KEEP_CACHED) != 0,
+                                  grid_tiles_per_chunk, unscale_of(div_scale), flags,
                                   (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
     }
     if (int rc = elx_put_hypers(h_hypers, n_hypers, d_hypers, stream)) return rc;
@@ -1529,7 +1564,7 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
     us.inv_scale = 1.0f;
     us.mode = kDivNone;
     return dispatch_step(grad_dtype, lowp_dtype, lds, (hipStream_t)stream, d_chunks, n_chunks, d_segs, d_hypers,
-                         grid_tiles_per_chunk, us, true, (flags & ELX_FLAG_KEEP_CACHED) != 0,
+                         grid_tiles_per_chunk, us, true, flags,
                          (flags & ELX_FLAG_SCALAR_ONLY) ? 1u : 0u);
 }
 

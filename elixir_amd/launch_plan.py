@@ -72,6 +72,14 @@ def choose_block_elems(buffers: Sequence[FlatBuffer], tile: int) -> int:
 # there the streaming stores are the better ones.
 KEEP_LOWP_CACHED_BELOW = 2 << 30
 
+# Everything an update launch touches -- gradients, master weights, exp_avg, exp_avg_sq, low-precision copy --
+# is at most this many bytes: the size of the memory-side cache.  The launch then reads with ordinary loads
+# and stores everything the way it stores the low-precision copy above, and the next step finds the state in
+# the cache.  Measured on a flat fp32 parameter with fp32 gradients, step time with against without: 0.0363 /
+# 0.0405 ms at 4 Mi elements, 0.0548 / 0.0544 at 8 Mi, 0.0845 / 0.0906 at 16 Mi (256 MiB in all: the limit);
+# beyond it the policy loses: 0.1043 / 0.1044 at 19.9 Mi, 0.1264 / 0.1204 at 23.7 Mi, 0.1805 / 0.1581 at 32 Mi.
+KEEP_STATE_CACHED_BELOW = 256 << 20
+
 FOLD_PADDING_BELOW = 24 << 20    # elements: about 20 us of refresh, less than what a launch of its own costs a small set
 
 
@@ -121,7 +129,14 @@ def build_plan(buffers: Sequence[FlatBuffer], grad_esize: int, lowp_esize: int, 
     info = _abi.check_tables(rows_np, segs_np, n_hypers, grad_dtype, lowp_dtype) if len(rows_np) else None
     if info is not None:
         lowp_bytes = sum(b.n_alloc for b in buffers if b.lowp_out) * lowp_esize
-        info = info.with_keep_lowp_cached(device_resident and 0 < lowp_bytes <= KEEP_LOWP_CACHED_BELOW)
+        state_bytes = sum(b.n_alloc * (12 + (grad_esize if b.grad else 0)
+                                       + (lowp_esize if b.lowp_out and b.lowp_out != b.grad else 0)) for b in buffers)
+        policy = 0
+        if device_resident and 0 < lowp_bytes <= KEEP_LOWP_CACHED_BELOW:
+            policy = 1
+        if device_resident and state_bytes <= KEEP_STATE_CACHED_BELOW:
+            policy = 2
+        info = info.with_cache_policy(policy)
     refresh_np, refresh_max = None, 0
     if refresh:
         refresh_np = np.array(refresh, dtype=_abi.CHUNK_DTYPE)

@@ -51,7 +51,7 @@ enum {
 enum {
     ELX_FLAG_SCALAR_ONLY = 1u,   /* take the element-by-element path for every tile (set by the host when
                                     elx_check_tables reports base pointers that are not 16-byte aligned) */
-    ELX_FLAG_KEEP_CACHED = 2u    /* stats and landing launches: touch the gradients with ordinary loads / stores
+    ELX_FLAG_KEEP_CACHED = 2u,   /* stats and landing launches: touch the gradients with ordinary loads / stores
                                     instead of non-temporal ones, so that they stay in the memory-side cache
                                     (256 MiB) for the update launch that reads them next.  Pays when all
                                     gradients of the launch fit that cache (2-5 % of the step at 64-256 MiB);
@@ -63,6 +63,12 @@ enum {
                                     to about 2 GB of low-precision shards (3 % of the step at 0.25-0.5 GB, 1 %
                                     at 1-2 GB); larger sets lose up to 1 % with it.
                                     Results never depend on it */
+    ELX_FLAG_KEEP_STATE_CACHED = 4u  /* update launches: everything the launch touches (gradients, master, m, v,
+                                    low-precision copy) fits the memory-side cache: ordinary loads, and every
+                                    store as ELX_FLAG_KEEP_CACHED stores the low-precision copy, so that the
+                                    next step finds the state there.  7 % of the step for 16 Mi fp32 elements
+                                    with fp32 gradients (256 MiB in all); a set twice that size loses 14 %
+                                    with it.  Implies ELX_FLAG_KEEP_CACHED.  Results never depend on it */
 };
 
 /*
@@ -286,7 +292,7 @@ uint32_t elx_static_partials(void);
  *                          elx_check_tables reported; 0, or a grid that cannot hold total_tiles, is
  *                          ELX_E_TILES.  n_chunks <= 65535: list a long shard as several records
  *   flags          0, ELX_FLAG_SCALAR_ONLY (elx_check_tables found a base pointer that is not 16-byte
- *                  aligned), ELX_FLAG_KEEP_CACHED (store policy of the low-precision copy, above), or both
+ *                  aligned), ELX_FLAG_KEEP_CACHED / ELX_FLAG_KEEP_STATE_CACHED (cache policy, above), or a sum
  *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (13 for
  *                  16-bit gradients, 12 for fp32 gradients).
  *                  The update streams best with a shallow, orderly queue of memory requests.

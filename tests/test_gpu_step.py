@@ -928,10 +928,11 @@ def test_update_on_misaligned_buffers(oracle, gdtype, how):
             g[n_valid] = float('inf')
         data.append((g, master, m, v))
 
-    def launch(offsets, keep_lowp_cached=False):
+    def launch(offsets, cache_policy=0):
         """Runs the update on copies of ``data`` placed at the given element offsets; returns the
-        buffers afterwards and whether the tables were reported aligned.  ``keep_lowp_cached``: the
-        low-precision copy goes out with the stores of ELX_FLAG_KEEP_CACHED."""
+        buffers afterwards and whether the tables were reported aligned.  ``cache_policy`` 1: the
+        low-precision copy goes out with the stores of ELX_FLAG_KEEP_CACHED; 2: every access follows
+        ELX_FLAG_KEEP_STATE_CACHED."""
         bufs, rows, segs, tiles = [], np.zeros(len(layout), dtype=_abi.CHUNK_DTYPE), [], 0
         for i, ((n_alloc, n_valid, seg_list), (g, master, m, v)) in enumerate(zip(layout, data)):
             views = [_offset_view(t, o) for t, o in zip((g, master, m, v), offsets)]
@@ -944,8 +945,9 @@ def test_update_on_misaligned_buffers(oracle, gdtype, how):
             segs += [(b, e, h, 0) for b, e, h in seg_list]
             rows[i]['seg_end'] = len(segs)
         segs = np.array(segs, dtype=_abi.SEG_DTYPE)
-        info = _abi.check_tables(rows, segs, len(hyper_host), code, code).with_keep_lowp_cached(keep_lowp_cached)
-        assert bool(info.flags & _abi.ELX_FLAG_KEEP_CACHED) == keep_lowp_cached
+        info = _abi.check_tables(rows, segs, len(hyper_host), code, code).with_cache_policy(cache_policy)
+        assert bool(info.flags & _abi.ELX_FLAG_KEEP_CACHED) == (cache_policy >= 1)
+        assert bool(info.flags & _abi.ELX_FLAG_KEEP_STATE_CACHED) == (cache_policy == 2)
         d_rows, d_segs = DeviceTable(rows, torch.device(DEV, 0)), DeviceTable(segs, torch.device(DEV, 0))
         d_hyp = DeviceTable(hyper_host, torch.device(DEV, 0))
         stream = torch.cuda.current_stream().cuda_stream
@@ -975,7 +977,8 @@ def test_update_on_misaligned_buffers(oracle, gdtype, how):
 
     odd, odd_aligned = launch((1, 1, 2, 3))
     even, even_aligned = launch((0, 0, 0, 0))
-    kept, _ = launch((0, 0, 0, 0), keep_lowp_cached=True)    # the other store policy: same bits
+    kept, _ = launch((0, 0, 0, 0), cache_policy=1)    # the other cache policies: same bits
+    kept_all, _ = launch((0, 0, 0, 0), cache_policy=2)
     assert not odd_aligned and even_aligned
 
     for i, ((n_alloc, n_valid, seg_list), (g, master, m, v)) in enumerate(zip(layout, data)):
@@ -989,10 +992,11 @@ def test_update_on_misaligned_buffers(oracle, gdtype, how):
         else:
             assert np.array_equal(pn, to_np(master))
         want = (oracle.writeback(pn, code), pn, mn, vn)    # the whole record is refreshed, padding included
-        for name, w, a, b, k in zip(('lowp', 'master', 'm', 'v'), want, odd[i], even[i], kept[i]):
+        for name, w, a, b, k, k2 in zip(('lowp', 'master', 'm', 'v'), want, odd[i], even[i], kept[i], kept_all[i]):
             assert np.array_equal(to_np(a).view(np.uint8), w.view(np.uint8)), f'{how} record {i} {name}: misaligned vs oracle'
             assert np.array_equal(to_np(b).view(np.uint8), w.view(np.uint8)), f'{how} record {i} {name}: aligned vs oracle'
             assert np.array_equal(to_np(k).view(np.uint8), w.view(np.uint8)), f'{how} record {i} {name}: kept stores vs oracle'
+            assert np.array_equal(to_np(k2).view(np.uint8), w.view(np.uint8)), f'{how} record {i} {name}: kept state vs oracle'
 
 
 # ------------------------------------------------------------------------------------------------

@@ -357,13 +357,15 @@ def test_launch_plan_blocks_segments_and_padding():
     assert plan.refresh_rows is not None and int(plan.rows['n_alloc'].sum()) + int(plan.refresh_rows['n_alloc'].sum()) == 1 << 26
 
 
-def test_launch_plan_chooses_the_store_policy_of_the_low_precision_copy_by_size():
+def test_launch_plan_chooses_the_cache_policy_of_the_update_launch_by_size():
     """Low-precision shards of up to 2 GiB in all, in device memory: the update launch is told to write them
-    with the stores the memory-side cache takes in (ELX_FLAG_KEEP_CACHED); larger sets, host-resident ones
-    and launches without a low-precision copy keep the streaming stores."""
-    from elixir_amd.launch_plan import KEEP_LOWP_CACHED_BELOW, FlatBuffer, build_plan
+    with the stores the memory-side cache takes in (ELX_FLAG_KEEP_CACHED).  Everything the launch touches at
+    most 256 MiB: ELX_FLAG_KEEP_STATE_CACHED on top.  Larger sets, host-resident ones and large launches
+    without a low-precision copy stream."""
+    from elixir_amd.launch_plan import KEEP_LOWP_CACHED_BELOW, KEEP_STATE_CACHED_BELOW, FlatBuffer, build_plan
     base = 0x40000000
-    assert KEEP_LOWP_CACHED_BELOW == 2 << 30
+    assert KEEP_LOWP_CACHED_BELOW == 2 << 30 and KEEP_STATE_CACHED_BELOW == 256 << 20
+    lowp_flag, state_flags = _abi.ELX_FLAG_KEEP_CACHED, _abi.ELX_FLAG_KEEP_CACHED | _abi.ELX_FLAG_KEEP_STATE_CACHED
 
     def plan_of(n_buffers, n_alloc, lowp=True, **kw):
         bufs = [FlatBuffer(grad=base + (i << 34), lowp_out=(base + (i << 34)) if lowp else 0, master=base + (i << 34) + (1 << 32),
@@ -373,17 +375,25 @@ def test_launch_plan_chooses_the_store_policy_of_the_low_precision_copy_by_size(
         return build_plan(bufs, esize, esize, 1, _abi.ELX_F16 if lowp else _abi.ELX_F32,
                           _abi.ELX_F16 if lowp else _abi.ELX_NONE, **kw)
 
-    small = plan_of(2, 64 << 20)                     # 256 MiB of fp16
-    assert small.info.keep_lowp_cached and small.info.flags == _abi.ELX_FLAG_KEEP_CACHED
-    assert plan_of(8, 128 << 20).info.keep_lowp_cached              # exactly 2 GiB
-    large = plan_of(9, 128 << 20)                                   # 2.25 GiB
-    assert not large.info.keep_lowp_cached and large.info.flags == 0
-    assert not plan_of(2, 64 << 20, device_resident=False).info.keep_lowp_cached
-    assert not plan_of(1, 1 << 20, lowp=False).info.keep_lowp_cached
+    small = plan_of(2, 64 << 20)                     # 256 MiB of fp16 shards, 1.75 GiB of state
+    assert small.info.cache_policy == 1 and small.info.flags == lowp_flag
+    assert plan_of(8, 128 << 20).info.cache_policy == 1              # exactly 2 GiB of shards
+    large = plan_of(9, 128 << 20)                                    # 2.25 GiB
+    assert large.info.cache_policy == 0 and large.info.flags == 0
+    assert plan_of(2, 64 << 20, device_resident=False).info.cache_policy == 0
+    # the whole state: 14 B per element with the gradients in the low-precision shard, 16 B for a flat fp32
+    # parameter with fp32 gradients
+    tiny = plan_of(1, (256 << 20) // 14 // 1024 * 1024)
+    assert tiny.info.cache_policy == 2 and tiny.info.flags == state_flags
+    assert plan_of(1, (256 << 20) // 14 // 1024 * 1024 + 1024).info.cache_policy == 1
+    flat = plan_of(1, 1 << 24, lowp=False)           # configuration 1: 4 x 64 MiB
+    assert flat.info.cache_policy == 2 and flat.info.flags == state_flags and flat.info.keep_state_cached
+    assert plan_of(1, (1 << 24) + 1024, lowp=False).info.cache_policy == 0
+    assert plan_of(1, 1 << 24, lowp=False, device_resident=False).info.cache_policy == 0
     # what elx_check_tables reports carries no choice
     info = _abi.check_tables(small.rows, small.segs, 1, _abi.ELX_F16, _abi.ELX_F16)
-    assert not info.keep_lowp_cached and info.with_keep_lowp_cached(True).flags == _abi.ELX_FLAG_KEEP_CACHED
-    assert info.with_keep_lowp_cached(True)[:3] == tuple(info)
+    assert info.cache_policy == 0 and not info.keep_lowp_cached and info.with_keep_lowp_cached(True).flags == lowp_flag
+    assert info.with_cache_policy(2).flags == state_flags and info.with_cache_policy(2)[:3] == tuple(info)
 
 
 def test_launch_plan_keeps_rows_bounded_for_the_large_workloads():
