@@ -35,8 +35,8 @@ BYTES_STATS = 2                 # per valid element: the compulsory second read 
 # first 16 hex digits), and the line names the summary it comes from.
 RECORDED_TRAFFIC = {
     # workload: (bytes per launch, summary under profiles/, kernel source the counters were read on)
-    'c5': (94.411e9 + 94.364e9, 'profiles/adam_step_kernel_c5_llama7b.md', '1bf9630de3c9d9ed'),
-    'c4': (18.4445e9 + 18.4305e9, 'profiles/all_kernels_c4_opt1b3_c2_gpt2_c1.md', '1bf9630de3c9d9ed'),
+    'c5': (94.411e9 + 94.364e9, 'profiles/adam_step_kernel_c5_llama7b.md', 'f71d1dd64ff960a3'),
+    'c4': (18.4445e9 + 18.4305e9, 'profiles/all_kernels_c4_opt1b3_c2_gpt2_c1.md', 'f71d1dd64ff960a3'),
 }
 KERNEL_SOURCE = os.path.join(ROOT, 'elixir_amd', 'csrc', 'elx_kernels.hip')
 
@@ -310,8 +310,9 @@ def config1_line(args, with_cpu: bool = True):
     """Configuration 1: plain fp32 Adam on one flat buffer of 16,777,216 elements (p ~ N(0, 0.02),
     g ~ N(0, 1e-2), m = v = 0 at the start, lr 1e-3, betas (0.9, 0.999), eps 1e-8, no weight decay,
     no loss scale, no stats pass, no low-precision copy) -- the case torch.optim.Adam runs on the
-    CPU.  28 B per element: read p, g, m, v, write p, m, v.  The whole state (268 MB) is about the
-    size of the last-level cache, so this line says little about HBM; it is the latency case.
+    CPU.  28 B per element: read p, g, m, v, write p, m, v.  The whole state (256 MiB) is exactly the
+    size of the memory-side cache and the launch keeps it there between steps (ELX_FLAG_KEEP_STATE_CACHED),
+    so this line says little about HBM; it is the latency case.
     The timed steps carry no event records; the launch itself is timed in extra steps afterwards."""
     import elixir_amd as ea
     n = 1 << 24
