@@ -1153,6 +1153,9 @@ Unscale unscale_of(float div_scale) {
     return us;
 }
 
+// flag bits an update launch understands
+constexpr uint32_t kUpdateFlags = ELX_FLAG_SCALAR_ONLY | ELX_FLAG_KEEP_CACHED | ELX_FLAG_KEEP_STATE_CACHED;
+
 // dynamic LDS bytes that let exactly `blocks_per_cu` update workgroups share a compute unit
 int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes, uint32_t fallback = kDefaultBlocksPerCu) {
     if (blocks_per_cu == 0) blocks_per_cu = fallback;
@@ -1499,6 +1502,7 @@ int elx_adam_step_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxSeg *
     if (grid_tiles_per_chunk == 0 || (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    if (flags & ~kUpdateFlags) return ELX_E_RANGE;
     uint32_t lds = 0;
     if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
         return rc;
@@ -1521,6 +1525,7 @@ int elx_adam_step_put_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const ElxS
     if (grid_tiles_per_chunk == 0 || (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    if (flags & ~kUpdateFlags) return ELX_E_RANGE;
     uint32_t lds = 0;
     if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
         return rc;
@@ -1556,6 +1561,7 @@ int elx_adam_step_gated_mt(const ElxChunk *d_chunks, uint32_t n_chunks, const El
     if (grid_tiles_per_chunk == 0 || (uint64_t)grid_tiles_per_chunk * n_chunks < total_tiles) return ELX_E_TILES;
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
+    if (flags & ~kUpdateFlags) return ELX_E_RANGE;
     uint32_t lds = 0;
     if (int rc = occupancy_reservation(blocks_per_cu, &lds, grad_dtype == ELX_F32 ? kDefaultBlocksPerCu : kDefaultBlocksPerCuLowp))
         return rc;

@@ -263,7 +263,8 @@ uint32_t elx_max_ctl_hypers(void);
  * elx_grad_stats_mt.
  *   - n_chunks * blocks_per_chunk must not exceed elx_static_partials(): ELX_E_SIZE otherwise;
  *   - the device that owns `stream` must be the current device of the calling thread (the array's
- *     address is looked up once per device, on the first call there);
+ *     address is looked up once per device, on the first call there: make that first call outside
+ *     stream capture, later ones may be captured);
  *   - all calls on one GPU share the array: two calls whose work overlaps on that GPU (different
  *     streams, or different threads) race.  Calls on one stream are ordered and safe; the array keeps
  *     the last call's partials, and every record a call reads it has written first.
@@ -292,7 +293,8 @@ uint32_t elx_static_partials(void);
  *                          elx_check_tables reported; 0, or a grid that cannot hold total_tiles, is
  *                          ELX_E_TILES.  n_chunks <= 65535: list a long shard as several records
  *   flags          0, ELX_FLAG_SCALAR_ONLY (elx_check_tables found a base pointer that is not 16-byte
- *                  aligned), ELX_FLAG_KEEP_CACHED / ELX_FLAG_KEEP_STATE_CACHED (cache policy, above), or a sum
+ *                  aligned), ELX_FLAG_KEEP_CACHED / ELX_FLAG_KEEP_STATE_CACHED (cache policy, above), or a sum;
+ *                  any other bit is ELX_E_RANGE
  *   blocks_per_cu  cap on resident workgroups per compute unit, 3..32; 0 = the library default (13 for
  *                  16-bit gradients, 12 for fp32 gradients).
  *                  The update streams best with a shallow, orderly queue of memory requests.

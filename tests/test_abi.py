@@ -126,6 +126,11 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     # a grid of zero tiles per record is refused, by both update entry points
     assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 0, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -6
     assert lib.elx_adam_step_gated_mt(1, 1, None, 0, None, 0, 4, 0, _abi.ELX_F16, _abi.ELX_F16, 0, 0, None) == -6
+    # flags of the update launches: scalar-only (1), the two cache policies (2, 4) and their sums; other bits are refused
+    assert lib.elx_adam_step_mt(1, 1, None, 0, None, 0, 4, 4, -1.0, _abi.ELX_F16, _abi.ELX_F16, 8, 0, None) == -4
+    assert lib.elx_adam_step_gated_mt(1, 1, None, 0, None, 0, 4, 4, _abi.ELX_F16, _abi.ELX_F16, 16, 0, None) == -4
+    assert lib.elx_adam_step_put_mt(8, 1, None, 0, 8, 8, 1, 4, 4, -1.0, _abi.ELX_F16, _abi.ELX_F16, 0x100, 0, None) == -4
+    assert _abi.ELX_FLAG_KEEP_STATE_CACHED == 4
     assert lib.elx_writeback_mt(None, 1, _abi.ELX_F16, 4, 0, None) == -1
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_NONE, 4, 0, None) == -2
     assert lib.elx_writeback_mt(1, 1, _abi.ELX_F16, 0, 0, None) == -7
