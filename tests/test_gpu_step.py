@@ -243,13 +243,28 @@ def test_flat_fp16_grads_fp32_params(oracle):
     assert np.array_equal(to_np(p.data).view(np.uint32), pn.view(np.uint32))
 
 
+def _cache_policy_of_seed(monkeypatch, seed: int) -> int:
+    """The seeded tests run on sets so small that every update launch would take the third cache policy
+    (the state fits the memory-side cache).  One seed in three keeps it, one runs with only the
+    low-precision copy stored through the cache, one streams everything: the plan reads the thresholds
+    when it is built, at the first step."""
+    from elixir_amd import launch_plan
+    policy = (2, 1, 0)[seed % 3]
+    if policy < 2:
+        monkeypatch.setattr(launch_plan, 'KEEP_STATE_CACHED_BELOW', -1)
+    if policy < 1:
+        monkeypatch.setattr(launch_plan, 'KEEP_LOWP_CACHED_BELOW', -1)
+    return policy
+
+
 @pytest.mark.parametrize('seed', seeds(12))
-def test_flat_random_hypers_match_oracle(oracle, seed):
+def test_flat_random_hypers_match_oracle(oracle, seed, monkeypatch):
     """Hyper-parameters, gradient type and divisor drawn at random, the edges included (beta1 of 0 and
     of exactly 0.5, beta2 of 0, no bias correction, a divisor that is not a power of two, two groups
     in one launch): identical bits to the oracle over four steps."""
     rng = np.random.default_rng(9100 + seed)
     gdtype = [torch.float32, torch.float16, torch.bfloat16][seed % 3]
+    _cache_policy_of_seed(monkeypatch, seed // 3)
     adamw = bool(rng.integers(2))
     groups = []
     for _ in range(2):
@@ -608,11 +623,12 @@ def test_abi_rejects_bad_tables():
 
 
 @pytest.mark.parametrize('seed', seeds(16))
-def test_random_layouts_match_oracle(oracle, seed):
+def test_random_layouts_match_oracle(oracle, seed, monkeypatch):
     """Whatever the packing looks like -- boundaries inside vectors, tensors of one element, chunks
     that are not a multiple of the tile, a padded tail or none -- an unclipped step is bit-identical
     to the oracle's, over two steps (the second with new gradients and warm state)."""
     rng = np.random.default_rng(1000 + seed)
+    policy = _cache_policy_of_seed(monkeypatch, seed // 3)    # the dtype below goes by seed % 3: cross the two
     n_tensors = int(rng.integers(1, 24))
     kinds = rng.integers(0, 4, n_tensors)
     sizes = [int({0: rng.integers(1, 9), 1: rng.integers(9, 700), 2: rng.integers(700, 9000),
@@ -642,10 +658,11 @@ def test_random_layouts_match_oracle(oracle, seed):
         info = _run_and_compare(module, opt, ochunks, dtype, scaler, adamw_mode=adamw, tag=f'seed {seed} step {step}')
         assert info['found_inf'] is False
         assert compare_state(module, opt, ochunks, dtype, exact=True, tag=f'seed {seed} step {step}') == 0
+    assert all(dp.plan.info.cache_policy == policy for dp in opt.optim._plans.values())
 
 
 @pytest.mark.parametrize('seed', seeds(12))
-def test_random_trajectories_match_oracle(oracle, seed):
+def test_random_trajectories_match_oracle(oracle, seed, monkeypatch):
     """Seven steps on a random layout with everything drawn at random: hysteresis and growth interval of
     the scaler, clipping threshold, non-finite values in valid data (skip, back-off) or in the padding
     (must not count), gradients landed by the fused launch or written into the shards, the step decided
@@ -654,6 +671,7 @@ def test_random_trajectories_match_oracle(oracle, seed):
     compared on its own), and the low-precision copy is always the exact cast of the master."""
     from elixir_amd.chunk import land_chunks
     rng = np.random.default_rng(50_000 + seed)
+    _cache_policy_of_seed(monkeypatch, seed // 2)    # the dtype below goes by seed % 2
     n_tensors = int(rng.integers(1, 16))
     sizes = [int(rng.choice([rng.integers(1, 9), rng.integers(9, 700), rng.integers(700, 9000), rng.integers(9000, 40000)]))
              for _ in range(n_tensors)]
