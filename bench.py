@@ -640,6 +640,9 @@ def main():
         print('bench.py needs a GPU: the optimizer step has no CPU path', file=sys.stderr)
         sys.exit(2)
 
+    from elixir_amd.build import ensure_built
+    ensure_built()    # loads what is built; compiles only a tree that was never built
+
     if args.offload_step > 0:
         print(json.dumps(offload_step_leg(args.offload_step)))
         return

@@ -42,6 +42,15 @@ def build(verbose: bool = True) -> str:
     return OUTPUT
 
 
+def ensure_built(verbose: bool = False) -> str:
+    """For test runs, the smoke check and the benchmark: compiles the library only when no built one is
+    there (a tree that was never built).  The product itself never builds behind the caller's back:
+    ``elixir_amd._abi.load`` raises when the library is missing."""
+    if not os.path.exists(OUTPUT):
+        build(verbose=verbose)
+    return OUTPUT
+
+
 if __name__ == '__main__':
     build()
     sys.exit(0)
