@@ -111,6 +111,36 @@ def cpu_baseline(built, sample_elems: int, steps: int = 8):
     }
 
 
+def cpu_baseline_whole_set(built, steps: int = 5):
+    """The torch CPU step of ``cpu_baseline`` over EVERY chunk of the set, one chunk after the other (for a set
+    small enough to do so: the GPT-2 one).  No extrapolation: the time of a step is the sum over the chunks."""
+    from oracle.torch_ref import TorchCpuStep
+    spec = built.spec
+    assert spec.max_norm == 0.0, 'a clipped step needs the global norm first; this helper times unclipped sets'
+    total = 0.0
+    for pc, g_dev in zip(built.module.param_chunks, built.grads):
+        oc = pc.paired_chunk
+        n = pc.utilized_size
+        m, v = built.optimizer._binding.moments(oc)
+        ref = TorchCpuStep(oc.shard[:n].cpu(), spec.dtype, lr=spec.lr, betas=spec.betas, eps=spec.eps,
+                           weight_decay=spec.weight_decay, adamw_mode=spec.adamw_mode, exp_avg=m[:n].cpu(),
+                           exp_avg_sq=v[:n].cpu())
+        g = g_dev[:n].cpu()
+        times = []
+        for _ in range(steps + 1):
+            t0 = time.perf_counter()
+            ref.step(g, loss_scale=spec.loss_scale, max_norm=0.0)
+            times.append(time.perf_counter() - t0)
+        total += float(np.median(times[1:]))
+        del ref, g
+    return {
+        'value': built.n_valid / total, 'unit': 'elements/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+        'sample': f'the whole configuration, {len(built.grads)} chunks one after the other: torch CPU ops (isinf/isnan, '
+                  f'float().div_, torch.optim.Adam, .to(lowp)); per chunk the median of {steps} steps after 1 warm-up',
+        'extrapolation': 'none: full size', 'ms_per_step_sample': total * 1e3,
+    }
+
+
 def fused_landing_leg(built, steps):
     """The same step when the gradients arrive through the landing launch that leaves the flags on
     the device: the step then holds no pass over the gradients (28 B per valid element).  Reports
@@ -710,6 +740,8 @@ def main():
             line, b = chunk_set_line(small, name, device, events_in_timed_steps=False)
             if name == 'c2':
                 configs['c3'] = skip_step_leg(b)
+                if args.cpu_sample > 0:
+                    line['cpu_baseline'] = cpu_baseline_whole_set(b)
             del b
             free_device_memory()
             configs[name] = summary_of(line)
