@@ -368,6 +368,14 @@ def config1_line(args, with_cpu: bool = True):
             ev = opt.kernel_events['adam_step']
             adam_ms.append(ev[0].elapsed_time(ev[1]))
     opt.kernel_events = None
+    # K steps in one bracket: nothing has to happen between two steps of this configuration (the gradient
+    # stays where it is), so the launches can queue up behind each other and the host's share disappears
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        opt.step()
+    torch.cuda.synchronize()
+    t_queued = (time.perf_counter() - t0) / args.steps
     # the same step with the memory-side cache emptied in front of it (a 1 GiB device copy, as the forward and
     # backward pass of a training loop would leave it): what the step costs when its state comes from HBM
     junk = torch.empty(2, 256 << 20, dtype=torch.float32, device='cuda')
@@ -391,6 +399,8 @@ def config1_line(args, with_cpu: bool = True):
                                'copy', 'valid_elements': n},
         'step': {'ms_min': float(np.min(step_s)) * 1e3, 'gbps_28B': BYTES_UPDATE * n / t_step / 1e9,
                  'frac_28B': BYTES_UPDATE * n / t_step / 1e9 / HBM_PEAK_GBPS},
+        'steps_back_to_back': {'what': f'{args.steps} steps between one pair of synchronisations, nothing between them',
+                               'ms_per_step': t_queued * 1e3, 'frac_28B': BYTES_UPDATE * n / t_queued / 1e9 / HBM_PEAK_GBPS},
         'step_cold_cache': {'what': 'the same step behind a 1 GiB device copy that empties the memory-side cache',
                             'ms_per_step': t_cold * 1e3, 'ms_min': float(np.min(cold_s)) * 1e3,
                             'frac_28B': BYTES_UPDATE * n / t_cold / 1e9 / HBM_PEAK_GBPS},
@@ -646,6 +656,7 @@ def summary_of(line):
         keep['vs_baseline'] = line['vs_baseline']
     if 'step_cold_cache' in line:
         keep['step_cold_cache_ms'] = line['step_cold_cache']['ms_per_step']
+        keep['steps_back_to_back_ms'] = line['steps_back_to_back']['ms_per_step']
         keep['state_stays_in_memory_side_cache'] = True
     if 'cpu_baseline' in line:
         keep['cpu_baseline'] = line['cpu_baseline']
