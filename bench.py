@@ -182,6 +182,33 @@ def fused_landing_leg(built, steps):
             step_s.append(dt)
     t_step, t_land, t_plain = float(np.mean(step_s)), float(np.mean(land_s)), float(np.mean(plain_s))
 
+    # the flow of a training loop: backward lands every chunk with a launch of its own as soon as its last
+    # gradient exists, the last chunk first; the records still end up side by side (the optimizer gave every
+    # chunk its slot in chunk order) and the step is decided on the device
+    from elixir_amd.chunk import land_chunks
+    pc_land_s, pc_step_s = [], []
+    for i in range(steps + 1):
+        for pc in chunks:
+            pc.invalidate_stats()
+
+        def one_by_one():
+            for pc, g in zip(reversed(chunks), reversed(built.grads)):
+                land_chunks([pc], [g])
+
+        t_pc_land = timed(one_by_one)
+        opt.mark_gradients_scaled()
+        torch.cuda.synchronize()
+        assert opt._stats_source()[0] == 'arena'
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert opt.last_step_info['found_inf'] is False
+        if i > 0:
+            pc_land_s.append(t_pc_land)
+            pc_step_s.append(dt)
+    t_pc_step, t_pc_land = float(np.mean(pc_step_s)), float(np.mean(pc_land_s))
+
     # the same landing straight from per-tensor gradients (views of the saved buffers stand in for
     # the .grad tensors), next to what it replaces: a zeroed payload per chunk, one slice copy per
     # tensor, and the copy of the payload into the shard
@@ -198,6 +225,19 @@ def fused_landing_leg(built, steps):
                 payload[info.offset:info.end].copy_(grads[t])
             pc.shard.copy_(payload)
 
+    blocker = torch.empty(2, 1 << 30, dtype=torch.uint8, device=chunks[0].shard_device)
+
+    def behind_blocker(fn):
+        """Device time of what ``fn`` enqueues: a 1 GiB copy runs in front, so that the host's part of ``fn``
+        (building the row table) is over before the device gets to its launches."""
+        b, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        blocker[1].copy_(blocker[0])
+        b.record()
+        fn()
+        e.record()
+        e.synchronize()
+        return b.elapsed_time(e) * 1e-3
+
     pt_gpu, pt_wall, sc_gpu = [], [], []
     for i in range(steps + 1):
         a = timed(slice_copies)
@@ -205,12 +245,17 @@ def fused_landing_leg(built, steps):
             pc.invalidate_stats()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        b = timed(lambda: land_tensors(chunks, lambda t: grads[t]))
+        land_tensors(chunks, lambda t: grads[t])
+        torch.cuda.synchronize()
         w = time.perf_counter() - t0
+        for pc in chunks:
+            pc.invalidate_stats()
+        b = behind_blocker(lambda: land_tensors(chunks, lambda t: grads[t]))
         if i > 0:
             sc_gpu.append(a)
             pt_gpu.append(b)
             pt_wall.append(w)
+    del blocker
     assert not any(pc.overflow for pc in chunks)
     return {
         'what': 'gradients landed by land_grads_kernel (copy + flags in one pass, outside the step); '
@@ -220,6 +265,14 @@ def fused_landing_leg(built, steps):
         'elements_per_sec': n_valid / t_step,
         'step_gbps_28B': BYTES_UPDATE * n_valid / t_step / 1e9,
         'step_frac_28B': BYTES_UPDATE * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
+        'per_chunk_landing': {
+            'what': 'every chunk landed by a launch of its own, the last chunk first (what the hooks of backward do); '
+                    'the step that follows is decided on the device all the same',
+            'launches': len(chunks),
+            'landing_ms_all_chunks': t_pc_land * 1e3,
+            'ms_per_step': t_pc_step * 1e3,
+            'step_frac_28B': BYTES_UPDATE * n_valid / t_pc_step / 1e9 / HBM_PEAK_GBPS,
+        },
         'land_kernel': {
             'kernel': 'land_grads_kernel+stats_fold_kernel+stats_finish_kernel',
             'ms_per_launch': t_land * 1e3,
@@ -231,7 +284,10 @@ def fused_landing_leg(built, steps):
         },
         'per_tensor_landing': {
             'what': 'the same launch fed by one row list over the %d per-tensor gradients (no payload)' % len(grads),
-            'ms_launch_to_done': float(np.mean(pt_gpu)) * 1e3,
+            'ms_on_device': float(np.mean(pt_gpu)) * 1e3,
+            'ms_min_on_device': float(np.min(pt_gpu)) * 1e3,
+            'frac_of_hbm_peak': 2 * esize * n_alloc / float(np.mean(pt_gpu)) / 1e9 / HBM_PEAK_GBPS,
+            'vs_payload_landing': float(np.mean(pt_gpu)) / t_land,
             'ms_wall_with_table_build': float(np.mean(pt_wall)) * 1e3,
             'zero_payload_slice_copies_and_shard_copy_ms': float(np.mean(sc_gpu)) * 1e3,
         },
@@ -336,14 +392,39 @@ def offload_step_leg(mi_elements, steps=5):
     return out
 
 
+def launch_sync_floor_us(samples: int = 200) -> float:
+    """What the machine charges for ANY step, however short its kernel: one launch of a single wavefront
+    that writes 48 bytes (elx_put_hypers with one record) between two device synchronisations; the median
+    over ``samples`` in microseconds.  Launch latency on the way in, completion signal and wake-up on the
+    way out."""
+    from elixir_amd import _abi
+    from elixir_amd.hybrid_adam import make_hyper_record
+    lib = _abi.load()
+    rec = make_hyper_record(1e-3, 0.9, 0.999, 1e-8, 0.0, 1, True, True)
+    src = rec.ctypes.data
+    dst = torch.zeros(64, dtype=torch.uint8, device='cuda')
+    d_ptr = dst.data_ptr()
+    stream = torch.cuda.current_stream().cuda_stream
+    ts = []
+    for i in range(samples + 20):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        lib.elx_put_hypers(src, 1, d_ptr, stream)
+        torch.cuda.synchronize()
+        ts.append(time.perf_counter() - t0)
+    return float(np.median(ts[20:])) * 1e6
+
+
 def config1_line(args, with_cpu: bool = True):
     """Configuration 1: plain fp32 Adam on one flat buffer of 16,777,216 elements (p ~ N(0, 0.02),
     g ~ N(0, 1e-2), m = v = 0 at the start, lr 1e-3, betas (0.9, 0.999), eps 1e-8, no weight decay,
     no loss scale, no stats pass, no low-precision copy) -- the case torch.optim.Adam runs on the
     CPU.  28 B per element: read p, g, m, v, write p, m, v.  The whole state (256 MiB) is exactly the
-    size of the memory-side cache and the launch keeps it there between steps (ELX_FLAG_KEEP_STATE_CACHED),
-    so this line says little about HBM; it is the latency case.
-    The timed steps carry no event records; the launch itself is timed in extra steps afterwards."""
+    size of the memory-side cache and the launch keeps it there between steps (ELX_FLAG_KEEP_STATE_CACHED).
+    The line's own figure is the step a training loop sees: behind a 1 GiB device copy that empties that
+    cache, as a forward and backward pass would (`value`, `ms_per_step`, `roofline`); the step that finds
+    its state still in the cache, and steps queued back to back, stand beside it.  The timed steps carry no
+    event records; the launch itself is timed in extra steps afterwards."""
     import elixir_amd as ea
     n = 1 << 24
     gen = torch.Generator(device='cuda')
@@ -352,22 +433,33 @@ def config1_line(args, with_cpu: bool = True):
     g = torch.randn(n, device='cuda', generator=gen) * 1e-2
     opt = ea.HybridAdam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
     p.grad = g
-    step_s, adam_ms = [], []
+    junk = torch.empty(2, 256 << 20, dtype=torch.float32, device='cuda')
     extra = 6
-    for i in range(args.warmup + args.steps + extra):
-        if i == args.warmup + args.steps:
-            opt.kernel_events = {}
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        opt.step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        if args.warmup <= i < args.warmup + args.steps:
-            step_s.append(dt)
-        elif i > args.warmup + args.steps:    # the first instrumented step creates the event pair
-            ev = opt.kernel_events['adam_step']
-            adam_ms.append(ev[0].elapsed_time(ev[1]))
-    opt.kernel_events = None
+
+    def timed_steps(cold: bool):
+        step_s, call_s, adam_ms = [], [], []
+        for i in range(args.warmup + args.steps + extra):
+            if i == args.warmup + args.steps:
+                opt.kernel_events = {}
+            if cold:
+                junk[1].copy_(junk[0])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            opt.step()
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            if args.warmup <= i < args.warmup + args.steps:
+                step_s.append(dt)
+                call_s.append(t1 - t0)
+            elif i > args.warmup + args.steps:    # the first instrumented step creates the event pair
+                ev = opt.kernel_events['adam_step']
+                adam_ms.append(ev[0].elapsed_time(ev[1]))
+        opt.kernel_events = None
+        return step_s, call_s, float(np.mean(adam_ms)) * 1e-3
+
+    warm_s, warm_call_s, t_upd_warm = timed_steps(cold=False)
+    cold_s, cold_call_s, t_upd_cold = timed_steps(cold=True)
     # K steps in one bracket: nothing has to happen between two steps of this configuration (the gradient
     # stays where it is), so the launches can queue up behind each other and the host's share disappears
     torch.cuda.synchronize()
@@ -376,39 +468,44 @@ def config1_line(args, with_cpu: bool = True):
         opt.step()
     torch.cuda.synchronize()
     t_queued = (time.perf_counter() - t0) / args.steps
-    # the same step with the memory-side cache emptied in front of it (a 1 GiB device copy, as the forward and
-    # backward pass of a training loop would leave it): what the step costs when its state comes from HBM
-    junk = torch.empty(2, 256 << 20, dtype=torch.float32, device='cuda')
-    cold_s = []
-    for i in range(args.steps + 2):
-        junk[1].copy_(junk[0])
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        opt.step()
-        torch.cuda.synchronize()
-        if i >= 2:
-            cold_s.append(time.perf_counter() - t0)
     del junk
-    t_cold = float(np.mean(cold_s))
-    t_step, t_upd = float(np.mean(step_s)), float(np.mean(adam_ms)) * 1e-3
+    floor_us = launch_sync_floor_us()
+    t_cold, t_warm = float(np.mean(cold_s)), float(np.mean(warm_s))
+    host_us = float(np.median(cold_call_s)) * 1e6
     out = {
-        'metric': 'adam_elements_per_sec', 'value': n / t_step, 'unit': 'elements/s', 'n_gpus': 1, 'steps': args.steps,
-        'warmup': args.warmup, 'ms_per_step': t_step * 1e3, 'higher_is_better': True, 'scaling': 'weak',
+        'metric': 'adam_elements_per_sec', 'value': n / t_cold, 'unit': 'elements/s', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': t_cold * 1e3, 'higher_is_better': True, 'scaling': 'weak',
         'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
         'config': {'workload': 'c1: plain fp32 Adam, one flat buffer of 16Mi elements, no loss scale, no low-precision '
-                               'copy', 'valid_elements': n},
-        'step': {'ms_min': float(np.min(step_s)) * 1e3, 'gbps_28B': BYTES_UPDATE * n / t_step / 1e9,
-                 'frac_28B': BYTES_UPDATE * n / t_step / 1e9 / HBM_PEAK_GBPS},
+                               'copy; every step behind a 1 GiB device copy that empties the memory-side cache',
+                   'valid_elements': n},
+        'step': {'ms_min': float(np.min(cold_s)) * 1e3, 'gbps_28B': BYTES_UPDATE * n / t_cold / 1e9,
+                 'frac_28B': BYTES_UPDATE * n / t_cold / 1e9 / HBM_PEAK_GBPS},
+        'launch_sync_floor_us': floor_us,
+        'host_us_in_step': host_us,
+        'step_accounting_us': {
+            'what': 'step = update launch + what any launch between two synchronisations costs (launch_sync_floor_us, '
+                    'which already holds the host call of a launch) + what the host does in step() beyond such a call',
+            'step': t_cold * 1e6, 'update_launch': t_upd_cold * 1e6, 'launch_sync_floor': floor_us,
+            'host_call_of_step': host_us,
+            'unaccounted': t_cold * 1e6 - t_upd_cold * 1e6 - floor_us,
+            'steady_path_taken': opt._steady is not None,
+        },
+        'step_state_in_cache': {'what': 'the same step when nothing ran between two steps: the 256 MiB of state are '
+                                        'still in the memory-side cache',
+                                'ms_per_step': t_warm * 1e3, 'ms_min': float(np.min(warm_s)) * 1e3,
+                                'frac_28B': BYTES_UPDATE * n / t_warm / 1e9 / HBM_PEAK_GBPS,
+                                'update_launch_ms': t_upd_warm * 1e3,
+                                'update_launch_frac': BYTES_UPDATE * n / t_upd_warm / 1e9 / HBM_PEAK_GBPS},
         'steps_back_to_back': {'what': f'{args.steps} steps between one pair of synchronisations, nothing between them',
                                'ms_per_step': t_queued * 1e3, 'frac_28B': BYTES_UPDATE * n / t_queued / 1e9 / HBM_PEAK_GBPS},
-        'step_cold_cache': {'what': 'the same step behind a 1 GiB device copy that empties the memory-side cache',
+        'step_cold_cache': {'what': 'the line\'s own figure (kept under this name for comparison with earlier lines)',
                             'ms_per_step': t_cold * 1e3, 'ms_min': float(np.min(cold_s)) * 1e3,
                             'frac_28B': BYTES_UPDATE * n / t_cold / 1e9 / HBM_PEAK_GBPS},
-        'roofline': {'kernel': 'adam_step_kernel', 'bound': 'hbm', 'achieved': BYTES_UPDATE * n / t_upd / 1e9,
-                     'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': BYTES_UPDATE * n / t_upd / 1e9 / HBM_PEAK_GBPS,
-                     'traffic': None, 'bytes_per_launch': BYTES_UPDATE * n, 'ms_per_launch': t_upd * 1e3,
-                     'timed_in': f'{extra - 1} extra steps after the timed ones',
-                     'note': 'the 256 MiB of state stay in the memory-side cache between these steps: see step_cold_cache'},
+        'roofline': {'kernel': 'adam_step_kernel', 'bound': 'hbm', 'achieved': BYTES_UPDATE * n / t_upd_cold / 1e9,
+                     'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': BYTES_UPDATE * n / t_upd_cold / 1e9 / HBM_PEAK_GBPS,
+                     'traffic': None, 'bytes_per_launch': BYTES_UPDATE * n, 'ms_per_launch': t_upd_cold * 1e3,
+                     'timed_in': f'{extra - 1} extra steps after the timed ones, each behind the cache-emptying copy'},
     }
     if with_cpu:
         # the reference's own path for this configuration: torch.optim.Adam on CPU tensors, full size
@@ -652,12 +749,20 @@ def summary_of(line):
     if 'fused_landing' in line:
         keep['step_after_fused_landing_ms'] = line['fused_landing']['ms_per_step']
         keep['step_after_fused_landing_frac_28B'] = line['fused_landing']['step_frac_28B']
+        keep['step_after_per_chunk_landing_ms'] = line['fused_landing']['per_chunk_landing']['ms_per_step']
+        keep['per_chunk_landing'] = line['fused_landing']['per_chunk_landing']
+        keep['payload_landing_ms'] = line['fused_landing']['land_kernel']['ms_per_launch']
+        keep['payload_landing_frac'] = line['fused_landing']['land_kernel']['frac']
+        keep['per_tensor_landing'] = line['fused_landing']['per_tensor_landing']
     if line.get('vs_baseline') is not None:
         keep['vs_baseline'] = line['vs_baseline']
     if 'step_cold_cache' in line:
         keep['step_cold_cache_ms'] = line['step_cold_cache']['ms_per_step']
+        keep['step_state_in_cache_ms'] = line['step_state_in_cache']['ms_per_step']
         keep['steps_back_to_back_ms'] = line['steps_back_to_back']['ms_per_step']
-        keep['state_stays_in_memory_side_cache'] = True
+        keep['launch_sync_floor_us'] = line['launch_sync_floor_us']
+        keep['host_us_in_step'] = line['host_us_in_step']
+        keep['step_accounting_us'] = line['step_accounting_us']
     if 'cpu_baseline' in line:
         keep['cpu_baseline'] = line['cpu_baseline']
     return keep

@@ -10,12 +10,13 @@ from typing import Optional
 
 import numpy as np
 
-ELX_ABI_VERSION = 2
+ELX_ABI_VERSION = 3
 ELX_F32, ELX_F16, ELX_BF16, ELX_NONE = 0, 1, 2, -1
 ELX_FLAG_SCALAR_ONLY = 1
 ELX_FLAG_KEEP_CACHED = 2
 ELX_FLAG_KEEP_STATE_CACHED = 4
-ELX_E_NULL, ELX_E_DTYPE, ELX_E_ALIGN, ELX_E_RANGE, ELX_E_ORDER, ELX_E_TILES, ELX_E_SIZE = -1, -2, -3, -4, -5, -6, -7
+ELX_E_NULL, ELX_E_DTYPE, ELX_E_ALIGN, ELX_E_RANGE, ELX_E_ORDER, ELX_E_TILES, ELX_E_SIZE, ELX_E_STATE = -1, -2, -3, -4, -5, -6, -7, -8
+MAX_ARG_HYPERS = 32    # hyper records that ride in the arguments of an update launch (elx_adam_step_put_mt)
 ELX_HYPER_L2 = 1
 ELX_HYPER_LERP_FROM_G = 2
 
@@ -45,7 +46,42 @@ EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 
            'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems',
            'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
            'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers',
-           'elx_adam_step_put_mt')
+           'elx_adam_step_put_mt', 'elx_source_sha', 'elx_unscale_mode', 'elx_occupancy_lds_bytes')
+
+# what the validators' own build (the host-only source under sanitizers) exports
+HOST_EXPORTS = ('elx_check_tables', 'elx_check_land_rows', 'elx_tile_elems', 'elx_land_tile_elems', 'elx_land_max_blocks',
+                'elx_unscale_mode', 'elx_occupancy_lds_bytes', 'elx_source_sha')
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc')
+_HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), 'include', 'elx_abi.h')
+
+
+def source_files():
+    """The files a build of the library is made from, in the order their digest is taken."""
+    files = [os.path.join(_CSRC, f) for f in sorted(os.listdir(_CSRC)) if f.endswith(('.hip', '.cpp', '.h'))]
+    return files + [_HEADER]
+
+
+def source_sha16() -> str:
+    """First 16 hex digits of the SHA-256 over the library's sources as they are now."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in source_files():
+        h.update(os.path.basename(path).encode() + b'\0')
+        with open(path, 'rb') as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def built_source_sha(lib_path: str) -> str:
+    """The digest a built library carries ('' when it has none)."""
+    try:
+        L = ctypes.CDLL(lib_path)
+        L.elx_source_sha.restype = ctypes.c_char_p
+        L.elx_source_sha.argtypes = []
+        return (L.elx_source_sha() or b'').decode()
+    except (OSError, AttributeError):
+        return ''
 
 
 class ElxError(RuntimeError):
@@ -75,14 +111,13 @@ def load() -> ctypes.CDLL:
     L.elx_strerror.restype = ctypes.c_char_p
     L.elx_strerror.argtypes = [cint]
     for name in ('elx_tile_elems', 'elx_sizeof_chunk', 'elx_sizeof_seg', 'elx_sizeof_hyper', 'elx_sizeof_stats',
-                 'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
-           'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers',
-           'elx_adam_step_put_mt'):
+                 'elx_sizeof_decision', 'elx_refresh_piece_elems', 'elx_land_max_blocks', 'elx_land_fold_blocks',
+                 'elx_static_partials', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers'):
         getattr(L, name).restype = u32
         getattr(L, name).argtypes = []
-    L.elx_check_tables.restype = cint
-    L.elx_check_tables.argtypes = [vp, u32, vp, u32, u32, cint, cint, ctypes.POINTER(u64), ctypes.POINTER(u32),
-                                   ctypes.POINTER(cint)]
+    L.elx_source_sha.restype = ctypes.c_char_p
+    L.elx_source_sha.argtypes = []
+    _bind_host(L)
     L.elx_grad_stats_mt.restype = cint
     L.elx_grad_stats_mt.argtypes = [vp, u32, cint, u32, vp, vp, cint, vp]
     L.elx_grad_partials_mt.restype = cint
@@ -103,19 +138,19 @@ def load() -> ctypes.CDLL:
     L.elx_adam_step_gated_mt.argtypes = [vp, u32, vp, u32, vp, u32, u64, u32, cint, cint, u32, u32, vp]
     L.elx_writeback_mt.restype = cint
     L.elx_writeback_mt.argtypes = [vp, u32, cint, u32, u32, vp]
-    L.elx_land_tile_elems.restype = u32
-    L.elx_land_tile_elems.argtypes = [cint]
     L.elx_writeback.restype = cint
     L.elx_writeback.argtypes = [vp, vp, cint, u64, vp]
     L.elx_grad_stats.restype = cint
     L.elx_grad_stats.argtypes = [vp, cint, u64, u32, vp, vp, vp]
-    L.elx_check_land_rows.restype = cint
-    L.elx_check_land_rows.argtypes = [vp, u32, vp, u32, cint, cint, ctypes.POINTER(u32)]
     L.elx_land_grads_mt.restype = cint
     L.elx_land_grads_mt.argtypes = [vp, u32, vp, u32, cint, cint, flt, u32, vp, vp, u32, vp]
 
     if L.elx_version() != ELX_ABI_VERSION:
         raise RuntimeError(f'{LIB_PATH}: ABI version {L.elx_version()} != binding version {ELX_ABI_VERSION}; rebuild')
+    built, now = (L.elx_source_sha() or b'').decode(), source_sha16()
+    if built != now:
+        raise RuntimeError(f'{LIB_PATH} was built from other sources (digest {built or "none"}) than the ones beside it '
+                           f'({now}): rebuild with `python -m elixir_amd.build`')
     for name, dt in (('chunk', CHUNK_DTYPE), ('seg', SEG_DTYPE), ('hyper', HYPER_DTYPE), ('stats', STATS_DTYPE),
                      ('decision', DECISION_DTYPE), ('step_ctl', STEP_CTL_DTYPE), ('step_report', STEP_REPORT_DTYPE)):
         size = getattr(L, f'elx_sizeof_{name}')()
@@ -125,13 +160,65 @@ def load() -> ctypes.CDLL:
     return L
 
 
+def _bind_host(L) -> None:
+    """Signatures of the entry points that the host-only source file defines."""
+    u32, u64, vp, cint, flt = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    L.elx_check_tables.restype = cint
+    L.elx_check_tables.argtypes = [vp, u32, vp, u32, u32, cint, cint, ctypes.POINTER(u64), ctypes.POINTER(u32),
+                                   ctypes.POINTER(cint)]
+    L.elx_check_land_rows.restype = cint
+    L.elx_check_land_rows.argtypes = [vp, u32, vp, u32, cint, cint, ctypes.POINTER(u32)]
+    L.elx_land_tile_elems.restype = u32
+    L.elx_land_tile_elems.argtypes = [cint]
+    for name in ('elx_tile_elems', 'elx_land_max_blocks'):
+        getattr(L, name).restype = u32
+        getattr(L, name).argtypes = []
+    L.elx_unscale_mode.restype = cint
+    L.elx_unscale_mode.argtypes = [flt, ctypes.POINTER(flt)]
+    L.elx_occupancy_lds_bytes.restype = cint
+    L.elx_occupancy_lds_bytes.argtypes = [u32, ctypes.POINTER(u32)]
+
+
+_host_lib = None
+
+
+def host_lib() -> ctypes.CDLL:
+    """The library whose validators (and other host-only entry points) are called: ``libelx_hip.so``, or --
+    for the test run that puts the validators under AddressSanitizer / UBSan -- the build of the host-only
+    source file that the environment variable ELX_HOST_CHECKED_LIB names."""
+    global _host_lib
+    path = os.environ.get('ELX_HOST_CHECKED_LIB')
+    if not path:
+        return load()
+    if _host_lib is None:
+        L = ctypes.CDLL(path)
+        _bind_host(L)
+        _host_lib = L
+    return _host_lib
+
+
+def unscale_mode(div_scale: float):
+    """(mode, inv_scale): how an update launch divides by ``div_scale`` (0 not at all, 1 exact multiply, 2 division)."""
+    inv = ctypes.c_float(0.0)
+    mode = host_lib().elx_unscale_mode(div_scale, ctypes.byref(inv))
+    return int(mode), float(inv.value)
+
+
+def occupancy_lds_bytes(blocks_per_cu: int) -> int:
+    lds = ctypes.c_uint32(0)
+    code = host_lib().elx_occupancy_lds_bytes(blocks_per_cu, ctypes.byref(lds))
+    if code != 0:
+        raise ElxError('elx_occupancy_lds_bytes', code, load().elx_strerror(code).decode())
+    return int(lds.value)
+
+
 def check(func: str, code: int) -> None:
     if code != 0:
         raise ElxError(func, code, load().elx_strerror(code).decode())
 
 
 def tile_elems() -> int:
-    return int(load().elx_tile_elems())
+    return int(host_lib().elx_tile_elems())
 
 
 def _np_ptr(a: Optional[np.ndarray]):
@@ -196,7 +283,7 @@ def check_tables(chunks: np.ndarray, segs: Optional[np.ndarray], n_hypers: int, 
     tiles = ctypes.c_uint64(0)
     max_tiles = ctypes.c_uint32(0)
     aligned = ctypes.c_int(0)
-    code = load().elx_check_tables(_np_ptr(chunks), len(chunks), _np_ptr(segs), n_segs, n_hypers, grad_dtype, lowp_dtype,
+    code = host_lib().elx_check_tables(_np_ptr(chunks), len(chunks), _np_ptr(segs), n_segs, n_hypers, grad_dtype, lowp_dtype,
                                    ctypes.byref(tiles), ctypes.byref(max_tiles), ctypes.byref(aligned))
     check('elx_check_tables', code)
     return TableInfo((int(tiles.value), int(max_tiles.value), bool(aligned.value)))
@@ -305,7 +392,7 @@ def land_max_blocks() -> int:
 
 
 def land_tile_elems(src_dtype: int) -> int:
-    return int(load().elx_land_tile_elems(src_dtype))
+    return int(host_lib().elx_land_tile_elems(src_dtype))
 
 
 def land_fold_blocks() -> int:
@@ -337,7 +424,7 @@ def check_land_rows(rows: np.ndarray, slot_offsets: Optional[np.ndarray], src_dt
         n_slots = len(slot_offsets) - 1
     bpr = ctypes.c_uint32(0)
     check('elx_check_land_rows',
-          load().elx_check_land_rows(_np_ptr(rows), len(rows), _np_ptr(slot_offsets), n_slots, src_dtype, dst_dtype,
+          host_lib().elx_check_land_rows(_np_ptr(rows), len(rows), _np_ptr(slot_offsets), n_slots, src_dtype, dst_dtype,
                                      ctypes.byref(bpr)))
     return int(bpr.value)
 

@@ -204,6 +204,39 @@ class StatsArena:
         for i, c in enumerate(chunks):
             c._take_stats_slot(self, first + i)
 
+    def pin(self, chunks: List['Chunk']) -> None:
+        """Gives the chunks consecutive slots in list order for as long as they live (an optimizer does this
+        for its parameter chunks, in chunk order): in whatever order and grouping they land afterwards --
+        one launch per chunk from the hooks of backward, last chunk first -- their records end up side by
+        side, where one launch of the step folds them."""
+        if all(c._stats_pinned and c._stats_home[0] is self for c in chunks) and \
+                all(b._stats_slot == a._stats_slot + 1 for a, b in zip(chunks, chunks[1:])):
+            return
+        first = self.new_slots(len(chunks))
+        for i, c in enumerate(chunks):
+            c._take_stats_slot(self, first + i)
+            c._stats_pinned = True
+
+    def runs(self, chunks: List['Chunk']) -> List[List['Chunk']]:
+        """The chunks of one landing cut into runs that one launch each can serve (a launch writes its
+        records into consecutive slots, in list order).  A pinned chunk keeps its slot, and a run ends
+        where the next chunk's pinned slot does not follow; chunks without a pinned slot get consecutive
+        ones from ``assign``."""
+        runs: List[List['Chunk']] = []
+        for c in chunks:
+            pinned = c._stats_pinned and c._stats_home[0] is self
+            if runs:
+                prev = runs[-1][-1]
+                prev_pinned = prev._stats_pinned and prev._stats_home[0] is self
+                if pinned == prev_pinned and (not pinned or c._stats_slot == prev._stats_slot + 1):
+                    runs[-1].append(c)
+                    continue
+            runs.append([c])
+        for run in runs:
+            if not (run[0]._stats_pinned and run[0]._stats_home[0] is self):
+                self.assign(run)
+        return runs
+
     def ptr(self, slot: int) -> int:
         return self.buf.data_ptr() + slot * self.itemsize
 
@@ -239,7 +272,29 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
         assert dtype_code(c.chunk_dtype) == dst_code and dtype_code(pl.dtype) == src_code
         assert pl.numel() == c.shard_size, 'the payload slice must cover the shard'
     arena = StatsArena.get(device)
-    arena.assign(chunks)
+    payload_of = {c: pl for c, pl in zip(chunks, payloads)}
+    for run in arena.runs(list(chunks)):
+        _land_chunks_run(arena, run, [payload_of[c] for c in run], src_code, dst_code, mul)
+
+
+def _mark_landed(chunks: List['Chunk'], device: torch.device) -> None:
+    """The records of these chunks are on their way: an event behind the launch, on its stream."""
+    stream = torch.cuda.current_stream(device)
+    landed = torch.cuda.Event()
+    landed.record(stream)
+    for c in chunks:
+        c._overflow = False
+        c._l2_norm = None
+        c._stats_fresh = False
+        c._stats_pending = True
+        c._stats_event = landed
+        c._stats_stream = stream.cuda_stream
+
+
+def _land_chunks_run(arena: 'StatsArena', chunks: List['Chunk'], payloads: List[torch.Tensor], src_code: int,
+                     dst_code: int, mul: float) -> None:
+    """One launch: the records of ``chunks`` are consecutive slots of ``arena``."""
+    device = chunks[0].shard_device
     rows = np.zeros(len(chunks), dtype=_abi.CHUNK_DTYPE)
     for i, (c, pl) in enumerate(zip(chunks, payloads)):
         rows[i]['grad'] = pl.data_ptr()
@@ -260,23 +315,44 @@ def land_chunks(chunks: List['Chunk'], payloads: List[torch.Tensor], mul: float 
     _abi.land_grads_mt(cached.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
                        arena.ptr(chunks[0]._stats_slot), aligned, stream, LAND_BLOCKS_PER_CU,
                        keep_cached=keep_grads_cached(rows, dst_code))
-    landed = torch.cuda.Event()
-    landed.record(torch.cuda.current_stream(device))
-    for c in chunks:
-        c._overflow = False
-        c._l2_norm = None
-        c._stats_fresh = False
-        c._stats_pending = True
-        c._stats_event = landed
+    _mark_landed(chunks, device)
 
 
-def _land_block_elems(total: int, tile: int) -> int:
-    """Rows of a per-tensor landing are blocks of this many elements: 2048 tiles (where the launch
-    was measured to stream best), doubled while the launch would exceed about 32 Ki rows."""
-    block = 2048 * tile
-    while block * 32768 < total:
-        block <<= 1
-    return block
+LAND_MAX_BLOCK_TILES = 2048    # tiles per row where a launch over long tensors was measured to stream best
+LAND_MAX_ROWS = 32768          # the grid's y extent must stay below 65536
+LAND_IDLE_ALLOWED = 0.10       # share of workgroups without work that a larger block may cost
+
+
+def _land_block_elems(counts, tile: int) -> int:
+    """Rows of a per-tensor landing are blocks of a power-of-two number of tiles.  The launch is a grid of
+    (tiles of the longest row, rows), so every row shorter than that leaves workgroups that find no work:
+    with blocks of 2048 tiles the 148 gradients of GPT-2 small (768 ... 38.6 M elements) make 327,680
+    workgroups for 65,536 tiles of work and the launch runs at half its speed.  ``counts``: the element
+    counts of the pieces.  Picks the largest block, up to ``LAND_MAX_BLOCK_TILES`` tiles, whose launch
+    has at most ``LAND_IDLE_ALLOWED`` idle workgroups (failing that, the block with the fewest
+    workgroups) among those that keep the launch within ``LAND_MAX_ROWS`` rows; a set too large for that
+    gets longer blocks."""
+    counts = np.asarray(counts, dtype=np.int64)
+    tiles = -(-counts // tile)
+    work = int(tiles.sum())
+    longest = int(tiles.max()) if len(tiles) else 1
+    block_tiles = LAND_MAX_BLOCK_TILES
+    while int((-(-counts // (block_tiles * tile))).sum()) > LAND_MAX_ROWS:
+        block_tiles <<= 1
+    if block_tiles > LAND_MAX_BLOCK_TILES:
+        return block_tiles * tile
+    best, best_wgs = block_tiles, None
+    while block_tiles >= 8:
+        rows = int((-(-counts // (block_tiles * tile))).sum())
+        if rows > LAND_MAX_ROWS:
+            break
+        wgs = rows * min(block_tiles, longest)
+        if wgs <= (1.0 + LAND_IDLE_ALLOWED) * work:
+            return block_tiles * tile
+        if best_wgs is None or wgs < best_wgs:
+            best, best_wgs = block_tiles, wgs
+        block_tiles >>= 1
+    return best * tile
 
 
 def land_rows(pieces, n_slots: int, block: int, ssize: int, dsize: int):
@@ -344,36 +420,49 @@ def land_tensors(chunks: List['Chunk'], grad_of, mul: float = 1.0) -> None:
     src_code = dtype_code(src_dtype if src_dtype is not None else dst_dtype)
     ssize = 4 if src_code == _abi.ELX_F32 else 2
     tile = _abi.land_tile_elems(src_code)
-    block = _land_block_elems(sum(c.shard_size for c in chunks), tile)
+    arena = StatsArena.get(device)
+    index_of = {c: ci for ci, c in enumerate(chunks)}
+    for run in arena.runs(list(chunks)):
+        first = index_of[run[0]]
+        mine = [(ci - first, src, chunks[ci].shard.data_ptr() + begin * dsize, count)
+                for ci, src, begin, count in pieces if first <= ci < first + len(run)]
+        _land_tensors_run(arena, run, mine, tile, src_code, dst_code, ssize, dsize, mul)
 
-    rows, slot_offsets = land_rows([(ci, src, chunks[ci].shard.data_ptr() + begin * dsize, count)
-                                    for ci, src, begin, count in pieces], len(chunks), block, ssize, dsize)
+
+LAND_TABLES_KEPT = 4    # device copies of row tables kept per chunk (gradient buffers tend to come back at the same addresses)
+
+
+def _land_tensors_run(arena: 'StatsArena', chunks: List['Chunk'], pieces, tile: int, src_code: int, dst_code: int,
+                      ssize: int, dsize: int, mul: float) -> None:
+    """One launch: the records of ``chunks`` are consecutive slots of ``arena``; ``pieces`` as for
+    ``land_rows``, slots counted from the first chunk of the run."""
+    device = chunks[0].shard_device
+    block = _land_block_elems([count for _, _, _, count in pieces], tile)
+    rows, slot_offsets = land_rows(pieces, len(chunks), block, ssize, dsize)
     if len(rows) > 65535:
         raise RuntimeError(f'{len(rows)} rows in one landing launch: land fewer chunks at a time')
-
-    arena = StatsArena.get(device)
-    arena.assign(chunks)
     bpr = _abi.check_land_rows(rows, slot_offsets, src_code, dst_code)
     ws = chunks[0]._workspace
     need = _abi.land_workspace_records(len(rows), bpr, len(chunks)) * arena.itemsize
     buf = ws.get('land')
     if buf is None or buf.numel() < need:
         buf = ws['land'] = torch.empty(need, dtype=torch.uint8, device=device)
-    table = ws['land_table'] = DeviceTable(rows, device)
-    offsets = ws['land_offsets'] = torch.from_numpy(slot_offsets.view(np.int32).copy()).to(device)
+    # The tables of a landing are the same from step to step whenever the gradients come back at the same
+    # addresses: their device copies are kept (an upload from pageable memory makes the host wait for the stream).
+    tables = ws.setdefault('land_tables', {})
+    key = (rows.tobytes(), slot_offsets.tobytes())
+    kept = tables.get(key)
+    if kept is None:
+        if len(tables) >= LAND_TABLES_KEPT:
+            tables.pop(next(iter(tables)))
+        kept = tables[key] = (DeviceTable(rows, device), torch.from_numpy(slot_offsets.view(np.int32).copy()).to(device))
+    table, offsets = kept
     stream = torch.cuda.current_stream(device).cuda_stream
     _abi.land_grads_mt(table.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
                        arena.ptr(chunks[0]._stats_slot), True, stream, LAND_BLOCKS_PER_CU,
                        d_slot_offsets=offsets.data_ptr(), n_slots=len(chunks),
                        keep_cached=sum(c.n_valid for c in chunks) * dsize <= KEEP_GRADS_CACHED_BELOW)
-    landed = torch.cuda.Event()
-    landed.record(torch.cuda.current_stream(device))
-    for c in chunks:
-        c._overflow = False
-        c._l2_norm = None
-        c._stats_fresh = False
-        c._stats_pending = True
-        c._stats_event = landed
+    _mark_landed(chunks, device)
 
 
 def resolve_pending_stats(chunks: List['Chunk']) -> None:
@@ -385,8 +474,10 @@ def resolve_pending_stats(chunks: List['Chunk']) -> None:
             by_device.setdefault(c.shard_device, []).append(c)
     for device, pending in by_device.items():
         # the landing may have been enqueued on another stream than the one the copy below uses
-        for event in {c._stats_event for c in pending if c._stats_event is not None}:
-            torch.cuda.current_stream(device).wait_event(event)
+        stream = torch.cuda.current_stream(device)
+        for event in {c._stats_event for c in pending
+                      if c._stats_event is not None and c._stats_stream != stream.cuda_stream}:
+            stream.wait_event(event)
         lo = min(c._stats_slot for c in pending)
         hi = max(c._stats_slot for c in pending) + 1
         records = StatsArena.get(device).read(lo, hi)
@@ -473,10 +564,12 @@ class Chunk:
         # True once overflow / l2_norm describe the gradients that sit in the shard now
         self._stats_fresh = False
         self._stats_slot: Optional[int] = None    # this chunk's record in the device arena
+        self._stats_pinned = False                # the slot is this chunk's for good (StatsArena.pin)
         self._stats_home = [None, None]           # [arena, slot], shared with the finalizer that frees the slot
         weakref.finalize(self, _release_stats_home, self._stats_home)
         self._stats_pending = False               # a landing launch has written it, nobody has read it
         self._stats_event = None                  # recorded behind that launch, on its stream
+        self._stats_stream = None                 # that stream's handle
         self._workspace: Dict = {}
 
     # ------------------------------------------------------------------ properties
@@ -511,6 +604,7 @@ class Chunk:
         if old_arena is not None and old_slot is not None:
             old_arena.release(old_slot)
         self._stats_slot = slot
+        self._stats_pinned = False
         self._stats_home[0], self._stats_home[1] = arena, slot
 
     def invalidate_stats(self) -> None:

@@ -41,6 +41,9 @@
 #include <atomic>
 
 #include "elx_abi.h"
+#include "elx_host.h"
+
+using namespace elx_host;
 
 // Partials workspace of elx_grad_stats_mt_static, the one entry point that takes no workspace from
 // its caller and allocates none: every GPU the library runs on holds this array until the process
@@ -53,17 +56,6 @@ static __device__ __align__(256) unsigned char scratch[kStaticPartials * sizeof(
 
 namespace {
 
-constexpr int kWave = 64;                              // one wavefront per update workgroup
-constexpr int kVec = 4;                                // elements per lane per access
-constexpr int kUnroll = 1;                             // independent accesses per lane per stream
-constexpr uint32_t kSpan = kWave * kVec;               // elements one wavefront access covers
-constexpr uint32_t kTile = kSpan * kUnroll;            // 256 elements per tile
-constexpr uint64_t kMaxBufferElems = 1ull << 40;       // longest buffer a table row may describe (tile arithmetic stays far from overflow)
-constexpr uint32_t kLdsPerCu = 160u * 1024u;           // gfx950
-constexpr uint32_t kDefaultBlocksPerCu = 12;           // fp32 gradients (4 KiB of loads in flight per workgroup)
-constexpr uint32_t kDefaultBlocksPerCuLowp = 13;       // 16-bit gradients (3.5 KiB): one more workgroup pays
-constexpr uint32_t kMinBlocksPerCu = 3;                // keeps the reservation below 64 KiB
-constexpr uint32_t kMaxBlocksPerCu = 32;
 constexpr uint32_t kStatsStreamBlocksPerCu = 3;        // stats workgroups (256 threads) per CU when the set streams from HBM
 
 constexpr int kStatsThreads = 256;
@@ -212,14 +204,7 @@ __device__ __forceinline__ Hyper load_hyper(const ElxHyper *__restrict__ h) {
     return r;
 }
 
-// How the gradient is unscaled: not at all, by an exact multiply with 1/div_scale (div_scale a
-// power of two: same bits as the division), or by a true IEEE division.
-enum { kDivNone = 0, kDivMulInv = 1, kDivTrue = 2 };
-
-struct Unscale {
-    float div_scale, inv_scale;
-    int mode;
-};
+// (how the gradient is unscaled -- kDivNone / kDivMulInv / kDivTrue and struct Unscale -- is declared in elx_host.h)
 
 // One element, with the three launch-uniform choices (unscale mode, L2 vs decoupled decay, which
 // end the lerp starts from) fixed at compile time: the tile loop below is then straight-line code.
@@ -722,8 +707,6 @@ __global__ __launch_bounds__(kStatsThreads) void stats_finish_kernel(const ElxSt
 // (blocks_per_row, n_rows); when a row has more tiles than blocks a workgroup takes several
 // (stride gridDim.x).  Every workgroup leaves one ElxStats partial, folded afterwards in a fixed
 // order by stats_fold_kernel / stats_finish_kernel.
-constexpr int kLandUnroll = 4;
-constexpr uint32_t kMaxLandBlocks = 1u << 20;
 constexpr uint32_t kDefaultLandBlocksPerCu = 10;
 constexpr uint32_t kDefaultLandBlocksPerCuNarrowing = 13;    // fp32 payload into a 16-bit shard: half the bytes go out
 constexpr uint32_t kFoldBlocks = 64;           // first-stage workgroups per row when partials are many
@@ -969,7 +952,7 @@ __global__ void decide_kernel(const ElxStats *__restrict__ stats, uint32_t n, do
 // first, the sequence number of the control block last, all with system-scope stores, so that a host
 // polling the sequence number in pinned memory sees a complete report while the update launch that
 // follows is still running.
-constexpr uint32_t kMaxCtlHypers = 64;
+constexpr uint32_t kMaxCtlHypers = 256;
 constexpr uint32_t kCtlWords = (uint32_t)(sizeof(ElxStepCtl) + kMaxCtlHypers * sizeof(ElxHyper)) / 4u;
 constexpr uint32_t kCtlEarlyHypers = 4;    // records fetched with the header, before anyone knows how many there are
 static_assert((sizeof(ElxStepCtl) + kCtlEarlyHypers * sizeof(ElxHyper)) / 4u <= kStatsThreads, "one early load per thread");
@@ -1124,45 +1107,8 @@ __global__ __launch_bounds__(kWave) void put_hypers_kernel(HyperPack pack, uint3
 // host side of the ABI
 // ---------------------------------------------------------------------------------------------
 
-bool is_lowp_or_f32(int d) { return d == ELX_F32 || d == ELX_F16 || d == ELX_BF16; }
-
-uint32_t elem_size(int d) { return d == ELX_F32 ? 4u : 2u; }
-
-// div_scale is a power of two whose reciprocal is a normal fp32 number
-bool exact_reciprocal(float s) {
-    uint32_t u;
-    __builtin_memcpy(&u, &s, 4);
-    const uint32_t exp = (u >> 23) & 0xFFu, man = u & 0x7FFFFFu;
-    return (u >> 31) == 0 && man == 0 && exp >= 1 && exp <= 252;
-}
-
-// How the update launch divides by div_scale (the div_scale of optimizer.py:216; <= 0: not at all).
-Unscale unscale_of(float div_scale) {
-    Unscale us;
-    us.div_scale = div_scale;
-    us.inv_scale = 1.0f;
-    us.mode = kDivNone;
-    if (div_scale > 0.0f) {
-        if (exact_reciprocal(div_scale)) {
-            us.mode = kDivMulInv;
-            us.inv_scale = 1.0f / div_scale;
-        } else {
-            us.mode = kDivTrue;
-        }
-    }
-    return us;
-}
-
 // flag bits an update launch understands
 constexpr uint32_t kUpdateFlags = ELX_FLAG_SCALAR_ONLY | ELX_FLAG_KEEP_CACHED | ELX_FLAG_KEEP_STATE_CACHED;
-
-// dynamic LDS bytes that let exactly `blocks_per_cu` update workgroups share a compute unit
-int occupancy_reservation(uint32_t blocks_per_cu, uint32_t *lds_bytes, uint32_t fallback = kDefaultBlocksPerCu) {
-    if (blocks_per_cu == 0) blocks_per_cu = fallback;
-    if (blocks_per_cu < kMinBlocksPerCu || blocks_per_cu > kMaxBlocksPerCu) return ELX_E_SIZE;
-    *lds_bytes = (kLdsPerCu / blocks_per_cu) & ~255u;
-    return 0;
-}
 
 // The cache policy the flags of an update launch ask for.  Without a low-precision copy kKeepLowp has nothing
 // to act on and is the streaming launch.
@@ -1260,13 +1206,28 @@ int dispatch_step_args(int gd, int ld, uint32_t lds, hipStream_t st, const Hyper
 constexpr int kMaxDevices = 64;
 std::atomic<void *> g_scratch_ptr[kMaxDevices];
 
-int scratch_of_current_device(void **out) {
+// `stream` (NULL: the default stream) is the one the caller's launches will go to.  Refused with
+// ELX_E_STATE: a stream that belongs to another GPU than the calling thread's current one (the array's
+// address is only good there), and a first call on a device made while the stream is capturing (the
+// address lookup is not something to do inside a capture).
+int scratch_of_current_device(hipStream_t stream, void **out) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= kMaxDevices) return ELX_E_SIZE;
+    if (stream) {
+        hipDevice_t of_stream, current;
+        if (hipStreamGetDevice(stream, &of_stream) == hipSuccess && hipDeviceGet(&current, dev) == hipSuccess) {
+            if (of_stream != current) return ELX_E_STATE;
+        } else {
+            (void)hipGetLastError();    // the query is a courtesy: a runtime that cannot answer leaves the rule to the caller
+        }
+    }
     void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (!ptr) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+        if (capturing != hipStreamCaptureStatusNone) return ELX_E_STATE;
         e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return (int)e;
         if (!ptr) return ELX_E_NULL;
@@ -1316,7 +1277,6 @@ extern "C" {
 
 int elx_version(void) { return ELX_ABI_VERSION; }
 
-uint32_t elx_tile_elems(void) { return kTile; }
 uint32_t elx_sizeof_chunk(void) { return (uint32_t)sizeof(ElxChunk); }
 uint32_t elx_sizeof_seg(void) { return (uint32_t)sizeof(ElxSeg); }
 uint32_t elx_sizeof_hyper(void) { return (uint32_t)sizeof(ElxHyper); }
@@ -1333,82 +1293,11 @@ const char *elx_strerror(int code) {
         case ELX_E_ORDER: return "elx: segments of a chunk are not sorted or overlap";
         case ELX_E_TILES: return "elx: tile_begin / total_tiles disagree with the chunk sizes";
         case ELX_E_SIZE: return "elx: a count is zero, out of its allowed range, or exceeds what a launch can address";
+        case ELX_E_STATE: return "elx: the call cannot be made in this state (a stream of another GPU than the current one, or a first call on a device made under stream capture)";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
     return "elx: unknown error code";
-}
-
-int elx_check_tables(const ElxChunk *h_chunks, uint32_t n_chunks, const ElxSeg *h_segs, uint32_t n_segs,
-                     uint32_t n_hypers, int grad_dtype, int lowp_dtype, uint64_t *total_tiles,
-                     uint32_t *max_tiles_per_chunk, int *all_aligned16) {
-    if (!h_chunks || !total_tiles || !max_tiles_per_chunk || !all_aligned16 || (n_segs && !h_segs)) return ELX_E_NULL;
-    if (n_chunks == 0 || n_chunks > 65535u) return ELX_E_SIZE;
-    if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
-    if (lowp_dtype != ELX_NONE && lowp_dtype != grad_dtype) return ELX_E_DTYPE;
-    const uintptr_t gmask = elem_size(grad_dtype) - 1;
-    uint64_t tiles = 0;
-    int aligned = 1;
-    uint64_t max_tiles = 0;
-    for (uint32_t i = 0; i < n_chunks; ++i) {
-        const ElxChunk &c = h_chunks[i];
-        if (!c.master || !c.m || !c.v) return ELX_E_NULL;
-        if (c.lowp_out && lowp_dtype == ELX_NONE) return ELX_E_DTYPE;
-        if (c.n_alloc == 0 || c.n_alloc > kMaxBufferElems) return ELX_E_SIZE;
-        if ((c.n_alloc + kTile - 1) / kTile > max_tiles) max_tiles = (c.n_alloc + kTile - 1) / kTile;
-        if (c.n_valid > c.n_alloc) return ELX_E_RANGE;
-        const uintptr_t ptrs[5] = {(uintptr_t)c.grad, (uintptr_t)c.lowp_out, (uintptr_t)c.master, (uintptr_t)c.m,
-                                   (uintptr_t)c.v};
-        if ((ptrs[0] & gmask) || (ptrs[1] & gmask) || (ptrs[2] & 3u) || (ptrs[3] & 3u) || (ptrs[4] & 3u))
-            return ELX_E_ALIGN;
-        for (int k = 0; k < 5; ++k)
-            if (ptrs[k] & 15u) aligned = 0;
-        if (c.tile_begin != tiles) return ELX_E_TILES;
-        tiles += (c.n_alloc + kTile - 1) / kTile;
-        if (c.seg_begin > c.seg_end || c.seg_end > n_segs) return ELX_E_RANGE;
-        uint64_t prev_end = 0;
-        for (uint32_t s = c.seg_begin; s < c.seg_end; ++s) {
-            const ElxSeg &sg = h_segs[s];
-            if (sg.begin >= sg.end || sg.end > c.n_valid) return ELX_E_RANGE;
-            if (sg.hyper >= n_hypers) return ELX_E_RANGE;
-            if (sg.begin < prev_end) return ELX_E_ORDER;
-            prev_end = sg.end;
-        }
-    }
-    if (tiles > 0x7FFFFFFFull) return ELX_E_SIZE;    // one workgroup per tile
-    *total_tiles = tiles;
-    *max_tiles_per_chunk = (uint32_t)max_tiles;
-    *all_aligned16 = aligned;
-    return 0;
-}
-
-int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t *h_slot_offsets, uint32_t n_slots,
-                        int src_dtype, int dst_dtype, uint32_t *blocks_per_row) {
-    if (!h_rows || !blocks_per_row) return ELX_E_NULL;
-    if (!is_lowp_or_f32(src_dtype) || !is_lowp_or_f32(dst_dtype)) return ELX_E_DTYPE;
-    if (src_dtype != dst_dtype && src_dtype != ELX_F32) return ELX_E_DTYPE;
-    if (n_rows == 0 || n_rows > 65535u) return ELX_E_SIZE;
-    const uintptr_t smask = elem_size(src_dtype) - 1, dmask = elem_size(dst_dtype) - 1;
-    const uint64_t tile = kWave * (16u / elem_size(src_dtype)) * kLandUnroll;
-    uint64_t max_tiles = 1;
-    for (uint32_t i = 0; i < n_rows; ++i) {
-        const ElxChunk &r = h_rows[i];
-        if (!r.lowp_out) return ELX_E_NULL;
-        if (r.n_alloc == 0 || r.n_alloc > kMaxBufferElems) return ELX_E_SIZE;
-        if (r.n_valid > r.n_alloc) return ELX_E_RANGE;
-        if (((uintptr_t)r.grad & smask) || ((uintptr_t)r.lowp_out & dmask)) return ELX_E_ALIGN;
-        const uint64_t t = (r.n_alloc + tile - 1) / tile;
-        if (t > max_tiles) max_tiles = t;
-    }
-    if (max_tiles > kMaxLandBlocks) return ELX_E_SIZE;
-    if (h_slot_offsets) {
-        if (n_slots == 0 || n_slots > n_rows) return ELX_E_SIZE;
-        if (h_slot_offsets[0] != 0 || h_slot_offsets[n_slots] != n_rows) return ELX_E_RANGE;
-        for (uint32_t s = 0; s < n_slots; ++s)
-            if (h_slot_offsets[s] > h_slot_offsets[s + 1]) return ELX_E_ORDER;
-    }
-    *blocks_per_row = (uint32_t)max_tiles;
-    return 0;
 }
 
 int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_dtype, uint32_t blocks_per_chunk,
@@ -1486,7 +1375,7 @@ int elx_grad_stats_mt_static(const ElxChunk *d_chunks, uint32_t n_chunks, int gr
     if (!is_lowp_or_f32(grad_dtype)) return ELX_E_DTYPE;
     if ((uint32_t)flags & ~(uint32_t)(ELX_FLAG_SCALAR_ONLY | ELX_FLAG_KEEP_CACHED)) return ELX_E_RANGE;
     void *partials = nullptr;
-    if (int rc = scratch_of_current_device(&partials)) return rc;
+    if (int rc = scratch_of_current_device((hipStream_t)stream, &partials)) return rc;
     // every partial the finish launch reads is written by the stats launch first: nothing to clear
     return elx_grad_stats_mt(d_chunks, n_chunks, grad_dtype, blocks_per_chunk, reinterpret_cast<ElxStats *>(partials),
                              d_stats, flags, stream);
@@ -1685,10 +1574,6 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d
     return (int)hipGetLastError();
 }
 
-uint32_t elx_land_tile_elems(int src_dtype) { return kWave * (16u / elem_size(src_dtype)) * kLandUnroll; }
-
 uint32_t elx_land_fold_blocks(void) { return kFoldBlocks; }
-
-uint32_t elx_land_max_blocks(void) { return kMaxLandBlocks; }
 
 }    // extern "C"

@@ -77,6 +77,40 @@ def hyper_record_cached(key: Tuple, adamw_mode: bool) -> np.ndarray:
     return rec
 
 
+class _SteadyStep:
+    """A standalone step over the same buffers as the step before it, all of them one step further: the
+    walk over the parameters, the launch plan and the tables are those of the last step, and all that is
+    new are the hyper records (computed while the last launch was running).  What it keeps lets the next
+    ``step()`` go from its first line to the launch in a few microseconds -- on a 16 Mi-element parameter
+    the launch itself takes under 70, and whatever the host needs in front of it the device spends idle."""
+
+    __slots__ = ('watch', 'layout', 'states', 'step', 'group_of_hyper', 'dplan', 'grad_code', 'device', 'call', 'fixed',
+                 'tail', 'pack', 'pack_ptr')
+
+    def __init__(self, watch, layout, prep: '_Prepared', step: int, group_of_hyper):
+        plan = prep.dplan.plan
+        self.watch, self.layout, self.states, self.step = watch, layout, prep.states, step
+        self.group_of_hyper = group_of_hyper      # group index of every hyper record, in table order
+        self.dplan, self.grad_code, self.device = prep.dplan, prep.grad_code, prep.device
+        self.call = _abi.load().elx_adam_step_put_mt
+        self.fixed = (prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs))
+        self.tail = (plan.info.total_tiles, plan.info.max_tiles)
+        n = len(group_of_hyper)
+        self.pack = np.zeros(n, dtype=_abi.HYPER_DTYPE) if n > 1 else None    # several records: gathered here
+        self.pack_ptr = self.pack.ctypes.data if n > 1 else 0
+
+
+_NO_HOOKS: Dict = {}
+
+
+def _global_step_hooks():
+    """torch's process-wide optimizer step hooks (``register_optimizer_step_pre_hook`` /
+    ``..._post_hook``).  They live in private module attributes of torch.optim.optimizer; a torch that
+    names them differently has no such hooks as far as this class can tell."""
+    return (getattr(_torch_optimizer, '_global_optimizer_pre_hooks', _NO_HOOKS),
+            getattr(_torch_optimizer, '_global_optimizer_post_hooks', _NO_HOOKS))
+
+
 class _CachedTable:
     """Device copy of a host table, re-uploaded only when the host contents change."""
 
@@ -176,8 +210,9 @@ class _Prepared:
     """Everything a step needs that does not depend on the gradient flags: built while the stats
     launch is still running, consumed (and only then committed to the optimizer state) by step()."""
 
-    def __init__(self, dplan, hyper_host, grad_code, lowp_code, device, states, hyper_keys=()):
+    def __init__(self, dplan, hyper_host, grad_code, lowp_code, device, states, hyper_keys=(), hyper_index=()):
         self.dplan: _DevicePlan = dplan
+        self.hyper_index = hyper_index        # per entry of ``states``: which hyper record it is updated with
         self.hyper_host: np.ndarray = hyper_host
         self.hyper_keys = tuple(hyper_keys)    # (lr, beta1, beta2, eps, weight_decay, step, bias_correction) per record
         self.grad_code, self.lowp_code, self.device = grad_code, lowp_code, device
@@ -222,6 +257,7 @@ class HybridAdam(torch.optim.Optimizer):
         self._launched: Optional[_Prepared] = None   # launched with defer_commit, not yet committed or aborted
         self._bound_entries = None                  # cached walk over the bound fake parameters
         self._standalone_cache = None               # cached walk over standalone parameters and their gradients
+        self._steady: Optional[_SteadyStep] = None   # a standalone step that can repeat the one before it
         # when set to a dict, step() records (begin, end) torch.cuda.Event pairs under 'adam_step' and 'refresh'
         self.kernel_events = None
 
@@ -318,10 +354,11 @@ class HybridAdam(torch.optim.Optimizer):
         torch wraps every optimizer's ``step`` in a profiler scope and its hook dispatch, tens of
         microseconds during which the device waits; this class opts out of that wrapper (the ``hooked``
         mark below) and runs registered step hooks itself, in torch's order."""
-        pre = list(_torch_optimizer._global_optimizer_pre_hooks.values()) + list(self._optimizer_step_pre_hooks.values())
-        post = list(self._optimizer_step_post_hooks.values()) + list(_torch_optimizer._global_optimizer_post_hooks.values())
-        if not pre and not post:
+        global_pre, global_post = _global_step_hooks()
+        if not (global_pre or global_post or self._optimizer_step_pre_hooks or self._optimizer_step_post_hooks):
             return self.launch_step(closure, div_scale, gated=gated, defer_commit=defer_commit)
+        pre = list(global_pre.values()) + list(self._optimizer_step_pre_hooks.values())
+        post = list(self._optimizer_step_post_hooks.values()) + list(global_post.values())
         args, kwargs = (closure, div_scale), dict(gated=gated, defer_commit=defer_commit)
         for hook in pre:
             result = hook(self, args, kwargs)
@@ -343,6 +380,13 @@ class HybridAdam(torch.optim.Optimizer):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        steady = self._steady
+        if steady is not None:
+            if (self._prepared is None and not gated and not defer_commit and self.kernel_events is None
+                    and self._steady_still_holds(steady)):
+                self._launch_steady(steady, div_scale)
+                return loss
+            self._steady = None
         if self._prepared is None:
             self.prepare_step(upload=False)    # the records go out with the launch below
         prep, self._prepared = self._prepared, None
@@ -392,7 +436,78 @@ class HybridAdam(torch.optim.Optimizer):
         self._launched = prep
         if not defer_commit:
             self.commit_step()
+            if together and self._binding is None and prep.dplan.refresh is None:
+                self._remember_steady(prep)
         return loss
+
+    # ---- a standalone step that repeats the one before it
+
+    def _remember_steady(self, prep: '_Prepared') -> None:
+        """After a standalone step whose records rode in its launch: keep what the next step can reuse if
+        nothing but the step counts has changed by then."""
+        cache = self._standalone_cache
+        if cache is None or not prep.states or len(prep.hyper_keys) > _abi.MAX_ARG_HYPERS:
+            return
+        watch, layout, (items, _, _) = cache
+        step = prep.states[0]['step']
+        if any(st['step'] != step for st in prep.states):
+            return    # per-parameter step counts differ: the records would have to be matched to parameters again
+        group_of_hyper = [None] * len(prep.hyper_keys)
+        for (state, gi, _), h in zip(items, prep.hyper_index):
+            if group_of_hyper[h] is None:
+                group_of_hyper[h] = gi
+            elif group_of_hyper[h] != gi:
+                return    # two groups share one record: a change in one of them would need a new plan
+        self._steady = _SteadyStep(watch, layout, prep, step, group_of_hyper)
+
+    def _steady_still_holds(self, steady: _SteadyStep) -> bool:
+        groups = self.param_groups
+        if len(groups) != len(steady.layout):
+            return False
+        for group, count in zip(groups, steady.layout):
+            if len(group['params']) != count:
+                return False
+        for p, p_ptr, g_ptr, g_dtype in steady.watch:
+            g = p.grad
+            if g is None:
+                if g_ptr is not None:
+                    return False
+            elif g_ptr is None or g.data_ptr() != g_ptr or g.dtype != g_dtype or p.data_ptr() != p_ptr:
+                return False
+        step = steady.step
+        for state in steady.states:
+            if state['step'] != step:
+                return False
+        return True
+
+    def _launch_steady(self, steady: _SteadyStep, div_scale: float) -> None:
+        groups = self.param_groups
+        step = steady.step + 1
+        if steady.pack is None:
+            key = self._group_key(groups[steady.group_of_hyper[0]], step)
+            rec = hyper_record_cached(key, self.adamw_mode)
+            ptr = rec.__array_interface__['data'][0]
+            keys = (key, )
+        else:
+            keys = tuple(self._group_key(groups[gi], step) for gi in steady.group_of_hyper)
+            # (two groups whose hyper-parameters have become equal would share a record in a freshly built plan;
+            # this plan keeps one record each, which is the same arithmetic)
+            for h, key in enumerate(keys):
+                steady.pack[h] = hyper_record_cached(key, self.adamw_mode)[0]
+            ptr = steady.pack_ptr
+        plan = steady.dplan.plan
+        stream = torch.cuda.current_stream(steady.device).cuda_stream
+        d_hypers = self._hyper_table_dev.reserve(len(keys) * _abi.HYPER_DTYPE.itemsize, steady.device)
+        code = steady.call(*steady.fixed, ptr, d_hypers, len(keys), *steady.tail, float(div_scale), steady.grad_code,
+                           _abi.ELX_NONE, plan.info.flags, self.blocks_per_cu, stream)
+        if code != 0:
+            _abi.check('elx_adam_step_put_mt', code)
+        # the launch is out: bookkeeping, and the records of the step after this one
+        for state in steady.states:
+            state['step'] = step
+        steady.step = step
+        for (lr, b1, b2, eps, wd, st, bc) in keys:
+            hyper_record_cached((lr, b1, b2, eps, wd, st + 1, bc), self.adamw_mode)
 
     def commit_step(self) -> None:
         """The launched step happened: step counts advance (after the launches, so that the device is
@@ -472,6 +587,7 @@ class HybridAdam(torch.optim.Optimizer):
             state['step'] = int(step.item()) if torch.is_tensor(step) else int(step)
         self._prepared = None
         self._standalone_cache = None
+        self._steady = None
 
     def _walk_bound(self):
         """(state dict, group index, chunk index, begin, end) per bound fake parameter, in group order."""
@@ -625,7 +741,7 @@ class HybridAdam(torch.optim.Optimizer):
 
         dplan = self._device_plan(key, buffers, grad_dtype, grad_code, _abi.ELX_NONE, len(hypers), device)
         return _Prepared(dplan, self._hyper_table(hypers), grad_code, _abi.ELX_NONE, device, [it[0] for it in items],
-                         hypers.keys())
+                         hypers.keys(), idx_of)
 
 
 class FusedAdam(HybridAdam):

@@ -29,6 +29,7 @@ Differences from the reference, all on purpose:
     flat buffers in place;
   * shards in pinned host memory are stepped by the same launches, in place over the host link.
 """
+import logging
 import math
 import time
 from collections import defaultdict
@@ -46,6 +47,9 @@ from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
 from .hybrid_adam import CPUAdam, FusedAdam, HybridAdam
 
 _AVAIL_OPTIM_LIST = {FusedAdam, CPUAdam, HybridAdam}
+
+# the one runtime signal of this path in the reference: optimizer.py:88 (a distributed logger) and :199
+logger = logging.getLogger('elixir_amd.optimizer')
 
 
 class OptimState(Enum):
@@ -199,6 +203,12 @@ class ElixirOptimizer(torch.optim.Optimizer):
         self.param_chunk_set: Set[Chunk] = self.param_chunk_group.fused_chunks.union(
             self.param_chunk_group.float_chunks)
         self._param_chunk_list: List[Chunk] = sorted(self.param_chunk_set)
+        # Every parameter chunk gets its record slot in the device arena now, in chunk order: landings then
+        # leave the flags side by side whatever order the chunks land in (backward lands the last chunk
+        # first, one launch per chunk), and the step folds them with one launch, without a host read.
+        shards = [c.shard for c in self._param_chunk_list]
+        if shards and all(t.is_cuda and t.device == shards[0].device for t in shards):
+            StatsArena.get(shards[0].device).pin(self._param_chunk_list)
 
         self.clipping_flag = max_norm > 0.0
         self.max_norm = max_norm
@@ -239,6 +249,9 @@ class ElixirOptimizer(torch.optim.Optimizer):
         # over a set of tables runs eagerly, the second records; nothing is recorded while kernel_events is set)
         self.graph_step = False
         self._device_step: _DeviceStep = None
+        # most hyper records a step decided on the device can carry (the control block's capacity); a step
+        # with more is decided on the host, from the same single pass over the gradients
+        self.max_device_hypers = _abi.max_ctl_hypers()
         self._wb_table = None
         self.last_step_info: Dict = {}
         # when set to a dict, step() records (begin, end) torch.cuda.Event pairs on the launch
@@ -576,13 +589,25 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 early = True
         else:
             arena = StatsArena.get(chunks[0].shard_device)
-            for event in {c._stats_event for c in chunks if c._stats_event is not None}:
-                main.wait_event(event)    # the landings may have run on another stream
+            for event in {c._stats_event for c in chunks
+                          if c._stats_event is not None and c._stats_stream != main.cuda_stream}:
+                main.wait_event(event)    # landings that ran on another stream
             bpc, partials, stats_args, keep, cached = 1, arena.ptr(first_slot), None, (arena, ), False
         inner.prepare_step(upload=False)
         prep = inner._prepared
-        if prep is None or prep.dplan.rows is None or len(prep.hyper_host) > _abi.max_ctl_hypers():
-            return False    # (a stats launch that went out early is then simply repeated by the host-decided step)
+        if prep is None or prep.dplan.rows is None or len(prep.hyper_host) > min(self.max_device_hypers, eng.max_hypers):
+            if early:
+                # The gradients have been read already: the partials are folded by the same launch, with a
+                # control block that carries no hyper records, and its report brings every chunk's flags to
+                # the host, which decides.  The gradients are not read a second time.
+                seq = eng.write_ctl(float(self.loss_scale), float(self.max_norm) if self.clipping_flag else 1.0,
+                                    self.clipping_flag, np.zeros(0, dtype=_abi.HYPER_DTYPE))
+                _abi.finish_decide(partials, n, bpc, eng.d_stats, eng.ctl.data_ptr(), eng.d_hypers, eng.max_hypers,
+                                   eng.d_decision, eng.report.data_ptr(), eng.d_counter, main.cuda_stream)
+                _, stats = eng.wait_report(seq, main)
+                for c, r in zip(chunks, stats):
+                    c._apply_stats(bool(r['overflow']), float(r['sumsq']))
+            return False
         assert prep.device == device
         # the control block is complete before the launch that reads it is issued
         seq = eng.write_ctl(float(self.loss_scale), float(self.max_norm), self.clipping_flag, prep.hyper_host)
@@ -628,6 +653,7 @@ class ElixirOptimizer(torch.optim.Optimizer):
                                    chunk_overflow=[c._overflow for c in chunks])
         self.optim_state = OptimState.UNSCALED
         if found_inf:
+            logger.info('Found overflow. Skip step')
             inner.abort_step()
         else:
             inner.commit_step()
@@ -662,6 +688,7 @@ class ElixirOptimizer(torch.optim.Optimizer):
                                    chunk_overflow=[c._overflow for c in self._param_chunk_list])
 
         if found_inf:
+            logger.info('Found overflow. Skip step')
             if self._binding is not None:
                 self.optim.discard_prepared()
             self.optim_state = OptimState.UNSCALED    # no need to unscale grad

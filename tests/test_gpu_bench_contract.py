@@ -32,6 +32,11 @@ def test_bench_json_line():
     c = out['cpu_baseline']
     assert c['kind'] == 'port' and c['cores'] >= 1 and c['value'] > 0 and c['unit'] == 'elements/s'
     assert out['fused_landing']['ms_per_step'] > 0
+    # the training flow: one landing launch per chunk, last chunk first, and still a step decided on the device
+    per_chunk = out['fused_landing']['per_chunk_landing']
+    assert per_chunk['launches'] == 2 and per_chunk['ms_per_step'] > 0
+    per_tensor = out['fused_landing']['per_tensor_landing']
+    assert per_tensor['ms_on_device'] > 0 and 0 < per_tensor['frac_of_hbm_peak'] < 1
     # configuration 3's timed part rides the c2 line: the step that finds an overflow
     skip = out['skip_step']
     assert skip['bytes_per_step'] == 2 * 124_439_808 + 6 * 134_217_728 and 0 < skip['frac'] < 1
@@ -49,3 +54,21 @@ def test_velocity_line():
     assert abs(out['vs_baseline'] - out['value'] / 50.0) < 1e-9
     assert abs(out['value'] - 1.0 / (out['ms_per_step'] * 1e-3)) <= 1e-6 * out['value']
     assert out['roofline']['bytes_per_launch'] == 28 * 10**9 and 0 < out['roofline']['frac'] < 1
+
+
+def test_config1_line():
+    """Configuration 1 (flat fp32 Adam, 16 Mi elements): the line's own figure is the step behind a copy that
+    empties the memory-side cache, and it accounts for the step in microseconds: update launch, the floor any
+    launch between two synchronisations costs, the host's own call."""
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--workload', 'c1', '--steps', '5',
+                           '--warmup', '2', '--cpu-sample', '0'], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                          timeout=280)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = json.loads([l for l in proc.stdout.splitlines() if l.startswith('{')][0])
+    assert out['config']['valid_elements'] == 1 << 24 and out['roofline']['bytes_per_launch'] == 28 << 24
+    assert out['ms_per_step'] == out['step_cold_cache']['ms_per_step'] > 0
+    acc = out['step_accounting_us']
+    assert acc['steady_path_taken'] is True
+    assert 0 < out['launch_sync_floor_us'] < 200 and 0 < out['host_us_in_step'] < 200
+    assert abs(acc['step'] - acc['update_launch'] - acc['launch_sync_floor'] - acc['unaccounted']) < 1e-6
+    assert out['step_state_in_cache']['ms_per_step'] > 0 and out['steps_back_to_back']['ms_per_step'] > 0

@@ -1,0 +1,204 @@
+"""Branches of the kernels and of the wrapper that the broader GPU tests do not reach: the decision
+kernel over more chunks than it stages, a refresh workgroup that takes several pieces, and a wrapper
+step with more hyper records than the update launch's arguments or the control block can carry."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import elixir_amd as ea
+from elixir_amd import _abi
+from elixir_amd.chunk import DeviceTable
+from elixir_amd.hybrid_adam import make_hyper_record
+from oracle import oracle as O
+
+from helpers import CODE, build_workload, compare_state, refresh_oracle_grads, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+REC = _abi.STATS_DTYPE.itemsize
+HSZ = _abi.HYPER_DTYPE.itemsize
+
+
+@pytest.mark.parametrize('overflow', [False, True])
+@pytest.mark.parametrize('n', [1500, 4000])
+def test_finish_decide_over_more_chunks_than_it_stages(n, overflow):
+    """The decision workgroup stages 1024 per-chunk records in LDS and reads the rest from memory, both
+    in its decision loop and when it copies the records into the report: 1,500 and 4,000 tiny chunks
+    (two partials each; with ``overflow`` an inf in chunk 1,400; clipping on) against elx_grad_stats_mt
+    followed by elx_decide on the same gradients -- identical records, decision, gate words and report."""
+    rng = np.random.default_rng(n)
+    sizes = rng.integers(1, 400, n)
+    starts = np.concatenate(([0], np.cumsum((sizes + 7) // 8 * 8)))    # every chunk starts on a 16-byte boundary
+    gen = torch.Generator(device=DEV).manual_seed(n)
+    g = (torch.randn(int(starts[-1]), generator=gen, device=DEV) * 2.0).half()
+    if overflow:
+        g[int(starts[1400]) + int(sizes[1400]) - 1] = float('inf')
+    rows = np.zeros(n, dtype=_abi.CHUNK_DTYPE)
+    rows['grad'] = g.data_ptr() + 2 * starts[:-1].astype(np.uint64)
+    rows['n_alloc'] = rows['n_valid'] = sizes
+    table = DeviceTable(rows, torch.device(DEV, 0))
+    stream = torch.cuda.current_stream().cuda_stream
+    bpc, n_hyp, loss_scale, max_norm = 2, 3, 64.0, 0.75
+    hyp_host = np.concatenate([make_hyper_record(1e-3 * (k + 1), 0.9, 0.999, 1e-8, 0.01 * k, 1 + k, True, True)
+                               for k in range(n_hyp)])
+    H = _abi.max_ctl_hypers()
+
+    ws = torch.empty((n * bpc + n) * REC, dtype=torch.uint8, device=DEV)
+    _abi.grad_stats_mt(table.ptr, n, _abi.ELX_F16, bpc, ws.data_ptr(), ws.data_ptr() + n * bpc * REC, False, stream)
+    hyp_a = torch.from_numpy(hyp_host.view(np.uint8).copy()).to(DEV)
+    dec_a = torch.zeros(32, dtype=torch.uint8, device=DEV)
+    _abi.decide(ws.data_ptr() + n * bpc * REC, n, loss_scale, max_norm, True, hyp_a.data_ptr(), n_hyp, dec_a.data_ptr(),
+                stream)
+
+    ctl_head, rep_head = _abi.STEP_CTL_DTYPE.itemsize, _abi.STEP_REPORT_DTYPE.itemsize
+    ctl = torch.zeros(ctl_head + H * HSZ, dtype=torch.uint8, pin_memory=True)
+    cb = ctl.numpy()
+    cb[:ctl_head].view(_abi.STEP_CTL_DTYPE)[0] = (loss_scale, max_norm, 1, n_hyp, 4242)
+    cb[ctl_head:ctl_head + hyp_host.nbytes] = hyp_host.view(np.uint8).reshape(-1)
+    report = torch.zeros(rep_head + n * REC, dtype=torch.uint8, pin_memory=True)
+    partials = torch.empty(n * bpc * REC, dtype=torch.uint8, device=DEV)
+    stats_b = torch.zeros(n * REC, dtype=torch.uint8, device=DEV)
+    hyp_b = torch.full((H * HSZ, ), 0xEE, dtype=torch.uint8, device=DEV)
+    dec_b = torch.zeros(32, dtype=torch.uint8, device=DEV)
+    counter = torch.zeros(4, dtype=torch.int32, device=DEV)
+    _abi.grad_partials_mt(table.ptr, n, _abi.ELX_F16, bpc, partials.data_ptr(), False, stream)
+    _abi.finish_decide(partials.data_ptr(), n, bpc, stats_b.data_ptr(), ctl.data_ptr(), hyp_b.data_ptr(), H,
+                       dec_b.data_ptr(), report.data_ptr(), counter.data_ptr(), stream)
+    torch.cuda.synchronize()
+
+    want_stats = ws[n * bpc * REC:].cpu().numpy()
+    assert want_stats.tobytes() == stats_b.cpu().numpy().tobytes()
+    assert dec_a.cpu().numpy().tobytes() == dec_b.cpu().numpy().tobytes()
+    assert hyp_a.cpu().numpy().tobytes() == hyp_b[:n_hyp * HSZ].cpu().numpy().tobytes()
+    assert bool((hyp_b[n_hyp * HSZ:] == 0xEE).all())
+    rb = report.numpy()
+    rh = rb[:rep_head].view(_abi.STEP_REPORT_DTYPE)[0]
+    assert rh['seq'] == 4242 and rh['n_chunks'] == n and rh['status'] == 0 and bool(rh['skip']) == overflow
+    assert rb[:32].tobytes() == dec_b.cpu().numpy().tobytes()
+    assert rb[rep_head:].tobytes() == want_stats.tobytes()          # every record, staged or not, reached the host
+    assert int(counter[0]) == 0
+    recs = want_stats.view(_abi.STATS_DTYPE)
+    assert int(recs['overflow'].sum()) == (1 if overflow else 0) and (not overflow or recs['overflow'][1400] == 1)
+    # the decision itself, from the records, in the reference's float64 arithmetic
+    if not overflow:
+        l2 = [float(np.float32(np.sqrt(x)))**2 for x in recs['sumsq']]
+        norm = O.global_norm(l2)
+        assert float(rh['total_norm']) == norm
+        assert float(rh['combined_scale']) == float(ea.calc_combined_scale(loss_scale, norm, max_norm, True))
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+def test_refresh_workgroups_take_several_pieces(oracle, dtype):
+    """elx_writeback_mt with fewer workgroups per record than the record has pieces: three workgroups
+    walk the 100 pieces of the first record (the last piece partial) with the stride of the grid, and the
+    5 pieces of the second.  Every element equals the oracle's round-to-nearest-even cast."""
+    piece = _abi.refresh_piece_elems()
+    sizes = [100 * piece - 77, 5 * piece]
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    masters = [torch.randn(k, generator=gen, device=DEV) * 3.0 for k in sizes]
+    masters[0][:4] = torch.tensor([65504.0, 65520.0, -0.0, 1e-8], device=DEV)
+    outs = [torch.full((k, ), 7.0, dtype=dtype, device=DEV) for k in sizes]
+    rows = np.zeros(2, dtype=_abi.CHUNK_DTYPE)
+    for i in range(2):
+        rows[i]['lowp_out'], rows[i]['master'], rows[i]['n_alloc'] = outs[i].data_ptr(), masters[i].data_ptr(), sizes[i]
+    table = DeviceTable(rows, torch.device(DEV, 0))
+    stream = torch.cuda.current_stream().cuda_stream
+    _abi.check('elx_writeback_mt', _abi.load().elx_writeback_mt(table.ptr, 2, CODE[dtype], 3, 0, stream))
+    torch.cuda.synchronize()
+    for out, master in zip(outs, masters):
+        want = oracle.writeback(to_np(master), CODE[dtype])
+        got = to_np(out)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def _groups_one_per_tensor(entries):
+    """Every tensor a parameter group of its own, each with its own learning rate (layer-wise decay) and
+    one of three weight decays."""
+    return [dict(params=[p], lr=1e-3 * (0.97**i), weight_decay=(0.0, 0.01, 0.1)[i % 3]) for i, (_, _, p) in enumerate(entries)]
+
+
+@pytest.mark.parametrize('cap', [None, 64], ids=['control_block', 'host_fallback'])
+@pytest.mark.parametrize('gated', [True, False])
+def test_seventy_param_groups(oracle, monkeypatch, gated, cap):
+    """optimizer.py:246-265: the group hyper-parameters survive untouched, however many groups there
+    are.  70 tensors in 70 groups (distinct learning rates, three weight decays) over two fp16 chunks,
+    clipping on, three steps of which the second overflows.  Decided on the device through the control
+    block; with the device's capacity forced down to 64 records, decided on the host from the partials
+    the early stats launch left (the gradients are read once all the same); and with ``gated_step`` off.
+    Every step issues exactly one stats launch; the results follow the oracle."""
+    dtype = torch.float16
+    named = [(f't{i}', (257 + 61 * i, )) for i in range(70)]
+    total = sum(s[0] for _, s in named)
+    module, opt, ochunks = build_workload(named, 1 << int(math.ceil(math.log2(total / 2 + 20000))), dtype, seed=41,
+                                          grad_std=2e-2, loss_scale=128.0, groups_of=_groups_one_per_tensor,
+                                          max_norm=1.0, initial_scale=128.0, hysteresis=1)
+    assert len(module.param_chunks) == 2 and len(opt.param_groups) == 70
+    assert len({g['lr'] for g in opt.param_groups}) == 70
+    opt.gated_step = gated
+    if cap is not None:
+        opt.max_device_hypers = cap
+    scaler = O.DynamicGradScalerOracle(initial_scale=128.0, min_scale=1, max_scale=2**24, hysteresis=1)
+    launches = []
+    for name in ('grad_partials_mt', 'grad_stats_mt', 'grad_stats'):
+        real = getattr(_abi, name)
+        monkeypatch.setattr(_abi, name, lambda *a, _real=real, _name=name, **k: (launches.append(_name), _real(*a, **k))[1])
+    updates = []
+    for name in ('adam_step_gated_mt', 'adam_step_mt', 'adam_step_put_mt'):
+        real = getattr(_abi, name)
+        monkeypatch.setattr(_abi, name, lambda *a, _real=real, _name=name, **k: (updates.append(_name), _real(*a, **k))[1])
+    gen = torch.Generator(device=DEV).manual_seed(42)
+    for step in range(3):
+        if step:
+            for pc in module.param_chunks:
+                g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (2e-2 * opt.loss_scale)
+                g[pc.utilized_size:] = 0
+                pc.shard.copy_(g.to(dtype))
+                pc.invalidate_stats()
+            if step == 1:
+                module.param_chunks[1].shard[17] = float('-inf')
+            refresh_oracle_grads(module, ochunks)
+        launches.clear()
+        updates.clear()
+        opt.mark_gradients_scaled()
+        assert len(opt.optim._prepared.hyper_host) == 70
+        opt.step()
+        assert len(launches) == 1, launches                       # one pass over the gradients per step
+        info = O.reference_step(ochunks, CODE[dtype], scaler, max_norm=1.0)
+        assert opt.last_step_info['found_inf'] == info['found_inf'] == (step == 1)
+        assert opt.loss_scale == info['loss_scale']
+        if step == 1:
+            assert updates in ([], ['adam_step_gated_mt'])        # skipped: the host-decided step launches no update
+        else:
+            assert updates == (['adam_step_gated_mt'] if gated and cap is None else ['adam_step_mt'])
+            assert math.isclose(opt.last_step_info['combined_scale'], info['combined_scale'], rel_tol=1e-6)
+        compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-8, atol_v=1e-10, tag=f'step {step}')
+    assert [g['lr'] for g in opt.param_groups] == [1e-3 * (0.97**i) for i in range(70)]
+    assert opt.loss_scale == 64.0
+
+
+def test_more_groups_than_the_control_block_holds(oracle):
+    """300 groups: beyond the 256 records of the control block, the step is decided on the host from
+    the one pass over the gradients that went out early; identical bits to the same step with
+    ``gated_step`` off."""
+    dtype = torch.bfloat16
+    named = [(f't{i}', (64 + 8 * (i % 17), )) for i in range(300)]
+    states = []
+    for gated in (True, False):
+        module, opt, ochunks = build_workload(named, 1 << 14, dtype, seed=43, grad_std=1e-2, loss_scale=1.0,
+                                              groups_of=_groups_one_per_tensor, max_norm=0.5)
+        assert len(opt.param_groups) == 300 > _abi.max_ctl_hypers()
+        opt.gated_step = gated
+        opt.mark_gradients_scaled()
+        opt.step()
+        info = O.reference_step(ochunks, CODE[dtype], O.ConstantGradScalerOracle(1.0), max_norm=0.5)
+        assert opt.last_step_info['found_inf'] is False
+        assert math.isclose(opt.last_step_info['combined_scale'], info['combined_scale'], rel_tol=1e-6)
+        compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-8, atol_v=1e-10)
+        states.append([(pc.shard.clone(), pc.paired_chunk.shard.clone(), *[t.clone() for t in
+                                                                            opt._binding.moments(pc.paired_chunk)])
+                       for pc in module.param_chunks])
+    for a, b in zip(*states):
+        for x, y in zip(a, b):
+            assert torch.equal(x.view(torch.int16) if x.dtype == dtype else x, y.view(torch.int16) if y.dtype == dtype else y)

@@ -1083,7 +1083,7 @@ def test_finish_decide_matches_the_two_separate_launches():
     rec, hsz = _abi.STATS_DTYPE.itemsize, _abi.HYPER_DTYPE.itemsize
     ctl_head, rep_head = _abi.STEP_CTL_DTYPE.itemsize, _abi.STEP_REPORT_DTYPE.itemsize
     H = _abi.max_ctl_hypers()
-    assert (ctl_head, rep_head, H) == (32, 48, 64)
+    assert (ctl_head, rep_head, H) == (32, 48, 256)
     counter = torch.zeros(4, dtype=torch.int32, device=DEV)
     for trial in range(24):
         n = int(rng.integers(1, 9))

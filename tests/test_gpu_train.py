@@ -10,6 +10,7 @@ import torch
 import torch.nn as nn
 
 import elixir_amd as ea
+from elixir_amd import _abi
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda'
@@ -371,6 +372,114 @@ def test_chunks_land_from_hooks_during_backward(monkeypatch):
     module.module.zero_grad(set_to_none=True)
     opt.step()
     assert opt.last_step_info['found_inf'] is False
+
+
+def test_hook_driven_backward_takes_the_device_decided_step(oracle, monkeypatch):
+    """The flow training takes (module.py:177-190, fetcher.py:133-153: a chunk is reduced as soon as it is
+    ready; optimizer.py:137-142): ``opt.backward`` lands the chunks from the hooks, one launch per chunk,
+    the last chunk first.  The optimizer gave every chunk its record slot in chunk order when it was built,
+    so the flags still end up side by side and the step is decided on the device: no stats launch, no host
+    read before the update.  Its result has the bits of the host-decided step on the same gradients, and
+    of the oracle's step."""
+    import elixir_amd.chunk as C
+    from helpers import CODE, to_np
+    from oracle import oracle as O
+    dtype = torch.float16
+    torch.manual_seed(11)
+    model = Net().to(DEV)
+    twin = copy.deepcopy(model)
+    module, opt = wrap(model, dtype, initial_scale=256.0, hysteresis=1, max_norm=0.5)
+    module_h, opt_h = wrap(twin, dtype, initial_scale=256.0, hysteresis=1, max_norm=0.5)
+    opt_h.gated_step = False
+    chunks = module.param_chunks
+    assert len(chunks) >= 4
+    poison = {'on': False}
+
+    def maybe_poison(g):    # an overflow that backward itself produces, so that the landing sees it
+        if poison['on']:
+            g = g.clone()
+            g.view(-1)[3] = float('inf')
+        return g
+
+    model.head.weight.register_hook(maybe_poison)
+    slots = [c._stats_slot for c in chunks]
+    assert slots == list(range(slots[0], slots[0] + len(chunks))) and all(c._stats_pinned for c in chunks)
+
+    order = []
+    real_land = C._land_tensors_run
+
+    def spy_land(arena, run, *a, **k):
+        order.extend(run)
+        return real_land(arena, run, *a, **k)
+
+    monkeypatch.setattr(C, '_land_tensors_run', spy_land)
+    stats_launches = []
+    for name in ('grad_partials_mt', 'grad_stats_mt', 'grad_stats'):
+        real = getattr(_abi, name)
+        monkeypatch.setattr(_abi, name, lambda *a, _real=real, _name=name, **k: (stats_launches.append(_name), _real(*a, **k))[1])
+    reads = []
+    real_read = C.StatsArena.read
+    monkeypatch.setattr(C.StatsArena, 'read', lambda self, lo, hi: (reads.append((lo, hi)), real_read(self, lo, hi))[1])
+
+    gen = torch.Generator(device=DEV).manual_seed(12)
+    scaler = O.DynamicGradScalerOracle(initial_scale=256.0, min_scale=1, max_scale=2**24, hysteresis=1)
+    for step in range(3):
+        x = batch(gen)
+        order.clear()
+        opt.zero_grad()
+        poison['on'] = step == 1
+        opt.backward(module(x))
+        assert [c.chunk_id for c in order[:len(chunks)]] != sorted(c.chunk_id for c in chunks)    # not in chunk order
+        assert set(order) == set(chunks) and len(order) == len(chunks)                          # one launch per chunk
+        assert [c._stats_slot for c in chunks] == slots                                         # nobody moved
+        assert opt._stats_source() == ('arena', slots[0])
+        # the oracle's and the host-decided twin's view of the same gradients and state
+        ochunks = []
+        for pc in chunks:
+            fc = pc.paired_chunk
+            m, v = opt._binding.moments(fc)
+            segs = []
+            for group in opt.param_groups:
+                for fake in group['params']:
+                    if opt.param_to_optim_chunk[fake] is fc:
+                        b, e = opt.param_to_range[fake]
+                        segs.append(O.OracleSegment(b, e, lr=group['lr'], betas=tuple(group['betas']), eps=group['eps'],
+                                                    weight_decay=group['weight_decay'],
+                                                    bias_correction=group['bias_correction'],
+                                                    step=opt.state[fake]['step'] if opt.state[fake] else 0))
+            segs.sort(key=lambda sg: sg.begin)
+            ochunks.append(O.OracleChunk(lowp=to_np(pc.shard), master=to_np(fc.shard), m=to_np(m), v=to_np(v),
+                                         valid_end=pc.n_valid, segments=segs))
+        for pc, ph in zip(chunks, module_h.param_chunks):
+            ph.shard.copy_(pc.shard)
+            ph.invalidate_stats()
+        opt_h.mark_gradients_scaled()
+
+        stats_launches.clear()
+        reads.clear()
+        opt.step()
+        assert stats_launches == [] and reads == []      # the flags never left the device before the update
+        opt_h.step()
+        info = O.reference_step(ochunks, CODE[dtype], scaler, max_norm=0.5)
+        assert opt.last_step_info['found_inf'] == opt_h.last_step_info['found_inf'] == info['found_inf'] == (step == 1)
+        assert opt.loss_scale == opt_h.loss_scale == info['loss_scale']
+        if step != 1:
+            assert opt.last_step_info['combined_scale'] == opt_h.last_step_info['combined_scale']
+            assert opt.last_step_info['total_norm'] == opt_h.last_step_info['total_norm']
+            assert abs(opt.last_step_info['combined_scale'] - info['combined_scale']) <= 1e-6 * info['combined_scale']
+        for pc, ph, oc in zip(chunks, module_h.param_chunks, ochunks):
+            ma, va = opt._binding.moments(pc.paired_chunk)
+            mb, vb = opt_h._binding.moments(ph.paired_chunk)
+            for a, b in ((pc.shard, ph.shard), (pc.paired_chunk.shard, ph.paired_chunk.shard), (ma, mb), (va, vb)):
+                assert torch.equal(a.view(torch.int16) if a.dtype == dtype else a.view(torch.int32),
+                                   b.view(torch.int16) if b.dtype == dtype else b.view(torch.int32)), step
+            assert_close = np.testing.assert_allclose
+            assert_close(to_np(pc.paired_chunk.shard), oc.master, rtol=1e-6, atol=1e-9)
+            assert_close(to_np(ma), oc.m, rtol=1e-6, atol=1e-8)
+            assert_close(to_np(va), oc.v, rtol=1e-6, atol=1e-10)
+        module_h.mark_params_stale()
+    assert [st['step'] for st in opt.state.values()] == [st['step'] for st in opt_h.state.values()]
+    assert set(st['step'] for st in opt.state.values()) == {2}
 
 
 def test_tables_prepared_at_backward_follow_late_hyperparameter_changes():

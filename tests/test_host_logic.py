@@ -438,10 +438,84 @@ def test_land_rows_tile_every_piece_exactly():
             left -= n
             k += 1
     assert k == len(rows)
-    # block choice: a power of two of at least 16 tiles that keeps a 7.2 G element set below 32 Ki rows
-    assert _land_block_elems(1000, 2048) == 2048 * 2048 == _land_block_elems(7_247_757_312, 2048)
-    b = _land_block_elems(1 << 40, 2048)
-    assert b & (b - 1) == 0 and (1 << 40) // b <= 32768 < (1 << 40) // (b // 2)
+
+
+def test_land_block_is_sized_to_the_tensors():
+    """The grid of a per-tensor landing is (tiles of the longest row, rows): the block is chosen so that
+    few workgroups find no work.  Long tensors keep the 2048-tile block; a set of many short tensors gets
+    a shorter one; a set too large for 32 Ki rows a longer one.  Checked on the tensor lists of the three
+    model families, chunk by chunk (one launch per chunk, as backward issues them) and all at once."""
+    from elixir_amd import shapes as S
+    from elixir_amd.chunk import LAND_IDLE_ALLOWED, LAND_MAX_ROWS, _land_block_elems
+    from elixir_amd.module import greedy_groups
+    tile = 2048
+
+    def idle_share(counts, block):
+        counts = np.asarray(counts, dtype=np.int64)
+        rows = int((-(-counts // block)).sum())
+        work = int((-(-counts // tile)).sum())
+        width = min(block // tile, int((-(-counts // tile)).max()))
+        return rows, (rows * width - work) / work
+
+    assert _land_block_elems([1000], tile) == 2048 * tile                  # one short row: nothing idles
+    assert _land_block_elems([7_247_757_312], tile) == 2048 * tile         # one long tensor
+    b = _land_block_elems([1 << 40], tile)
+    assert b & (b - 1) == 0 and (1 << 40) // b <= LAND_MAX_ROWS < (1 << 40) // (b // 2)
+    for shapes, csize, expect_small in ((S.gpt2_shapes(), 64 << 20, True), (S.opt_shapes(), 128 << 20, True),
+                                        (S.llama_shapes(), 256 << 20, False)):
+        sizes = [S.numel(shape) for _, shape in shapes]
+        groups = greedy_groups(sizes, csize)
+        per_chunk = [[sizes[i] for i in g] + [csize - sum(sizes[i] for i in g)] for g in groups]    # tensors + padding
+        for counts in per_chunk + [[c for cs in per_chunk for c in cs]]:
+            counts = [c for c in counts if c > 0]
+            block = _land_block_elems(counts, tile)
+            assert block % tile == 0 and (block // tile) & (block // tile - 1) == 0 and 8 * tile <= block <= 2048 * tile
+            rows, idle = idle_share(counts, block)
+            assert rows <= LAND_MAX_ROWS and idle <= LAND_IDLE_ALLOWED + 1e-9, (len(counts), block // tile, rows, idle)
+            _, idle_at_2048 = idle_share(counts, 2048 * tile)
+            if idle_at_2048 <= LAND_IDLE_ALLOWED:
+                assert block == 2048 * tile
+        whole = [c for cs in per_chunk for c in cs if c > 0]
+        assert (_land_block_elems(whole, tile) < 2048 * tile) == expect_small
+
+
+def test_pinned_arena_slots_survive_any_landing_order():
+    """An optimizer pins its chunks' record slots in chunk order; landings in any order and grouping then
+    keep them, a landing over chunks whose slots do not follow each other is cut into runs, and chunks
+    nobody pinned still get consecutive slots per landing.  (CPU arena: nothing is launched.)"""
+    from elixir_amd.chunk import StatsArena
+
+    def chunk():
+        c = ea.Chunk(None, 64, torch.float16, None, shard_device='cpu', temp_device='cpu')
+        c.append_tensor(torch.zeros(8).half())
+        c.close_chunk()
+        return c
+
+    arena = StatsArena(torch.device('cpu'))
+    loose = chunk()
+    arena.assign([loose])
+    cs = [chunk() for _ in range(5)]
+    arena.pin(cs)
+    first = cs[0]._stats_slot
+    assert [c._stats_slot for c in cs] == [first + i for i in range(5)] and all(c._stats_pinned for c in cs)
+    arena.pin(cs)                                                    # again: nothing moves
+    assert [c._stats_slot for c in cs] == [first + i for i in range(5)]
+    for c in reversed(cs):                                           # last chunk first, one landing each
+        assert arena.runs([c]) == [[c]]
+    assert [c._stats_slot for c in cs] == [first + i for i in range(5)]
+    assert arena.runs(cs) == [cs]                                    # all at once: one run
+    assert arena.runs([cs[0], cs[2], cs[3]]) == [[cs[0]], [cs[2], cs[3]]]    # a gap cuts the landing in two
+    extra = [chunk(), chunk()]
+    runs = arena.runs([cs[4]] + extra + [loose])                     # pinned, then chunks without a pinned slot
+    assert runs == [[cs[4]], extra + [loose]]
+    assert extra[1]._stats_slot == extra[0]._stats_slot + 1 and loose._stats_slot == extra[1]._stats_slot + 1
+    assert [c._stats_slot for c in cs] == [first + i for i in range(5)]
+    arena.assign(cs[1:3])                                            # already side by side: kept, still pinned
+    assert cs[1]._stats_pinned and [c._stats_slot for c in cs] == [first + i for i in range(5)]
+    arena.assign([cs[3], cs[1]])                                     # an explicit assign out of order moves and unpins
+    assert not cs[1]._stats_pinned and not cs[3]._stats_pinned and cs[1]._stats_slot == cs[3]._stats_slot + 1
+    arena.pin(cs)                                                    # the optimizer is built again: a fresh run
+    assert all(c._stats_pinned for c in cs) and [c._stats_slot - cs[0]._stats_slot for c in cs] == list(range(5))
 
 
 # ------------------------------------------------------------------------------------------------

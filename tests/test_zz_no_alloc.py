@@ -13,6 +13,7 @@ pytestmark = pytest.mark.gpu
 DEV = 'cuda'
 REC = _abi.STATS_DTYPE.itemsize
 TORCH = {_abi.ELX_F16: torch.float16, _abi.ELX_BF16: torch.bfloat16, _abi.ELX_F32: torch.float32}
+_WARM = [False]
 
 
 def _grads(sizes, code, seed, poison=None):
@@ -43,10 +44,20 @@ def _both(table, n, code, bpc):
     want = torch.full((n * REC, ), 0xAB, dtype=torch.uint8, device=DEV)
     got = torch.full((n * REC, ), 0xCD, dtype=torch.uint8, device=DEV)
     _abi.grad_stats_mt(table.ptr, n, code, bpc, partials.data_ptr(), want.data_ptr(), False, stream)
-    before = torch.cuda.memory_allocated()
-    _abi.grad_stats_mt_static(table.ptr, n, code, bpc, got.data_ptr(), False, stream)
-    assert torch.cuda.memory_allocated() == before
+    if not _WARM[0]:    # the first call on a device looks the array's address up; what is measured is every later one
+        warm = torch.empty(n * REC, dtype=torch.uint8, device=DEV)
+        _abi.grad_stats_mt_static(table.ptr, n, code, bpc, warm.data_ptr(), False, stream)
+        _WARM[0] = True
     torch.cuda.synchronize()
+    # the driver's own count of free device memory (torch's allocator statistics would not see a hipMalloc
+    # made inside the library) and torch's, before the call and right after it, before anything is freed
+    free_before, _ = torch.cuda.mem_get_info()
+    torch_before = torch.cuda.memory_allocated()
+    _abi.grad_stats_mt_static(table.ptr, n, code, bpc, got.data_ptr(), False, stream)
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before and torch.cuda.memory_allocated() == torch_before
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
     return want.cpu().numpy().view(_abi.STATS_DTYPE), got.cpu().numpy().view(_abi.STATS_DTYPE)
 
 
@@ -95,3 +106,88 @@ def test_static_partials_refuse_what_does_not_fit():
     torch.cuda.synchronize()
     rec = out.cpu().numpy().view(_abi.STATS_DTYPE)
     assert not rec['overflow'].any() and not rec['sumsq'].any()
+
+
+def test_static_variant_inside_a_captured_graph():
+    """After one eager call on the device, the entry point can be recorded into a HIP graph (it
+    allocates nothing and looks nothing up any more): three replays over changing gradients, with eager
+    work and synchronisations between them, each equal to elx_grad_stats_mt on the same gradients."""
+    torch.cuda.set_device(0)
+    code, bpc = _abi.ELX_F16, 16
+    sizes = [200_000, 70_001, 4096]
+    grads = _grads(sizes, code, seed=21)
+    table = _table(grads, sizes)
+    n = len(sizes)
+    got = torch.zeros(n * REC, dtype=torch.uint8, device=DEV)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        _abi.grad_stats_mt_static(table.ptr, n, code, bpc, got.data_ptr(), False, side.cuda_stream)    # eager, first
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side, capture_error_mode='thread_local'):
+        _abi.grad_stats_mt_static(table.ptr, n, code, bpc, got.data_ptr(), False, torch.cuda.current_stream().cuda_stream)
+    partials = torch.empty(n * bpc * REC, dtype=torch.uint8, device=DEV)
+    want = torch.zeros(n * REC, dtype=torch.uint8, device=DEV)
+    for replay in range(3):
+        for i, g in enumerate(grads):    # the program's own eager work between the replays: new gradients
+            g.mul_(1.5)
+            if replay == 1 and i == 1:
+                g[77] = float('nan')
+        torch.cuda.synchronize()
+        got.fill_(0xCD)
+        graph.replay()
+        torch.cuda.synchronize()
+        _abi.grad_stats_mt(table.ptr, n, code, bpc, partials.data_ptr(), want.data_ptr(), False,
+                           torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        a, b = want.cpu().numpy().view(_abi.STATS_DTYPE), got.cpu().numpy().view(_abi.STATS_DTYPE)
+        assert a.tobytes() == b.tobytes(), replay
+        assert list(a['overflow']) == [0, 1 if replay >= 1 else 0, 0]
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import sys
+import numpy as np
+import torch
+sys.path.insert(0, sys.argv[1])
+from elixir_amd import _abi
+from elixir_amd.chunk import DeviceTable
+torch.cuda.set_device(0)
+g = torch.ones(4096, dtype=torch.float16, device='cuda')
+rows = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+rows[0]['grad'], rows[0]['n_alloc'], rows[0]['n_valid'] = g.data_ptr(), 4096, 4096
+table = DeviceTable(rows, torch.device('cuda', 0))
+out = torch.zeros(16, dtype=torch.uint8, device='cuda')
+side = torch.cuda.Stream()
+torch.cuda.synchronize()
+graph = torch.cuda.CUDAGraph()
+code = None
+with torch.cuda.graph(graph, stream=side, capture_error_mode='thread_local'):
+    try:
+        _abi.grad_stats_mt_static(table.ptr, 1, _abi.ELX_F16, 1, out.data_ptr(), False, torch.cuda.current_stream().cuda_stream)
+    except _abi.ElxError as e:
+        code = e.code
+assert code == _abi.ELX_E_STATE, code
+# outside capture the same call goes through, and from then on it may be captured
+_abi.grad_stats_mt_static(table.ptr, 1, _abi.ELX_F16, 1, out.data_ptr(), False, torch.cuda.current_stream().cuda_stream)
+torch.cuda.synchronize()
+rec = out.cpu().numpy().view(_abi.STATS_DTYPE)[0]
+assert rec['sumsq'] == 4096.0 and rec['overflow'] == 0, rec
+print('refused under capture, accepted afterwards')
+"""
+
+
+def test_first_call_on_a_device_under_capture_is_refused(tmp_path):
+    """The first call on a device has to look the array's address up, which is not something to do while a
+    stream captures: it is refused with ELX_E_STATE before anything is launched (in a process of its own:
+    in this one the address is known already)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = tmp_path / 'first_call.py'
+    script.write_text(_FIRST_CALL_UNDER_CAPTURE)
+    proc = subprocess.run([sys.executable, str(script), root], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                          timeout=300)
+    assert proc.returncode == 0, proc.stdout
+    assert 'refused under capture, accepted afterwards' in proc.stdout
