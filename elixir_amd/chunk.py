@@ -88,10 +88,19 @@ class DeviceTable:
         return len(self.host)
 
 
-def stats_launch_blocks(n_valid_max: int) -> int:
+CACHED_STATS_WORKGROUPS = 1280    # whole launch, when the gradients are served from the memory-side cache
+
+
+def stats_launch_blocks(n_valid_max: int, n_chunks: int = 1, cached: bool = False) -> int:
     """Workgroups per chunk for the stats pass: enough to fill 256 compute units several times
-    over for large chunks, one per 16 Ki elements for small ones."""
-    return int(max(1, min(1024, math.ceil(n_valid_max / 16384))))
+    over for large chunks, one per 16 Ki elements for small ones.  A set that the memory-side cache
+    serves (``cached``: the launch reads it with ordinary loads) is read fastest by about five workgroups
+    per compute unit in all -- the two chunks of GPT-2 small: 43 us with 384 to 896 workgroups per chunk,
+    47 us with 1024 (every compute unit filled to its eight) and 46 us with 320."""
+    blocks = int(max(1, min(1024, math.ceil(n_valid_max / 16384))))
+    if cached:
+        blocks = max(1, min(blocks, CACHED_STATS_WORKGROUPS // max(1, n_chunks)))
+    return blocks
 
 
 # The memory-side cache of the GPU holds 256 MiB.  A gradient set below this size is read by the stats pass
@@ -117,7 +126,8 @@ def launch_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.dev
     n = len(chunk_rows)
     if table is None:
         table = DeviceTable(chunk_rows, device)
-    bpc = stats_launch_blocks(int(chunk_rows['n_valid'].max()))
+    cached = keep_grads_cached(chunk_rows, grad_dtype)
+    bpc = stats_launch_blocks(int(chunk_rows['n_valid'].max()), n, cached)
     aligned = bool(np.all(chunk_rows['grad'] % 16 == 0))
     if workspace is None:
         workspace = {}
@@ -130,8 +140,7 @@ def launch_grad_stats(chunk_rows: np.ndarray, grad_dtype: int, device: torch.dev
     d_partials = buf.data_ptr()
     d_stats = d_partials + n * bpc * _abi.STATS_DTYPE.itemsize
     stream = torch.cuda.current_stream(device).cuda_stream
-    _abi.grad_stats_mt(table.ptr, n, grad_dtype, bpc, d_partials, d_stats, not aligned, stream,
-                       keep_cached=keep_grads_cached(chunk_rows, grad_dtype))
+    _abi.grad_stats_mt(table.ptr, n, grad_dtype, bpc, d_partials, d_stats, not aligned, stream, keep_cached=cached)
     return buf[n * bpc * _abi.STATS_DTYPE.itemsize:need]
 
 
@@ -320,15 +329,18 @@ def _land_chunks_run(arena: 'StatsArena', chunks: List['Chunk'], payloads: List[
 
 LAND_MAX_BLOCK_TILES = 2048    # tiles per row where a launch over long tensors was measured to stream best
 LAND_MAX_ROWS = 32768          # the grid's y extent must stay below 65536
-LAND_IDLE_ALLOWED = 0.10       # share of workgroups without work that a larger block may cost
+LAND_IDLE_ALLOWED = 0.025      # share of workgroups without work that a larger block may cost
 
 
 def _land_block_elems(counts, tile: int) -> int:
     """Rows of a per-tensor landing are blocks of a power-of-two number of tiles.  The launch is a grid of
     (tiles of the longest row, rows), so every row shorter than that leaves workgroups that find no work:
     with blocks of 2048 tiles the 148 gradients of GPT-2 small (768 ... 38.6 M elements) make 327,680
-    workgroups for 65,536 tiles of work and the launch runs at half its speed.  ``counts``: the element
-    counts of the pieces.  Picks the largest block, up to ``LAND_MAX_BLOCK_TILES`` tiles, whose launch
+    workgroups for 65,536 tiles of work and the launch runs at half its speed (178 us; 99 us with blocks of
+    16 tiles, 103 us for the same shards landed from whole payloads).  Short blocks cost nothing on the
+    device -- OPT-1.3B: 1.007 / 0.950 / 0.917 / 0.909 ms with 2048 / 512 / 128 / 64 tiles, LLaMA-7B 4.317 /
+    4.279 / 4.303 ms with 2048 / 512 / 128 -- only host time when the table is first built.  ``counts``: the
+    element counts of the pieces.  Picks the largest block, up to ``LAND_MAX_BLOCK_TILES`` tiles, whose launch
     has at most ``LAND_IDLE_ALLOWED`` idle workgroups (failing that, the block with the fewest
     workgroups) among those that keep the launch within ``LAND_MAX_ROWS`` rows; a set too large for that
     gets longer blocks."""
@@ -437,28 +449,32 @@ def _land_tensors_run(arena: 'StatsArena', chunks: List['Chunk'], pieces, tile: 
     """One launch: the records of ``chunks`` are consecutive slots of ``arena``; ``pieces`` as for
     ``land_rows``, slots counted from the first chunk of the run."""
     device = chunks[0].shard_device
-    block = _land_block_elems([count for _, _, _, count in pieces], tile)
-    rows, slot_offsets = land_rows(pieces, len(chunks), block, ssize, dsize)
-    if len(rows) > 65535:
-        raise RuntimeError(f'{len(rows)} rows in one landing launch: land fewer chunks at a time')
-    bpr = _abi.check_land_rows(rows, slot_offsets, src_code, dst_code)
     ws = chunks[0]._workspace
-    need = _abi.land_workspace_records(len(rows), bpr, len(chunks)) * arena.itemsize
+    # The tables of a landing are the same from step to step whenever the gradients come back at the same
+    # addresses: they are kept, device copies included, under the list of pieces they were built from (building
+    # them again costs the host a millisecond per 20,000 rows, and an upload from pageable memory makes it wait
+    # for the stream).
+    tables = ws.setdefault('land_tables', {})
+    key = (tuple(pieces), tuple(c.chunk_id for c in chunks), src_code, dst_code)
+    kept = tables.get(key)
+    if kept is None:
+        block = _land_block_elems([count for _, _, _, count in pieces], tile)
+        rows, slot_offsets = land_rows(pieces, len(chunks), block, ssize, dsize)
+        if len(rows) > 65535:
+            raise RuntimeError(f'{len(rows)} rows in one landing launch: land fewer chunks at a time')
+        bpr = _abi.check_land_rows(rows, slot_offsets, src_code, dst_code)
+        if len(tables) >= LAND_TABLES_KEPT:
+            tables.pop(next(iter(tables)))
+        kept = tables[key] = (DeviceTable(rows, device), torch.from_numpy(slot_offsets.view(np.int32).copy()).to(device),
+                              bpr)
+    table, offsets, bpr = kept
+    n_rows = len(table)
+    need = _abi.land_workspace_records(n_rows, bpr, len(chunks)) * arena.itemsize
     buf = ws.get('land')
     if buf is None or buf.numel() < need:
         buf = ws['land'] = torch.empty(need, dtype=torch.uint8, device=device)
-    # The tables of a landing are the same from step to step whenever the gradients come back at the same
-    # addresses: their device copies are kept (an upload from pageable memory makes the host wait for the stream).
-    tables = ws.setdefault('land_tables', {})
-    key = (rows.tobytes(), slot_offsets.tobytes())
-    kept = tables.get(key)
-    if kept is None:
-        if len(tables) >= LAND_TABLES_KEPT:
-            tables.pop(next(iter(tables)))
-        kept = tables[key] = (DeviceTable(rows, device), torch.from_numpy(slot_offsets.view(np.int32).copy()).to(device))
-    table, offsets = kept
     stream = torch.cuda.current_stream(device).cuda_stream
-    _abi.land_grads_mt(table.ptr, len(rows), src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
+    _abi.land_grads_mt(table.ptr, n_rows, src_code, dst_code, float(np.float32(mul)), bpr, buf.data_ptr(),
                        arena.ptr(chunks[0]._stats_slot), True, stream, LAND_BLOCKS_PER_CU,
                        d_slot_offsets=offsets.data_ptr(), n_slots=len(chunks),
                        keep_cached=sum(c.n_valid for c in chunks) * dsize <= KEEP_GRADS_CACHED_BELOW)

@@ -71,10 +71,34 @@ def hyper_record_cached(key: Tuple, adamw_mode: bool) -> np.ndarray:
     if rec is None:
         if len(_HYPER_RECORDS) > 4096:
             _HYPER_RECORDS.clear()
+            _HYPER_ADDRESSES.clear()
         lr, b1, b2, eps, wd, step, bc = key
         rec = _HYPER_RECORDS[(key, adamw_mode)] = make_hyper_record(lr, b1, b2, eps, wd, step, bc, adamw_mode)
         rec.flags.writeable = False    # shared between steps: nobody edits it
     return rec
+
+
+_HYPER_ADDRESSES: Dict = {}
+
+
+def hyper_record_address(key: Tuple, adamw_mode: bool) -> int:
+    """Host address of the cached record for ``key`` (the record stays alive in the cache, which is emptied
+    together with this table)."""
+    ptr = _HYPER_ADDRESSES.get((key, adamw_mode))
+    if ptr is None:
+        if (key, adamw_mode) not in _HYPER_RECORDS or len(_HYPER_ADDRESSES) > 4096:
+            _HYPER_ADDRESSES.clear()
+        ptr = _HYPER_ADDRESSES[(key, adamw_mode)] = hyper_record_cached(key, adamw_mode).ctypes.data
+    return ptr
+
+
+def _raw_current_stream(device: torch.device) -> int:
+    """The current stream's handle.  torch keeps a direct getter for it, a third of the cost of building a
+    ``torch.cuda.Stream`` object first; without that getter the object's handle is taken."""
+    getter = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+    if getter is not None:
+        return getter(device.index if device.index is not None else torch.cuda.current_device())
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 class _SteadyStep:
@@ -85,7 +109,7 @@ class _SteadyStep:
     the launch itself takes under 70, and whatever the host needs in front of it the device spends idle."""
 
     __slots__ = ('watch', 'layout', 'states', 'step', 'group_of_hyper', 'dplan', 'grad_code', 'device', 'call', 'fixed',
-                 'tail', 'pack', 'pack_ptr')
+                 'tail', 'flags', 'pack', 'pack_ptr')
 
     def __init__(self, watch, layout, prep: '_Prepared', step: int, group_of_hyper):
         plan = prep.dplan.plan
@@ -95,6 +119,7 @@ class _SteadyStep:
         self.call = _abi.load().elx_adam_step_put_mt
         self.fixed = (prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs))
         self.tail = (plan.info.total_tiles, plan.info.max_tiles)
+        self.flags = plan.info.flags
         n = len(group_of_hyper)
         self.pack = np.zeros(n, dtype=_abi.HYPER_DTYPE) if n > 1 else None    # several records: gathered here
         self.pack_ptr = self.pack.ctypes.data if n > 1 else 0
@@ -485,8 +510,7 @@ class HybridAdam(torch.optim.Optimizer):
         step = steady.step + 1
         if steady.pack is None:
             key = self._group_key(groups[steady.group_of_hyper[0]], step)
-            rec = hyper_record_cached(key, self.adamw_mode)
-            ptr = rec.__array_interface__['data'][0]
+            ptr = hyper_record_address(key, self.adamw_mode)
             keys = (key, )
         else:
             keys = tuple(self._group_key(groups[gi], step) for gi in steady.group_of_hyper)
@@ -495,11 +519,10 @@ class HybridAdam(torch.optim.Optimizer):
             for h, key in enumerate(keys):
                 steady.pack[h] = hyper_record_cached(key, self.adamw_mode)[0]
             ptr = steady.pack_ptr
-        plan = steady.dplan.plan
-        stream = torch.cuda.current_stream(steady.device).cuda_stream
+        stream = _raw_current_stream(steady.device)
         d_hypers = self._hyper_table_dev.reserve(len(keys) * _abi.HYPER_DTYPE.itemsize, steady.device)
         code = steady.call(*steady.fixed, ptr, d_hypers, len(keys), *steady.tail, float(div_scale), steady.grad_code,
-                           _abi.ELX_NONE, plan.info.flags, self.blocks_per_cu, stream)
+                           _abi.ELX_NONE, steady.flags, self.blocks_per_cu, stream)
         if code != 0:
             _abi.check('elx_adam_step_put_mt', code)
         # the launch is out: bookkeeping, and the records of the step after this one
@@ -507,7 +530,7 @@ class HybridAdam(torch.optim.Optimizer):
             state['step'] = step
         steady.step = step
         for (lr, b1, b2, eps, wd, st, bc) in keys:
-            hyper_record_cached((lr, b1, b2, eps, wd, st + 1, bc), self.adamw_mode)
+            hyper_record_address((lr, b1, b2, eps, wd, st + 1, bc), self.adamw_mode)
 
     def commit_step(self) -> None:
         """The launched step happened: step counts advance (after the launches, so that the device is

@@ -554,10 +554,11 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 rows[i]['grad'] = c.shard.data_ptr()
                 rows[i]['n_alloc'] = c.shard_size
                 rows[i]['n_valid'] = c.n_valid
+            cached = (all(c.shard.is_cuda for c in chunks)
+                      and keep_grads_cached(rows, dtype_code(chunks[0].chunk_dtype)))
             self._all_stats_table = ((ids, ptrs), DeviceTable(rows, device),
-                                     stats_launch_blocks(int(rows['n_valid'].max())), bool(np.all(rows['grad'] % 16 == 0)),
-                                     all(c.shard.is_cuda for c in chunks)
-                                     and keep_grads_cached(rows, dtype_code(chunks[0].chunk_dtype)))
+                                     stats_launch_blocks(int(rows['n_valid'].max()), len(chunks), cached),
+                                     bool(np.all(rows['grad'] % 16 == 0)), cached)
         return self._all_stats_table[1:]
 
     def _step_on_device(self, source) -> bool:
