@@ -32,7 +32,7 @@ Differences from the reference, all on purpose:
 import logging
 import math
 import time
-from collections import defaultdict
+from collections import OrderedDict, defaultdict
 from enum import Enum
 from typing import Dict, List, Set, Tuple
 
@@ -44,12 +44,23 @@ from . import _abi
 from .chunk import (Chunk, DeviceTable, StatsArena, dtype_code, keep_grads_cached, kernel_device, launch_grad_stats,
                     read_grad_stats, resolve_pending_stats, stats_launch_blocks)
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
-from .hybrid_adam import CPUAdam, FusedAdam, HybridAdam
+from .hybrid_adam import CPUAdam, FusedAdam, HybridAdam, _global_step_hooks
 
 _AVAIL_OPTIM_LIST = {FusedAdam, CPUAdam, HybridAdam}
 
 # the one runtime signal of this path in the reference: optimizer.py:88 (a distributed logger) and :199
 logger = logging.getLogger('elixir_amd.optimizer')
+
+
+# What the wrapper and the inner optimizer bound to it read and call on a chunk object.  The first tuple is what
+# the reference's wrapper uses of its own Chunk (optimizer.py:58-66,115-164,238-256; chunk.py:59-139); the second
+# is what this build's step needs on top: where the flags of the gradients are kept between a landing launch and
+# the step (a record slot in a device arena, fetched lazily), and the bookkeeping around it.
+CHUNK_MEMBERS_OF_THE_REFERENCE = ('tensors_info', 'shard_begin', 'shard_size', 'shard', 'paired_chunk', 'overflow',
+                                  'l2_norm', 'l2_norm_flag', 'optim_update', 'optim_sync_flag', 'torch_pg', 'is_replica',
+                                  'chunk_dtype', 'shard_device', 'chunk_id')
+CHUNK_MEMBERS_ADDED = ('n_valid', 'invalidate_stats', '_apply_stats', '_overflow', '_stats_fresh', '_stats_pending',
+                       '_stats_slot', '_stats_pinned', '_stats_home', '_stats_event', '_stats_stream', '_take_stats_slot')
 
 
 class OptimState(Enum):
@@ -187,6 +198,10 @@ class ElixirOptimizer(torch.optim.Optimizer):
                  norm_type: float = 2.0,
                  init_step=False):
         self.optim = optimizer
+        # Optimizer.__init__ is not run (the groups, the state and the defaults are the inner optimizer's), so
+        # what it would have set up for hooks registered on THIS object is set up here; step() dispatches them
+        self._optimizer_step_pre_hooks = OrderedDict()
+        self._optimizer_step_post_hooks = OrderedDict()
         for attr in ('param_chunk_group', 'optim_chunk_group', 'fetcher', 'use_amp'):
             assert hasattr(module, attr), f'module lacks {attr}: it is not a chunked module'
         self.scaled_optimizer = False
@@ -295,6 +310,26 @@ class ElixirOptimizer(torch.optim.Optimizer):
 
     def add_param_group(self, *args, **kwargs):
         return self.optim.add_param_group(*args, **kwargs)
+
+    # hooks around state_dict / load_state_dict belong to the optimizer that produces and takes the state
+    def register_state_dict_pre_hook(self, *args, **kwargs):
+        return self.optim.register_state_dict_pre_hook(*args, **kwargs)
+
+    def register_state_dict_post_hook(self, *args, **kwargs):
+        return self.optim.register_state_dict_post_hook(*args, **kwargs)
+
+    def register_load_state_dict_pre_hook(self, *args, **kwargs):
+        return self.optim.register_load_state_dict_pre_hook(*args, **kwargs)
+
+    def register_load_state_dict_post_hook(self, *args, **kwargs):
+        return self.optim.register_load_state_dict_post_hook(*args, **kwargs)
+
+    def __getstate__(self):
+        raise TypeError('an ElixirOptimizer is tied to the chunk storage of its module and cannot be copied or '
+                        'pickled: save state_dict() and load it into a newly built one')
+
+    def __deepcopy__(self, memo):
+        self.__getstate__()
 
     def state_dict(self):
         """The inner optimizer's state in torch's packed layout (step, exp_avg, exp_avg_sq per fake
@@ -671,6 +706,23 @@ class ElixirOptimizer(torch.optim.Optimizer):
     # ------------------------------------------------------------------ the step
 
     def step(self, *args, **kwargs):
+        """optimizer.py:185-220.  Step hooks registered on this object (``register_step_pre_hook`` /
+        ``register_step_post_hook``) and torch's process-wide ones run around it, in torch's order."""
+        global_pre, global_post = _global_step_hooks()
+        if not (global_pre or global_post or self._optimizer_step_pre_hooks or self._optimizer_step_post_hooks):
+            return self._step(*args, **kwargs)
+        for hook in list(global_pre.values()) + list(self._optimizer_step_pre_hooks.values()):
+            result = hook(self, args, kwargs)
+            if result is not None:
+                if not (isinstance(result, tuple) and len(result) == 2):
+                    raise RuntimeError(f'{hook} must return None or a tuple of (new_args, new_kwargs), but got {result}.')
+                args, kwargs = result
+        out = self._step(*args, **kwargs)
+        for hook in list(self._optimizer_step_post_hooks.values()) + list(global_post.values()):
+            hook(self, args, kwargs)
+        return out
+
+    def _step(self, *args, **kwargs):
         if (self.gated_step and self._binding is not None and self.scaled_optimizer and not args and not kwargs
                 and not self._binding.zero_grads and self.optim_state == OptimState.SCALED):
             source = self._stats_source()

@@ -342,3 +342,78 @@ def test_device_code_has_no_packed_fp32_and_no_spills(tmp_path):
     # the update kernels keep a small register footprint: residency is capped by the LDS reservation, not by registers
     vgprs = [int(v) for v in re.findall(r'\.vgpr_count:\s*(\d+)', text)]
     assert max(vgprs) <= 128
+
+
+def test_unscale_mode_and_lds_reservation_queries():
+    """How a launch divides by div_scale, and the LDS reservation that caps residency, as the library's own
+    host code decides them: the exact-reciprocal rule against its definition (a power of two whose reciprocal
+    is a normal fp32 number), on every power of two and on neighbours of powers of two."""
+    assert _abi.unscale_mode(-1.0) == (0, 1.0) and _abi.unscale_mode(0.0) == (0, 1.0)
+    assert _abi.unscale_mode(float('nan'))[0] == 0
+    for e in range(-149, 128):
+        s = float(np.ldexp(np.float32(1.0), e))
+        mode, inv = _abi.unscale_mode(s)
+        with np.errstate(all='ignore'):
+            recip = np.float32(1.0) / np.float32(s)
+        # both the divisor and its reciprocal normal numbers; 2**126, whose reciprocal is the smallest normal
+        # number, is left to the division (same bits either way)
+        exact = -126 <= e <= 125
+        assert not exact or (np.isfinite(recip) and recip >= np.float32(1.17549435e-38) and recip * np.float32(s) == 1.0)
+        assert mode == (1 if exact else 2), (e, mode)
+        assert inv == (float(recip) if exact else 1.0)
+        if -126 <= e < 127:
+            for neighbour in (np.nextafter(np.float32(s), np.float32(np.inf)), np.nextafter(np.float32(s), np.float32(0))):
+                assert _abi.unscale_mode(float(neighbour)) == (2, 1.0)
+    assert _abi.unscale_mode(float('inf')) == (2, 1.0)
+    # the reservation: a multiple of 256 bytes that lets exactly the asked number of workgroups share 160 KiB
+    for k in range(3, 33):
+        lds = _abi.occupancy_lds_bytes(k)
+        assert lds % 256 == 0 and lds <= 65536 and (160 * 1024) // lds >= k and (160 * 1024) // (lds + 256) <= k
+    assert _abi.occupancy_lds_bytes(0) == _abi.occupancy_lds_bytes(12)
+    for bad in (1, 2, 33, 1000):
+        with pytest.raises(_abi.ElxError) as e:
+            _abi.occupancy_lds_bytes(bad)
+        assert e.value.code == _abi.ELX_E_SIZE
+
+
+SANITIZED_TESTS = ('test_check_tables_property_random', 'test_check_tables_accepts_and_rejects',
+                   'test_check_tables_reports_alignment_and_tile_counts', 'test_check_land_rows_accepts_and_rejects',
+                   'test_unscale_mode_and_lds_reservation_queries')
+
+
+def test_validators_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    """The table validators are what keeps a kernel inside its buffers, so their own reads must stay inside
+    the tables they are given: the host-only source file of the library is compiled alone with g++
+    -fsanitize=address,undefined, and the validator tests of this file (and the land-row tests of
+    test_host_logic.py) run once more against that build, in a child process whose allocator is
+    AddressSanitizer's (every numpy table then sits between red zones).  A read or write outside a table, or
+    any undefined arithmetic, ends the child with a report."""
+    import subprocess
+    import sys
+    from elixir_amd import build as B
+    if os.environ.get('ELX_HOST_CHECKED_LIB'):
+        pytest.skip('this is the child run')
+    lib = B.build_host_checked(str(tmp_path / 'libelx_host_checked.so'))
+    asan = subprocess.run(['g++', '-print-file-name=libasan.so'], check=True, stdout=subprocess.PIPE, text=True).stdout.strip()
+    asan = os.path.realpath(asan)
+    assert os.path.exists(asan), 'the AddressSanitizer runtime of g++ was not found'
+    env = dict(os.environ)
+    env['ELX_HOST_CHECKED_LIB'] = lib
+    # the runtime has to be the first library of the process; whatever else is preloaded stays behind it
+    env['LD_PRELOAD'] = asan + (':' + env['LD_PRELOAD'] if env.get('LD_PRELOAD') else '')
+    env['ASAN_OPTIONS'] = 'detect_leaks=0:abort_on_error=0:exitcode=97'
+    env['UBSAN_OPTIONS'] = 'halt_on_error=1:print_stacktrace=1'
+    here = os.path.dirname(os.path.abspath(__file__))
+    select = ' or '.join(SANITIZED_TESTS + ('test_land_rows_tile_every_piece_exactly', 'test_launch_plan_properties_random'))
+    proc = subprocess.run([sys.executable, '-m', 'pytest', '-x', '-q', '-p', 'no:cacheprovider',
+                           os.path.join(here, 'test_abi.py'), os.path.join(here, 'test_host_logic.py'), '-k', select],
+                          env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    tail = proc.stdout[-3000:]
+    assert proc.returncode == 0, tail
+    assert 'passed' in tail and 'ERROR: AddressSanitizer' not in proc.stdout and 'runtime error' not in proc.stdout, tail
+    # and the child really called into the checked build
+    probe = subprocess.run([sys.executable, '-c',
+                            'import sys; sys.path.insert(0, sys.argv[1]); from elixir_amd import _abi; '
+                            'L = _abi.host_lib(); print(L._name); print(_abi.tile_elems())', ROOT],
+                           env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert probe.returncode == 0 and 'libelx_host_checked.so' in probe.stdout and '256' in probe.stdout, probe.stdout[-2000:]

@@ -626,6 +626,121 @@ def test_hybrid_adam_dispatches_step_hooks_itself():
     assert seen == [('pre', (None, 4.0), dict(gated=False, defer_commit=False))]
 
 
+def test_wrapper_runs_step_hooks_in_torchs_order_and_refuses_to_be_copied(monkeypatch):
+    """Hooks registered on the wrapper -- which is an Optimizer that never ran Optimizer.__init__ -- and
+    torch's process-wide hooks fire around its step in torch's order: global pre, own pre, the step, own
+    post, global post; a pre-hook may replace the arguments.  State-dict hooks go to the inner optimizer,
+    whose state it is.  Copying or pickling the wrapper is refused with the reason."""
+    import copy
+    import pickle
+    from torch.optim.optimizer import register_optimizer_step_post_hook, register_optimizer_step_pre_hook
+    module, opt = _cpu_optimizer(5)
+    seen = []
+    monkeypatch.setattr(opt, '_step', lambda *a, **k: seen.append(('step', a, k)) or 'ret')
+    handles = [register_optimizer_step_pre_hook(lambda o, a, k: seen.append('global pre') if o is opt else None),
+               register_optimizer_step_post_hook(lambda o, a, k: seen.append('global post') if o is opt else None),
+               opt.register_step_pre_hook(lambda o, a, k: (seen.append('own pre'), ((), dict(marker=1)))[1]),
+               opt.register_step_post_hook(lambda o, a, k: seen.append(('own post', k)))]
+    try:
+        assert opt.step() == 'ret'
+    finally:
+        for h in handles:
+            h.remove()
+    assert seen == ['global pre', 'own pre', ('step', (), dict(marker=1)), ('own post', dict(marker=1)), 'global post']
+    seen.clear()
+    opt.step()                                   # no hook left: straight through
+    assert seen == [('step', (), {})]
+    # a torch that names its process-wide hook tables differently: no such hooks, no AttributeError
+    import torch.optim.optimizer as TO
+    from elixir_amd.hybrid_adam import _global_step_hooks
+    monkeypatch.delattr(TO, '_global_optimizer_pre_hooks')
+    monkeypatch.delattr(TO, '_global_optimizer_post_hooks')
+    assert _global_step_hooks() == ({}, {})
+    monkeypatch.undo()
+    called = []
+    opt.register_state_dict_post_hook(lambda o, sd: called.append(type(o).__name__))
+    opt.state_dict()
+    assert called == ['HybridAdam']
+    for attempt in (lambda: copy.deepcopy(opt), lambda: pickle.dumps(opt)):
+        with pytest.raises(TypeError, match='cannot be copied or pickled'):
+            attempt()
+
+
+def test_the_chunk_members_the_optimizer_touches_are_the_documented_ones():
+    """A chunk object has to offer the members the reference's wrapper reads of its own Chunk plus a dozen
+    that this build adds (where the flags wait between landing and step).  Stand-ins that carry exactly
+    those -- anything else raises AttributeError -- go through the wrapper's host logic: construction
+    with the ranges of optimizer.py:238-265, the flags, the global norm, the combined scale, the
+    decision where the flags come from, the state dict."""
+    from elixir_amd.optimizer import CHUNK_MEMBERS_ADDED, CHUNK_MEMBERS_OF_THE_REFERENCE
+    allowed = set(CHUNK_MEMBERS_OF_THE_REFERENCE) | set(CHUNK_MEMBERS_ADDED)
+
+    class StandIn:
+        """Exactly the documented members, taken from a real chunk; sorted and hashed like one."""
+
+        def __init__(self, real):
+            object.__setattr__(self, '_real', real)
+
+        def __getattr__(self, name):
+            if name not in allowed:
+                raise AttributeError(f'{name} is not among the documented chunk members')
+            value = getattr(object.__getattribute__(self, '_real'), name)
+            return value
+
+        def __setattr__(self, name, value):
+            if name not in allowed:
+                raise AttributeError(f'{name} is not among the documented chunk members')
+            setattr(object.__getattribute__(self, '_real'), name, value)
+
+        def __hash__(self):
+            return self.chunk_id
+
+        def __eq__(self, other):
+            return isinstance(other, StandIn) and other.chunk_id == self.chunk_id
+
+        def __lt__(self, other):
+            return self.chunk_id < other.chunk_id
+
+    module, _ = _cpu_optimizer(9)
+    real_chunks = module.param_chunks
+    stand = {c: StandIn(c) for c in real_chunks}
+    stand_optim = {c.paired_chunk: StandIn(c.paired_chunk) for c in real_chunks}
+
+    class Shim:    # what the wrapper reads of the module (optimizer.py:58-66,77,253)
+        use_amp = module.use_amp
+        optim_chunk_group = module.optim_chunk_group
+
+        class param_chunk_group:
+            fused_chunks = set()
+            float_chunks = set(stand.values())
+
+        class fetcher:
+            @staticmethod
+            def get_one_chunk(param):
+                return stand[module.fetcher.get_one_chunk(param)]
+
+    for c, s in stand.items():    # the pairing, between stand-ins
+        c.paired_chunk = stand_optim[c.paired_chunk]
+        c.paired_chunk._real.paired_chunk = s
+    params = [p for p in module.parameters()]
+    opt = ea.ElixirOptimizer(Shim, ea.HybridAdam(params, lr=1e-3), initial_scale=8.0, max_norm=2.0)
+    assert len(opt.param_to_range) == len(params) and all(b < e for b, e in opt.param_to_range.values())
+    chunks = opt._param_chunk_list
+    assert chunks == sorted(stand.values()) and all(c.l2_norm_flag for c in chunks)
+    assert opt._stats_source() == ('launch', None)
+    for i, c in enumerate(chunks):
+        c._apply_stats(False, 4.0 * (i + 1))
+    assert opt._check_overflow() is False
+    assert opt._calc_global_norm() == pytest.approx(math.sqrt(sum(4.0 * (i + 1) for i in range(len(chunks)))), rel=1e-6)
+    opt.optim_state = ea.OptimState.SCALED
+    assert opt._get_combined_scale() > 0
+    chunks[-1]._apply_stats(True, 1.0)
+    assert opt._check_overflow() is True
+    opt._clear_optim_states()
+    assert opt._stats_source() == ('launch', None) and opt._check_overflow() is False
+    assert len(opt.state_dict()['state']) == len(params)
+
+
 def test_every_optimizer_of_the_references_scaled_list_is_here():
     """optimizer.py:19 lists the optimizers that may be handed a ``div_scale``: FusedAdam, CPUAdam and
     HybridAdam.  All three exist with ColossalAI's argument order, count as scaled optimizers inside the
