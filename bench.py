@@ -31,20 +31,25 @@ BYTES_STATS = 2                 # per valid element: the compulsory second read 
 # HBM bytes per adam_step_kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script, scaled by what the same counters read for a plain copy of known size (--calibrate-copy).
 # Counter runs cannot ride along with a timed run, so the figure is a recorded one: it is only put into
-# the line while the kernel source is still the one it was measured on (sha256 of elx_kernels.hip,
-# first 16 hex digits), and the line names the summary it comes from.
+# the line while the device code is still the one it was measured on (sha256 over elx_kernels.hip and
+# elx_host.h, first 16 hex digits), and the line names the summary it comes from.
 RECORDED_TRAFFIC = {
     # workload: (bytes per launch, summary under profiles/, kernel source the counters were read on)
     'c5': (94.411e9 + 94.364e9, 'profiles/adam_step_kernel_c5_llama7b.md', '56311dfbb75f1dd5'),
     'c4': (18.4445e9 + 18.4305e9, 'profiles/all_kernels_c4_opt1b3_c2_gpt2_c1.md', '56311dfbb75f1dd5'),
 }
-KERNEL_SOURCE = os.path.join(ROOT, 'elixir_amd', 'csrc', 'elx_kernels.hip')
+DEVICE_SOURCES = [os.path.join(ROOT, 'elixir_amd', 'csrc', name) for name in ('elx_kernels.hip', 'elx_host.h')]
 
 
 def kernel_source_sha16() -> str:
+    """Digest of the files the device code is made from (the kernels and the header with the constants that
+    shape them); the recorded counter figures name the digest they were read on."""
     import hashlib
-    with open(KERNEL_SOURCE, 'rb') as f:
-        return hashlib.sha256(f.read()).hexdigest()[:16]
+    h = hashlib.sha256()
+    for path in DEVICE_SOURCES:
+        with open(path, 'rb') as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def traffic_fields(workload: str):
@@ -57,7 +62,10 @@ def traffic_fields(workload: str):
     now = kernel_source_sha16()
     if sha != now:
         return None, {'summary': summary, 'note': f'counters were read on kernel source {sha}, this build is {now}: stale'}
+    from elixir_amd import _abi
     return nbytes, {'summary': summary, 'kernel_source_sha16': sha,
+                    # _abi.load() has refused a library that was not built from the sources beside it
+                    'library_built_from': (_abi.load().elx_source_sha() or b'').decode(),
                     'method': 'rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy of known size'}
 
 
