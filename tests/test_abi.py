@@ -29,6 +29,32 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert lib.elx_version() == _abi.ELX_ABI_VERSION
 
 
+def test_library_carries_the_digest_of_its_sources_and_a_stale_one_is_refused(monkeypatch, tmp_path):
+    """An edited kernel must never be measured through an old binary: the build compiles the digest of the
+    sources in, the binding compares it with the sources beside it when it loads the library, and the
+    test / benchmark entry (``ensure_built``) rebuilds a library that does not match."""
+    from elixir_amd import build as B
+    lib = _abi.load()
+    now = _abi.source_sha16()
+    assert len(now) == 16 and lib.elx_source_sha().decode() == now == _abi.built_source_sha(_abi.LIB_PATH)
+    assert not B.is_stale()
+    assert [os.path.basename(f) for f in _abi.source_files()] == ['elx_host.cpp', 'elx_host.h', 'elx_kernels.hip', 'elx_abi.h']
+    # the same library next to sources that have changed since
+    monkeypatch.setattr(_abi, '_lib', None)
+    monkeypatch.setattr(_abi, 'source_sha16', lambda: '0123456789abcdef')
+    with pytest.raises(RuntimeError, match='built from other sources'):
+        _abi.load()
+    monkeypatch.setattr(B, 'source_sha16', lambda: '0123456789abcdef')
+    assert B.is_stale()
+    built = []
+    monkeypatch.setattr(B, 'build', lambda verbose=False: built.append(1))
+    B.ensure_built()
+    assert built == [1]
+    monkeypatch.undo()
+    assert _abi.load().elx_version() == _abi.ELX_ABI_VERSION
+    assert _abi.built_source_sha(str(tmp_path / 'missing.so')) == ''
+
+
 def test_record_layouts_match_the_header():
     lib = _abi.load()
     assert lib.elx_sizeof_chunk() == _abi.CHUNK_DTYPE.itemsize == 72
@@ -47,7 +73,7 @@ def test_record_layouts_match_the_header():
 def test_strerror_covers_every_code():
     lib = _abi.load()
     seen = set()
-    for code in range(0, -8, -1):
+    for code in range(0, -9, -1):
         text = lib.elx_strerror(code).decode()
         assert text and text not in seen
         seen.add(text)
