@@ -202,3 +202,65 @@ def test_more_groups_than_the_control_block_holds(oracle):
     for a, b in zip(*states):
         for x, y in zip(a, b):
             assert torch.equal(x.view(torch.int16) if x.dtype == dtype else x, y.view(torch.int16) if y.dtype == dtype else y)
+
+
+@pytest.mark.parametrize('n_groups', [1, 2])
+def test_standalone_steps_over_unchanged_buffers_take_the_steady_path(oracle, monkeypatch, n_groups):
+    """A standalone HybridAdam whose parameters and gradient buffers stay where they are (the gradients
+    are rewritten in place) repeats the launch of the step before with new hyper records only.  Twelve
+    steps with a learning rate that changes every step and a divisor that changes too: every step after
+    the first goes that way, and master / exp_avg / exp_avg_sq have the oracle's bits after each.  A step
+    count edited behind the optimizer's back, a gradient that moves and a loaded state each send one step
+    through the full preparation again -- with the right result."""
+    import elixir_amd.hybrid_adam as H
+    sizes = [50_001, 4_097][:n_groups]
+    torch.manual_seed(3)
+    params = [torch.nn.Parameter((torch.randn(n) * 0.02).to(DEV)) for n in sizes]
+    host = [(to_np(p.data).copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)) for p, n in zip(params, sizes)]
+    steps = [0] * n_groups
+    wds = [0.1, 0.0][:n_groups]
+    opt = ea.HybridAdam([dict(params=[p], lr=1e-3 * (k + 1), weight_decay=wd) for k, (p, wd) in enumerate(zip(params, wds))])
+    for p in params:
+        p.grad = torch.zeros_like(p)
+    taken = []
+    real = H.HybridAdam._launch_steady
+    monkeypatch.setattr(H.HybridAdam, '_launch_steady', lambda self, *a, **k: (taken.append(1), real(self, *a, **k))[1])
+    gen = torch.Generator().manual_seed(4)
+
+    def one_step(expect_steady):
+        for k, group in enumerate(opt.param_groups):
+            group['lr'] = 1e-3 * (k + 1) * (0.9**sum(steps))
+        div = [-1.0, 4.0, 3.0][sum(steps) % 3]
+        grads = [torch.randn(n, generator=gen) * 1e-2 * max(div, 1.0) for n in sizes]
+        for p, g in zip(params, grads):
+            p.grad.copy_(g.to(DEV))                      # the same buffer, new values
+        before = len(taken)
+        opt.step(div_scale=div)
+        assert (len(taken) - before == 1) == expect_steady, (steps, expect_steady)
+        for k, (p, g, (pn, mn, vn)) in enumerate(zip(params, grads, host)):
+            steps[k] += 1
+            oracle.adam(to_np(g), O.F32, pn, mn, vn, lr=opt.param_groups[k]['lr'], beta1=0.9, beta2=0.999, eps=1e-8,
+                        weight_decay=wds[k], step=steps[k], adamw_mode=True, div_scale=div)
+            st = opt.state[p]
+            assert st['step'] == steps[k]
+            for name, got, want in (('p', p.data, pn), ('m', st['exp_avg'], mn), ('v', st['exp_avg_sq'], vn)):
+                assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32)), (steps, name)
+
+    one_step(False)
+    for _ in range(11):
+        one_step(True)
+    # a step count changed behind the optimizer's back: the records must follow it
+    opt.state[params[0]]['step'] = 40
+    steps[0] = 40
+    one_step(False)
+    if n_groups == 1:
+        one_step(True)
+    else:
+        one_step(False)    # two step counts now: every step is prepared in full (the records are matched to parameters)
+    # a gradient that moved
+    params[0].grad = torch.zeros_like(params[0])
+    one_step(False)
+    # a loaded state
+    opt.load_state_dict(opt.state_dict())
+    one_step(False)
+    one_step(n_groups == 1)
