@@ -86,9 +86,8 @@ def hyper_record_address(key: Tuple, adamw_mode: bool) -> int:
     together with this table)."""
     ptr = _HYPER_ADDRESSES.get((key, adamw_mode))
     if ptr is None:
-        if (key, adamw_mode) not in _HYPER_RECORDS or len(_HYPER_ADDRESSES) > 4096:
-            _HYPER_ADDRESSES.clear()
-        ptr = _HYPER_ADDRESSES[(key, adamw_mode)] = hyper_record_cached(key, adamw_mode).ctypes.data
+        rec = hyper_record_cached(key, adamw_mode)    # may empty both tables first
+        ptr = _HYPER_ADDRESSES[(key, adamw_mode)] = rec.ctypes.data
     return ptr
 
 

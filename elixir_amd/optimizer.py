@@ -44,7 +44,7 @@ from . import _abi
 from .chunk import (Chunk, DeviceTable, StatsArena, dtype_code, keep_grads_cached, kernel_device, launch_grad_stats,
                     read_grad_stats, resolve_pending_stats, stats_launch_blocks)
 from .grad_scaler import BaseGradScaler, ConstantGradScaler, DynamicGradScaler
-from .hybrid_adam import CPUAdam, FusedAdam, HybridAdam, _global_step_hooks
+from .hybrid_adam import CPUAdam, FusedAdam, HybridAdam
 
 _AVAIL_OPTIM_LIST = {FusedAdam, CPUAdam, HybridAdam}
 
@@ -657,7 +657,7 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 _abi.finish_decide(partials, n, bpc, eng.d_stats, eng.ctl.data_ptr(), eng.d_hypers, eng.max_hypers,
                                    eng.d_decision, eng.report.data_ptr(), eng.d_counter, stream)
             with self._timed('update'):
-                inner.launch_step(gated=True, defer_commit=True)
+                inner.step(gated=True, defer_commit=True)    # through step(): the inner optimizer's hooks fire
 
         timing = self.kernel_events is not None or inner.kernel_events is not None
         key = (id(prep.dplan), kind, partials, bpc, inner.blocks_per_cu, stats_args[0] if stats_args else 0)
@@ -707,18 +707,20 @@ class ElixirOptimizer(torch.optim.Optimizer):
 
     def step(self, *args, **kwargs):
         """optimizer.py:185-220.  Step hooks registered on this object (``register_step_pre_hook`` /
-        ``register_step_post_hook``) and torch's process-wide ones run around it, in torch's order."""
-        global_pre, global_post = _global_step_hooks()
-        if not (global_pre or global_post or self._optimizer_step_pre_hooks or self._optimizer_step_post_hooks):
+        ``register_step_post_hook``) run around it.  torch's process-wide step hooks are not run here: as with
+        the reference's wrapper they fire in the inner optimizer's own ``step``, once per step, with the inner
+        optimizer as their argument (a step decided on the device has issued that call before it knows
+        whether the step is skipped, so they also fire on a skipped step)."""
+        if not (self._optimizer_step_pre_hooks or self._optimizer_step_post_hooks):
             return self._step(*args, **kwargs)
-        for hook in list(global_pre.values()) + list(self._optimizer_step_pre_hooks.values()):
+        for hook in list(self._optimizer_step_pre_hooks.values()):
             result = hook(self, args, kwargs)
             if result is not None:
                 if not (isinstance(result, tuple) and len(result) == 2):
                     raise RuntimeError(f'{hook} must return None or a tuple of (new_args, new_kwargs), but got {result}.')
                 args, kwargs = result
         out = self._step(*args, **kwargs)
-        for hook in list(self._optimizer_step_post_hooks.values()) + list(global_post.values()):
+        for hook in list(self._optimizer_step_post_hooks.values()):
             hook(self, args, kwargs)
         return out
 

@@ -626,27 +626,32 @@ def test_hybrid_adam_dispatches_step_hooks_itself():
     assert seen == [('pre', (None, 4.0), dict(gated=False, defer_commit=False))]
 
 
-def test_wrapper_runs_step_hooks_in_torchs_order_and_refuses_to_be_copied(monkeypatch):
-    """Hooks registered on the wrapper -- which is an Optimizer that never ran Optimizer.__init__ -- and
-    torch's process-wide hooks fire around its step in torch's order: global pre, own pre, the step, own
-    post, global post; a pre-hook may replace the arguments.  State-dict hooks go to the inner optimizer,
-    whose state it is.  Copying or pickling the wrapper is refused with the reason."""
+def test_wrapper_runs_its_step_hooks_and_refuses_to_be_copied(monkeypatch):
+    """Hooks registered on the wrapper -- which is an Optimizer that never ran Optimizer.__init__ -- fire
+    around its step, a pre-hook may replace the arguments; torch's process-wide hooks are left to the inner
+    optimizer's own step (where the reference's wrapper has them fire too).  State-dict hooks go to the
+    inner optimizer, whose state it is.  Copying or pickling the wrapper is refused with the reason."""
     import copy
     import pickle
     from torch.optim.optimizer import register_optimizer_step_post_hook, register_optimizer_step_pre_hook
     module, opt = _cpu_optimizer(5)
     seen = []
     monkeypatch.setattr(opt, '_step', lambda *a, **k: seen.append(('step', a, k)) or 'ret')
-    handles = [register_optimizer_step_pre_hook(lambda o, a, k: seen.append('global pre') if o is opt else None),
-               register_optimizer_step_post_hook(lambda o, a, k: seen.append('global post') if o is opt else None),
+    handles = [register_optimizer_step_pre_hook(lambda o, a, k: seen.append(('global pre', type(o).__name__))),
+               register_optimizer_step_post_hook(lambda o, a, k: seen.append(('global post', type(o).__name__))),
                opt.register_step_pre_hook(lambda o, a, k: (seen.append('own pre'), ((), dict(marker=1)))[1]),
                opt.register_step_post_hook(lambda o, a, k: seen.append(('own post', k)))]
     try:
         assert opt.step() == 'ret'
+        assert seen == ['own pre', ('step', (), dict(marker=1)), ('own post', dict(marker=1))]
+        # the process-wide ones fire in the inner optimizer's step, with the inner optimizer
+        seen.clear()
+        monkeypatch.setattr(opt.optim, 'launch_step', lambda *a, **k: seen.append('inner launch'))
+        opt.optim.step(gated=True, defer_commit=True)
+        assert seen == [('global pre', 'HybridAdam'), 'inner launch', ('global post', 'HybridAdam')]
     finally:
         for h in handles:
             h.remove()
-    assert seen == ['global pre', 'own pre', ('step', (), dict(marker=1)), ('own post', dict(marker=1)), 'global post']
     seen.clear()
     opt.step()                                   # no hook left: straight through
     assert seen == [('step', (), {})]
