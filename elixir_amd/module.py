@@ -327,11 +327,21 @@ class ElixirModule(nn.Module):
             ready.clear()
 
     def backward(self, loss: torch.Tensor):
+        """module.py:249-254: backward, during which every chunk lands as soon as its gradients are complete."""
+        self._backward(loss.backward)
+
+    def backward_by_grad(self, tensor: torch.Tensor, grad: torch.Tensor):
+        """Backward from an intermediate tensor and the gradient that arrived for it (what
+        ``ElixirOptimizer.backward_by_grad`` calls, optimizer.py:230-236: every stage of a pipeline but the
+        last); the chunks land as in ``backward``."""
+        self._backward(lambda: torch.autograd.backward(tensor, grad))
+
+    def _backward(self, run) -> None:
         self._landed.clear()
         self._ready.clear()
         self._landing_in_backward = True
         try:
-            loss.backward()
+            run()
         finally:
             self._landing_in_backward = False
         self.land_gradients(skip=self._landed)

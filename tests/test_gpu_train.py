@@ -482,6 +482,36 @@ def test_hook_driven_backward_takes_the_device_decided_step(oracle, monkeypatch)
     assert set(st['step'] for st in opt.state.values()) == {2}
 
 
+def test_backward_by_grad_lands_like_backward():
+    """optimizer.py:230-236: a pipeline stage that is not the last receives the (already scaled) gradient
+    of its output and runs backward from there.  The same gradients reach the shards as through
+    ``backward`` on a loss built from that output, the gradients count as scaled, and the step that follows
+    has the same bits."""
+    torch.manual_seed(21)
+    model = Net().to(DEV)
+    twin = copy.deepcopy(model)
+    module, opt = wrap(model, torch.float16, initial_scale=128.0, hysteresis=1)
+    module2, opt2 = wrap(twin, torch.float16, initial_scale=128.0, hysteresis=1)
+    gen = torch.Generator(device=DEV).manual_seed(22)
+    x = batch(gen)
+    upstream = torch.tensor(3.0, device=DEV)    # d(total loss) / d(this stage's output), loss scale not included
+    opt.zero_grad()
+    out = module(x)
+    opt.backward_by_grad(out, upstream * opt.loss_scale)
+    opt2.zero_grad()
+    opt2.backward(module2(x) * upstream)
+    assert opt.optim_state == opt2.optim_state == ea.OptimState.SCALED
+    for a, b in zip(module.param_chunks, module2.param_chunks):
+        assert a._stats_pending and torch.equal(a.shard.view(torch.int16), b.shard.view(torch.int16))
+    assert all(p.grad is None for p in model.parameters())
+    opt.step()
+    opt2.step()
+    assert opt.last_step_info['found_inf'] is False and opt.last_step_info == opt2.last_step_info
+    for a, b in zip(module.param_chunks, module2.param_chunks):
+        assert torch.equal(a.paired_chunk.shard, b.paired_chunk.shard)
+        assert torch.equal(a.shard.view(torch.int16), b.shard.view(torch.int16))
+
+
 def test_tables_prepared_at_backward_follow_late_hyperparameter_changes():
     """``backward`` prepares the tables of the coming step ahead of time; a learning rate changed
     between backward and step must still be the one the step uses."""
