@@ -46,7 +46,7 @@ EXPORTS = ('elx_version', 'elx_strerror', 'elx_tile_elems', 'elx_sizeof_chunk', 
            'elx_grad_stats', 'elx_land_grads_mt', 'elx_check_land_rows', 'elx_land_max_blocks', 'elx_land_tile_elems',
            'elx_land_fold_blocks', 'elx_grad_stats_mt_static', 'elx_static_partials', 'elx_grad_partials_mt',
            'elx_finish_decide', 'elx_sizeof_step_ctl', 'elx_sizeof_step_report', 'elx_max_ctl_hypers', 'elx_put_hypers',
-           'elx_adam_step_put_mt', 'elx_source_sha', 'elx_unscale_mode', 'elx_occupancy_lds_bytes')
+           'elx_adam_step_put_mt', 'elx_source_sha', 'elx_unscale_mode', 'elx_occupancy_lds_bytes', 'elx_finish_decide_rows')
 
 # what the validators' own build (the host-only source under sanitizers) exports
 HOST_EXPORTS = ('elx_check_tables', 'elx_check_land_rows', 'elx_tile_elems', 'elx_land_tile_elems', 'elx_land_max_blocks',
@@ -124,6 +124,8 @@ def load() -> ctypes.CDLL:
     L.elx_grad_partials_mt.argtypes = [vp, u32, cint, u32, vp, cint, vp]
     L.elx_finish_decide.restype = cint
     L.elx_finish_decide.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp]
+    L.elx_finish_decide_rows.restype = cint
+    L.elx_finish_decide_rows.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp, vp, u32, vp]
     L.elx_adam_step_put_mt.restype = cint
     L.elx_adam_step_put_mt.argtypes = [vp, u32, vp, u32, vp, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_put_hypers.restype = cint
@@ -311,8 +313,17 @@ def grad_partials_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_c
 
 
 def finish_decide(d_partials: int, n_chunks: int, blocks_per_chunk: int, d_stats: int, ctl: int, d_hypers: int,
-                  max_hypers: int, d_decision: int, report: int, d_counter: int, stream: int) -> None:
-    """Fold of the partials + the decisions of the step, everything that changes read from ``ctl``."""
+                  max_hypers: int, d_decision: int, report: int, d_counter: int, stream: int, d_rows: int = 0,
+                  d_gated_rows: int = 0, n_rows: int = 0) -> None:
+    """Fold of the partials + the decisions of the step, everything that changes read from ``ctl``.  With
+    ``d_gated_rows`` (a second device copy of the ``n_rows`` update rows at ``d_rows``, the table of the gated
+    update launch that follows) the launch also rewrites that table's n_valid column: the counts of ``d_rows``
+    when the step happens, zeros when it is skipped."""
+    if d_gated_rows:
+        check('elx_finish_decide_rows',
+              load().elx_finish_decide_rows(d_partials, n_chunks, blocks_per_chunk, d_stats, ctl, d_hypers, max_hypers,
+                                            d_decision, report or None, d_counter, d_rows, d_gated_rows, n_rows, stream))
+        return
     check('elx_finish_decide',
           load().elx_finish_decide(d_partials, n_chunks, blocks_per_chunk, d_stats, ctl, d_hypers, max_hypers, d_decision,
                                    report or None, d_counter, stream))

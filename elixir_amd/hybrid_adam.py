@@ -173,12 +173,23 @@ class _DevicePlan:
     def __init__(self, plan: LaunchPlan, device: torch.device):
         self.plan = plan
         self.rows = DeviceTable(plan.rows, device) if len(plan.rows) else None
+        self._gated_rows: Optional[DeviceTable] = None
         self.segs = DeviceTable(plan.segs, device) if len(plan.segs) else None
         self.refresh = DeviceTable(plan.refresh_rows, device) if plan.refresh_rows is not None else None
         self.refresh_aligned = True
         if plan.refresh_rows is not None:
             self.refresh_aligned = bool(
                 np.all(plan.refresh_rows['lowp_out'] % 16 == 0) and np.all(plan.refresh_rows['master'] % 16 == 0))
+
+
+    @property
+    def gated_rows(self) -> Optional[DeviceTable]:
+        """A second device copy of the update rows, made when a step is first decided on the device: the table
+        of the gated update launch, whose n_valid column the decision launch rewrites at every step (zeros on a
+        skip).  ``rows`` itself is never written: host-decided launches read it."""
+        if self._gated_rows is None and self.rows is not None:
+            self._gated_rows = DeviceTable(self.plan.rows, self.rows.dev.device)
+        return self._gated_rows
 
 
 class ChunkBinding:
@@ -369,10 +380,12 @@ class HybridAdam(torch.optim.Optimizer):
         records = [hyper_record_cached(key, self.adamw_mode) for key in hypers.keys()]
         return records[0] if len(records) == 1 else np.concatenate(records)
 
-    def step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
+    def step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False,
+             armed_rows: bool = False):
         """``gated``: the unscale parameters and the skip flag are read on the device from the gate
         words of the prepared hyper table, where ``elx_finish_decide`` has put them (``div_scale`` is then
-        ignored).  ``defer_commit``: launch only; the caller finishes with ``commit_step()`` once it
+        ignored).  ``armed_rows`` (with ``gated``): the launch reads the second copy of the update rows, whose
+        counts of valid elements the decision launch has just rewritten (``_DevicePlan.gated_rows``).  ``defer_commit``: launch only; the caller finishes with ``commit_step()`` once it
         knows that the step happened, or ``abort_step()`` when the device decided to skip.
 
         torch wraps every optimizer's ``step`` in a profiler scope and its hook dispatch, tens of
@@ -380,10 +393,12 @@ class HybridAdam(torch.optim.Optimizer):
         mark below) and runs registered step hooks itself, in torch's order."""
         global_pre, global_post = _global_step_hooks()
         if not (global_pre or global_post or self._optimizer_step_pre_hooks or self._optimizer_step_post_hooks):
-            return self.launch_step(closure, div_scale, gated=gated, defer_commit=defer_commit)
+            return self.launch_step(closure, div_scale, gated=gated, defer_commit=defer_commit, armed_rows=armed_rows)
         pre = list(global_pre.values()) + list(self._optimizer_step_pre_hooks.values())
         post = list(self._optimizer_step_post_hooks.values()) + list(global_post.values())
         args, kwargs = (closure, div_scale), dict(gated=gated, defer_commit=defer_commit)
+        if armed_rows:
+            kwargs['armed_rows'] = True
         for hook in pre:
             result = hook(self, args, kwargs)
             if result is not None:
@@ -397,7 +412,8 @@ class HybridAdam(torch.optim.Optimizer):
 
     step.hooked = True    # torch.optim.Optimizer leaves a step marked like this unwrapped
 
-    def launch_step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False):
+    def launch_step(self, closure=None, div_scale: float = -1, *, gated: bool = False, defer_commit: bool = False,
+                    armed_rows: bool = False):
         """The launches of one step (``step`` without the hook dispatch).  Nothing here builds an autograd
         graph, so no ``no_grad`` scope is entered either."""
         loss = None
@@ -433,7 +449,8 @@ class HybridAdam(torch.optim.Optimizer):
                     events['adam_step'] = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
                 events['adam_step'][0].record()
             if gated:
-                _abi.adam_step_gated_mt(prep.dplan.rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs),
+                rows = prep.dplan.gated_rows if armed_rows else prep.dplan.rows
+                _abi.adam_step_gated_mt(rows.ptr, len(plan.rows), prep.dplan.segs.ptr, len(plan.segs),
                                         prep.d_hypers, len(prep.hyper_host), plan.info, prep.grad_code,
                                         prep.lowp_code, self.blocks_per_cu, stream)
             elif together:

@@ -654,10 +654,15 @@ class ElixirOptimizer(torch.optim.Optimizer):
             with self._timed('stats' if stats_args is not None else 'decide'):
                 if stats_args is not None and not early:
                     _abi.grad_partials_mt(*stats_args, stream, keep_cached=cached)
+                # the decision launch also arms the row table of the update launch: no valid element in any row
+                # when the step is skipped (the update then only refreshes), every row's own count otherwise
                 _abi.finish_decide(partials, n, bpc, eng.d_stats, eng.ctl.data_ptr(), eng.d_hypers, eng.max_hypers,
-                                   eng.d_decision, eng.report.data_ptr(), eng.d_counter, stream)
+                                   eng.d_decision, eng.report.data_ptr(), eng.d_counter, stream,
+                                   d_rows=prep.dplan.rows.ptr, d_gated_rows=prep.dplan.gated_rows.ptr,
+                                   n_rows=len(prep.dplan.plan.rows))
             with self._timed('update'):
-                inner.step(gated=True, defer_commit=True)    # through step(): the inner optimizer's hooks fire
+                # through step(): the inner optimizer's hooks fire
+                inner.step(gated=True, defer_commit=True, armed_rows=True)
 
         timing = self.kernel_events is not None or inner.kernel_events is not None
         key = (id(prep.dplan), kind, partials, bpc, inner.blocks_per_cu, stats_args[0] if stats_args else 0)

@@ -264,3 +264,110 @@ def test_standalone_steps_over_unchanged_buffers_take_the_steady_path(oracle, mo
     opt.load_state_dict(opt.state_dict())
     one_step(False)
     one_step(n_groups == 1)
+
+
+def test_decision_launch_arms_and_disarms_the_row_table_of_the_update():
+    """elx_finish_decide_rows rewrites the n_valid column of the gated update launch's row table at every
+    call: zeros when the step is skipped (an overflow, or an unusable control block), the counts of the
+    untouched source table otherwise -- so a table armed for a skip is disarmed by the next decision, whatever
+    the host did in between.  Nothing else in the table changes, the source table never does, and the decision
+    and report are those of elx_finish_decide.  Then the whole path: a skipped gated update over the armed
+    table only refreshes, the step after it updates -- both equal to the same launches over an unarmed table."""
+    stream = torch.cuda.current_stream().cuda_stream
+    dev = torch.device(DEV, 0)
+    tile = _abi.tile_elems()
+    n_rows = 700                                       # more rows than the deciding workgroup has threads
+    rng = np.random.default_rng(5)
+    rows = np.zeros(n_rows, dtype=_abi.CHUNK_DTYPE)
+    rows['n_alloc'] = rng.integers(1, 50_000, n_rows)
+    rows['n_valid'] = (rows['n_alloc'] * rng.random(n_rows)).astype(np.uint64)
+    for name in ('grad', 'lowp_out', 'master', 'm', 'v'):
+        rows[name] = rng.integers(1, 1 << 40, n_rows) * 16
+    rows['tile_begin'] = np.concatenate(([0], np.cumsum(-(-rows['n_alloc'] // tile))[:-1]))
+    src, gated = DeviceTable(rows, dev), DeviceTable(rows, dev)
+    H = _abi.max_ctl_hypers()
+    ctl_head, rep_head = _abi.STEP_CTL_DTYPE.itemsize, _abi.STEP_REPORT_DTYPE.itemsize
+    ctl = torch.zeros(ctl_head + H * HSZ, dtype=torch.uint8, pin_memory=True)
+    head = ctl.numpy()[:ctl_head].view(_abi.STEP_CTL_DTYPE)
+    report = torch.zeros(rep_head + 2 * REC, dtype=torch.uint8, pin_memory=True)
+    stats = torch.zeros(2 * REC, dtype=torch.uint8, device=DEV)
+    hyp = torch.zeros(H * HSZ, dtype=torch.uint8, device=DEV)
+    dec = torch.zeros(32, dtype=torch.uint8, device=DEV)
+    counter = torch.zeros(4, dtype=torch.int32, device=DEV)
+
+    def decide(overflow, loss_scale=8.0):
+        recs = np.zeros(2, dtype=_abi.STATS_DTYPE)
+        recs['sumsq'] = [4.0, 9.0]
+        recs['overflow'][1] = 1 if overflow else 0
+        d_recs = torch.from_numpy(recs.view(np.uint8).copy()).to(DEV)
+        head[0] = (loss_scale, 1.0, 0, 0, int(head['seq'][0]) + 1)
+        _abi.finish_decide(d_recs.data_ptr(), 2, 1, stats.data_ptr(), ctl.data_ptr(), hyp.data_ptr(), H, dec.data_ptr(),
+                           report.data_ptr(), counter.data_ptr(), stream, d_rows=src.ptr, d_gated_rows=gated.ptr,
+                           n_rows=n_rows)
+        torch.cuda.synchronize()
+        got = gated.dev.cpu().numpy().view(_abi.CHUNK_DTYPE)
+        assert src.dev.cpu().numpy().tobytes() == rows.tobytes()           # the source table is never written
+        for name in rows.dtype.names:
+            if name != 'n_valid':
+                assert np.array_equal(got[name], rows[name]), name
+        rh = report.numpy()[:rep_head].view(_abi.STEP_REPORT_DTYPE)[0]
+        assert rh['seq'] == head['seq'][0]
+        return got['n_valid'].copy(), int(rh['skip']), int(rh['status'])
+
+    valid, skip, status = decide(False)
+    assert np.array_equal(valid, rows['n_valid']) and (skip, status) == (0, 0)
+    valid, skip, status = decide(True)
+    assert not valid.any() and (skip, status) == (1, 0)
+    valid, skip, status = decide(True)                                     # armed twice in a row
+    assert not valid.any() and skip == 1
+    valid, skip, status = decide(False)                                    # disarmed by the next decision
+    assert np.array_equal(valid, rows['n_valid']) and skip == 0
+    valid, skip, status = decide(False, loss_scale=0.0)                    # an unusable control block: nothing may update
+    assert not valid.any() and (skip, status) == (1, _abi.ELX_E_RANGE)
+    valid, skip, status = decide(False)
+    assert np.array_equal(valid, rows['n_valid']) and (skip, status) == (0, 0)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_skipped_step_over_the_armed_table_refreshes_everything_and_updates_nothing(oracle, dtype):
+    """The wrapper's device-decided step with an overflow: master, exp_avg, exp_avg_sq and the step counts stay
+    as they were, every element of every low-precision shard -- owned by a tensor or not, padding included,
+    whatever sat there -- becomes the cast of its master value, and the clean step behind it updates as the
+    oracle does."""
+    module, opt, ochunks = build_workload([('a', (70_001, )), ('b', (33, 1000)), ('c', (5, )), ('d', (100_000, ))], 1 << 17,
+                                          dtype, seed=51, grad_std=2e-2, loss_scale=256.0 if dtype == torch.float16 else 1.0,
+                                          weight_decay=0.1, max_norm=1.0, initial_scale=256.0, hysteresis=1)
+    if dtype == torch.float16:
+        scaler = O.DynamicGradScalerOracle(initial_scale=256.0, min_scale=1, max_scale=2**24, hysteresis=1)
+    else:    # bfloat16 trains with a constant scale of 1; the overflow check still runs
+        scaler = O.ConstantGradScalerOracle(1.0)
+    assert opt.gated_step and len(module.param_chunks) >= 2
+    before = [(pc.paired_chunk.shard.clone(), *[t.clone() for t in opt._binding.moments(pc.paired_chunk)])
+              for pc in module.param_chunks]
+    for pc in module.param_chunks:
+        pc.shard[pc.n_valid:] = 7.0                      # garbage in the padding
+        pc.invalidate_stats()
+    module.param_chunks[0].shard[11] = float('inf')
+    refresh_oracle_grads(module, ochunks)
+    opt.mark_gradients_scaled()
+    opt.step()
+    info = O.reference_step(ochunks, CODE[dtype], scaler, max_norm=1.0)
+    assert opt.last_step_info['found_inf'] is True and info['found_inf'] is True
+    assert opt.loss_scale == info['loss_scale'] == (128.0 if dtype == torch.float16 else 1.0)
+    for pc, (p0, m0, v0) in zip(module.param_chunks, before):
+        m, v = opt._binding.moments(pc.paired_chunk)
+        assert torch.equal(pc.paired_chunk.shard, p0) and torch.equal(m, m0) and torch.equal(v, v0)
+        assert torch.equal(pc.shard, p0.to(dtype))      # the whole shard, padding included
+    assert set(st['step'] for st in opt.state.values()) == {0}
+    gen = torch.Generator(device=DEV).manual_seed(52)
+    for pc in module.param_chunks:
+        g = torch.randn(pc.shard_size, generator=gen, device=DEV) * (2e-2 * opt.loss_scale)
+        g[pc.utilized_size:] = 0
+        pc.shard.copy_(g.to(dtype))
+        pc.invalidate_stats()
+    refresh_oracle_grads(module, ochunks)
+    opt.mark_gradients_scaled()
+    opt.step()
+    info = O.reference_step(ochunks, CODE[dtype], scaler, max_norm=1.0)
+    assert opt.last_step_info['found_inf'] is False and set(st['step'] for st in opt.state.values()) == {1}
+    compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-8, atol_v=1e-10, tag='after the skip')
