@@ -125,7 +125,7 @@ def load() -> ctypes.CDLL:
     L.elx_finish_decide.restype = cint
     L.elx_finish_decide.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp]
     L.elx_finish_decide_rows.restype = cint
-    L.elx_finish_decide_rows.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp, vp, u32, vp]
+    L.elx_finish_decide_rows.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, vp, vp, vp, vp, u32, vp, vp]
     L.elx_adam_step_put_mt.restype = cint
     L.elx_adam_step_put_mt.argtypes = [vp, u32, vp, u32, vp, vp, u32, u64, u32, flt, cint, cint, u32, u32, vp]
     L.elx_put_hypers.restype = cint
@@ -314,15 +314,16 @@ def grad_partials_mt(d_chunks: int, n_chunks: int, grad_dtype: int, blocks_per_c
 
 def finish_decide(d_partials: int, n_chunks: int, blocks_per_chunk: int, d_stats: int, ctl: int, d_hypers: int,
                   max_hypers: int, d_decision: int, report: int, d_counter: int, stream: int, d_rows: int = 0,
-                  d_gated_rows: int = 0, n_rows: int = 0) -> None:
+                  d_gated_rows: int = 0, n_rows: int = 0, d_armed: int = 0) -> None:
     """Fold of the partials + the decisions of the step, everything that changes read from ``ctl``.  With
     ``d_gated_rows`` (a second device copy of the ``n_rows`` update rows at ``d_rows``, the table of the gated
-    update launch that follows) the launch also rewrites that table's n_valid column: the counts of ``d_rows``
-    when the step happens, zeros when it is skipped."""
+    update launch that follows) the launch also keeps that table's n_valid column: zeros when the step is
+    skipped, the counts of ``d_rows`` again at the first step that happens afterwards (``d_armed``: one
+    uint32 of device memory that says which of the two the table holds; 0 for a fresh copy)."""
     if d_gated_rows:
         check('elx_finish_decide_rows',
               load().elx_finish_decide_rows(d_partials, n_chunks, blocks_per_chunk, d_stats, ctl, d_hypers, max_hypers,
-                                            d_decision, report or None, d_counter, d_rows, d_gated_rows, n_rows, stream))
+                                            d_decision, report or None, d_counter, d_rows, d_gated_rows, n_rows, d_armed, stream))
         return
     check('elx_finish_decide',
           load().elx_finish_decide(d_partials, n_chunks, blocks_per_chunk, d_stats, ctl, d_hypers, max_hypers, d_decision,

@@ -985,7 +985,8 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
                                                                       uint32_t max_hypers, ElxDecision *out,
                                                                       ElxStepReport *report, uint32_t *counter,
                                                                       const ElxChunk *__restrict__ rows,
-                                                                      ElxChunk *__restrict__ gated_rows, uint32_t n_rows) {
+                                                                      ElxChunk *__restrict__ gated_rows, uint32_t n_rows,
+                                                                      uint32_t *armed) {
     __shared__ uint32_t s_last;
     __shared__ __align__(16) uint32_t s_ctl[kCtlWords];
     __shared__ ElxDecision s_decision;
@@ -1070,13 +1071,19 @@ __global__ __launch_bounds__(kStatsThreads) void finish_decide_kernel(const ElxS
         if (word == kGateWord + 2) value = gate_words[2];
         dst[i] = value;
     }
-    // The row table of the gated update launch, when the caller keeps one for it: every row gets its count of
-    // valid elements back, or none at all when the step is skipped.  A row without valid elements only has its
-    // low-precision copy refreshed, and the update launch learns that from the record it fetches first of all:
-    // a skipped step then moves 6 bytes per element instead of 16, and an ordinary step pays nothing for it
-    // (asking for the skip flag itself at the top of the update kernel cost every step 3.6 %).
+    // The row table of the gated update launch, when the caller keeps one for it: no row has a valid element
+    // when the step is skipped, every row has its own count back afterwards.  A row without valid elements only
+    // has its low-precision copy refreshed, and the update launch learns that from the record it fetches first
+    // of all: a skipped step then moves 6 bytes per element instead of 16, and an ordinary step pays nothing
+    // for it (asking for the skip flag itself at the top of the update kernel cost every step 3.6 %).  *armed
+    // says whether the table holds zeros now, so that the ordinary step after an ordinary step writes nothing.
     if (gated_rows) {
-        for (uint32_t i = threadIdx.x; i < n_rows; i += kStatsThreads) gated_rows[i].n_valid = d.skip ? 0ull : rows[i].n_valid;
+        const uint32_t was_armed = __hip_atomic_load(armed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (d.skip || was_armed) {
+            for (uint32_t i = threadIdx.x; i < n_rows; i += kStatsThreads) gated_rows[i].n_valid = d.skip ? 0ull : rows[i].n_valid;
+            __syncthreads();
+            if (threadIdx.x == 0) __hip_atomic_store(armed, d.skip ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     if (report) {
         const uint32_t *dw = reinterpret_cast<const uint32_t *>(&s_decision);
@@ -1345,21 +1352,21 @@ int elx_grad_partials_mt(const ElxChunk *d_chunks, uint32_t n_chunks, int grad_d
 int elx_finish_decide_rows(const ElxStats *d_partials, uint32_t n_chunks, uint32_t blocks_per_chunk, ElxStats *d_stats,
                            const ElxStepCtl *ctl, ElxHyper *d_hypers, uint32_t max_hypers, ElxDecision *d_decision,
                            ElxStepReport *report, uint32_t *d_counter, const ElxChunk *d_rows, ElxChunk *d_gated_rows,
-                           uint32_t n_rows, void *stream) {
+                           uint32_t n_rows, uint32_t *d_armed, void *stream) {
     if (!d_partials || !d_stats || !ctl || !d_decision || !d_counter || (max_hypers && !d_hypers)) return ELX_E_NULL;
     if (n_chunks == 0 || n_chunks > 65535u || blocks_per_chunk == 0 || blocks_per_chunk > kMaxLandBlocks ||
         max_hypers > kMaxCtlHypers)
         return ELX_E_SIZE;
     if (((uintptr_t)ctl | (uintptr_t)report | (uintptr_t)d_stats | (uintptr_t)d_decision) & 7u) return ELX_E_ALIGN;
     if (d_gated_rows) {
-        if (!d_rows) return ELX_E_NULL;
+        if (!d_rows || !d_armed) return ELX_E_NULL;
         if (n_rows == 0 || n_rows > 65535u) return ELX_E_SIZE;
         if (d_rows == d_gated_rows) return ELX_E_RANGE;    // the counts are taken from a table nobody writes
-        if (((uintptr_t)d_rows | (uintptr_t)d_gated_rows) & 7u) return ELX_E_ALIGN;
+        if ((((uintptr_t)d_rows | (uintptr_t)d_gated_rows) & 7u) || ((uintptr_t)d_armed & 3u)) return ELX_E_ALIGN;
     }
     hipLaunchKernelGGL(finish_decide_kernel, dim3(n_chunks), dim3(kStatsThreads), 0, (hipStream_t)stream, d_partials,
                        blocks_per_chunk, d_stats, n_chunks, ctl, d_hypers, max_hypers, d_decision, report, d_counter, d_rows,
-                       d_gated_rows, d_gated_rows ? n_rows : 0u);
+                       d_gated_rows, d_gated_rows ? n_rows : 0u, d_armed);
     return (int)hipGetLastError();
 }
 
@@ -1367,7 +1374,7 @@ int elx_finish_decide(const ElxStats *d_partials, uint32_t n_chunks, uint32_t bl
                       const ElxStepCtl *ctl, ElxHyper *d_hypers, uint32_t max_hypers, ElxDecision *d_decision,
                       ElxStepReport *report, uint32_t *d_counter, void *stream) {
     return elx_finish_decide_rows(d_partials, n_chunks, blocks_per_chunk, d_stats, ctl, d_hypers, max_hypers, d_decision,
-                                  report, d_counter, nullptr, nullptr, 0, stream);
+                                  report, d_counter, nullptr, nullptr, 0, nullptr, stream);
 }
 
 int elx_put_hypers(const ElxHyper *h_hypers, uint32_t n_hypers, ElxHyper *d_hypers, void *stream) {

@@ -174,6 +174,7 @@ class _DevicePlan:
         self.plan = plan
         self.rows = DeviceTable(plan.rows, device) if len(plan.rows) else None
         self._gated_rows: Optional[DeviceTable] = None
+        self.armed: Optional[torch.Tensor] = None    # one device word: whether the gated copy holds zeros right now
         self.segs = DeviceTable(plan.segs, device) if len(plan.segs) else None
         self.refresh = DeviceTable(plan.refresh_rows, device) if plan.refresh_rows is not None else None
         self.refresh_aligned = True
@@ -189,6 +190,7 @@ class _DevicePlan:
         skip).  ``rows`` itself is never written: host-decided launches read it."""
         if self._gated_rows is None and self.rows is not None:
             self._gated_rows = DeviceTable(self.plan.rows, self.rows.dev.device)
+            self.armed = torch.zeros(1, dtype=torch.int32, device=self.rows.dev.device)
         return self._gated_rows
 
 

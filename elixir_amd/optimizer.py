@@ -659,7 +659,7 @@ class ElixirOptimizer(torch.optim.Optimizer):
                 _abi.finish_decide(partials, n, bpc, eng.d_stats, eng.ctl.data_ptr(), eng.d_hypers, eng.max_hypers,
                                    eng.d_decision, eng.report.data_ptr(), eng.d_counter, stream,
                                    d_rows=prep.dplan.rows.ptr, d_gated_rows=prep.dplan.gated_rows.ptr,
-                                   n_rows=len(prep.dplan.plan.rows))
+                                   n_rows=len(prep.dplan.plan.rows), d_armed=prep.dplan.armed.data_ptr())
             with self._timed('update'):
                 # through step(): the inner optimizer's hooks fire
                 inner.step(gated=True, defer_commit=True, armed_rows=True)

@@ -267,19 +267,22 @@ uint32_t elx_max_ctl_hypers(void);
 /*
  * elx_finish_decide that also arms the row table of the gated update launch: a skipped step
  * (optimizer.py:196-203) then costs what its refresh costs.  d_gated_rows is a second device copy of the n_rows
- * ElxChunk records at d_rows, and the table handed to elx_adam_step_gated_mt next on the same stream.  The
- * deciding workgroup rewrites its n_valid column on every call: the counts of d_rows (which nobody writes) when
- * the step happens, zeros when it is skipped.  A record without valid elements only has its low-precision copy
- * refreshed, and the update launch knows that from the record it fetches first of all, before it has issued a
- * load: a skipped step moves 4 B + 2 B per element instead of 14 B + 2 B, and an ordinary step pays nothing
- * (reading the skip flag itself at the top of the update kernel cost every step 3.6 %).  Because the column is
- * rewritten by every call, a table left armed for a skip cannot outlive the step it was armed for.
+ * ElxChunk records at d_rows, and the table handed to elx_adam_step_gated_mt next on the same stream.  When the
+ * step is skipped the deciding workgroup zeroes the n_valid column of d_gated_rows; at the first step that
+ * happens after that it writes the counts of d_rows (which nobody writes) back.  A record without valid elements
+ * only has its low-precision copy refreshed, and the update launch knows that from the record it fetches first of
+ * all, before it has issued a load: a skipped step moves 4 B + 2 B per element instead of 14 B + 2 B, and an
+ * ordinary step pays nothing (reading the skip flag itself at the top of the update kernel cost every step
+ * 3.6 %).
+ *   d_armed  one uint32 of device memory that belongs to d_gated_rows: 0 while the table holds the counts of
+ *            d_rows (as a fresh copy does), 1 while it holds zeros; read and kept by the launch, so that an
+ *            ordinary step after an ordinary step writes nothing
  * d_gated_rows NULL: exactly elx_finish_decide.  d_rows == d_gated_rows: ELX_E_RANGE.
  */
 int elx_finish_decide_rows(const ElxStats *d_partials, uint32_t n_chunks, uint32_t blocks_per_chunk, ElxStats *d_stats,
                            const ElxStepCtl *ctl, ElxHyper *d_hypers, uint32_t max_hypers, ElxDecision *d_decision,
                            ElxStepReport *report, uint32_t *d_counter, const ElxChunk *d_rows, ElxChunk *d_gated_rows,
-                           uint32_t n_rows, void *stream);
+                           uint32_t n_rows, uint32_t *d_armed, void *stream);
 
 /*
  * elx_grad_stats_mt without a workspace argument, for callers that cannot allocate one (code under

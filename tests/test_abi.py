@@ -180,12 +180,14 @@ def test_launch_entry_points_reject_bad_arguments_before_launching():
     assert lib.elx_finish_decide(8, 1, 1, 8, 12, 8, 1, 8, None, 8, None) == -3             # control block not 8-byte aligned
     # the variant that arms a row table: both tables or none, distinct, a sane row count
     rows_args = (8, 1, 1, 8, 8, 8, 1, 8, None, 8)
-    assert lib.elx_finish_decide_rows(*rows_args, None, 16, 4, None) == -1          # a table to arm, none to read the counts from
-    assert lib.elx_finish_decide_rows(*rows_args, 16, 16, 4, None) == -4            # one table for both
-    assert lib.elx_finish_decide_rows(*rows_args, 8, 16, 0, None) == -7
-    assert lib.elx_finish_decide_rows(*rows_args, 8, 16, 70000, None) == -7
-    assert lib.elx_finish_decide_rows(*rows_args, 8, 12, 4, None) == -3
-    assert lib.elx_finish_decide_rows(None, 1, 1, 8, 8, 8, 1, 8, None, 8, 8, 16, 4, None) == -1
+    assert lib.elx_finish_decide_rows(*rows_args, None, 16, 4, 8, None) == -1       # a table to arm, none to read the counts from
+    assert lib.elx_finish_decide_rows(*rows_args, 8, 16, 4, None, None) == -1       # no word that says what the table holds
+    assert lib.elx_finish_decide_rows(*rows_args, 16, 16, 4, 8, None) == -4         # one table for both
+    assert lib.elx_finish_decide_rows(*rows_args, 8, 16, 0, 8, None) == -7
+    assert lib.elx_finish_decide_rows(*rows_args, 8, 16, 70000, 8, None) == -7
+    assert lib.elx_finish_decide_rows(*rows_args, 8, 12, 4, 8, None) == -3
+    assert lib.elx_finish_decide_rows(*rows_args, 8, 16, 4, 6, None) == -3
+    assert lib.elx_finish_decide_rows(None, 1, 1, 8, 8, 8, 1, 8, None, 8, 8, 16, 4, 8, None) == -1
     assert lib.elx_put_hypers(None, 1, 8, None) == -1
     assert lib.elx_put_hypers(8, 0, 8, None) == -7
     assert lib.elx_put_hypers(8, 1, 6, None) == -3

@@ -267,10 +267,10 @@ def test_standalone_steps_over_unchanged_buffers_take_the_steady_path(oracle, mo
 
 
 def test_decision_launch_arms_and_disarms_the_row_table_of_the_update():
-    """elx_finish_decide_rows rewrites the n_valid column of the gated update launch's row table at every
-    call: zeros when the step is skipped (an overflow, or an unusable control block), the counts of the
-    untouched source table otherwise -- so a table armed for a skip is disarmed by the next decision, whatever
-    the host did in between.  Nothing else in the table changes, the source table never does, and the decision
+    """elx_finish_decide_rows keeps the n_valid column of the gated update launch's row table: zeros when the
+    step is skipped (an overflow, or an unusable control block), the counts of the untouched source table again
+    at the first decision that lets a step happen -- so a table armed for a skip is disarmed by the next
+    decision, whatever the host did in between -- and the word that says which of the two it holds.  Nothing else in the table changes, the source table never does, and the decision
     and report are those of elx_finish_decide.  Then the whole path: a skipped gated update over the armed
     table only refreshes, the step after it updates -- both equal to the same launches over an unarmed table."""
     stream = torch.cuda.current_stream().cuda_stream
@@ -294,6 +294,7 @@ def test_decision_launch_arms_and_disarms_the_row_table_of_the_update():
     hyp = torch.zeros(H * HSZ, dtype=torch.uint8, device=DEV)
     dec = torch.zeros(32, dtype=torch.uint8, device=DEV)
     counter = torch.zeros(4, dtype=torch.int32, device=DEV)
+    armed = torch.zeros(1, dtype=torch.int32, device=DEV)
 
     def decide(overflow, loss_scale=8.0):
         recs = np.zeros(2, dtype=_abi.STATS_DTYPE)
@@ -303,8 +304,9 @@ def test_decision_launch_arms_and_disarms_the_row_table_of_the_update():
         head[0] = (loss_scale, 1.0, 0, 0, int(head['seq'][0]) + 1)
         _abi.finish_decide(d_recs.data_ptr(), 2, 1, stats.data_ptr(), ctl.data_ptr(), hyp.data_ptr(), H, dec.data_ptr(),
                            report.data_ptr(), counter.data_ptr(), stream, d_rows=src.ptr, d_gated_rows=gated.ptr,
-                           n_rows=n_rows)
+                           n_rows=n_rows, d_armed=armed.data_ptr())
         torch.cuda.synchronize()
+        assert int(armed[0]) == (1 if overflow or not loss_scale > 0 else 0)
         got = gated.dev.cpu().numpy().view(_abi.CHUNK_DTYPE)
         assert src.dev.cpu().numpy().tobytes() == rows.tobytes()           # the source table is never written
         for name in rows.dtype.names:
