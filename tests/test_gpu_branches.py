@@ -373,3 +373,25 @@ def test_skipped_step_over_the_armed_table_refreshes_everything_and_updates_noth
     info = O.reference_step(ochunks, CODE[dtype], scaler, max_norm=1.0)
     assert opt.last_step_info['found_inf'] is False and set(st['step'] for st in opt.state.values()) == {1}
     compare_state(module, opt, ochunks, dtype, rtol=1e-6, atol_p=1e-9, atol_m=1e-8, atol_v=1e-10, tag='after the skip')
+
+
+@pytest.mark.parametrize('gated', [True, False])
+def test_a_skipped_step_is_logged_where_the_reference_logs_it(oracle, caplog, gated):
+    """optimizer.py:199: 'Found overflow. Skip step' at INFO, once per skipped step, on either way the step is
+    decided; a step that happens logs nothing."""
+    import logging
+    module, opt, ochunks = build_workload([('a', (5000, )), ('b', (300, 7))], 1 << 13, torch.float16, seed=61,
+                                          loss_scale=64.0, initial_scale=64.0, hysteresis=1)
+    opt.gated_step = gated
+    caplog.set_level(logging.INFO, logger='elixir_amd.optimizer')
+    opt.mark_gradients_scaled()
+    opt.step()
+    assert opt.last_step_info['found_inf'] is False and not caplog.records
+    module.param_chunks[0].shard[3] = float('nan')
+    for pc in module.param_chunks:
+        pc.invalidate_stats()
+    opt.mark_gradients_scaled()
+    opt.step()
+    assert opt.last_step_info['found_inf'] is True
+    assert [(r.name, r.levelname, r.getMessage()) for r in caplog.records] == [
+        ('elixir_amd.optimizer', 'INFO', 'Found overflow. Skip step')]
