@@ -198,16 +198,27 @@ def fused_landing_leg(built, steps):
     # the flow of a training loop: backward lands every chunk with a launch of its own as soon as its last
     # gradient exists, the last chunk first; the records still end up side by side (the optimizer gave every
     # chunk its slot in chunk order) and the step is decided on the device
-    from elixir_amd.chunk import land_chunks
-    pc_land_s, pc_step_s = [], []
+    from elixir_amd.chunk import land_chunks, land_tensors
+    grads = {}    # views of the saved buffers stand in for the .grad tensors
+    for pc, g in zip(chunks, built.grads):
+        for t, info in pc.tensors_info.items():
+            grads[t] = g[info.offset:info.end]
+    pc_land_s, pc_step_s, pc_payload_s = [], [], []
     for i in range(steps + 1):
         for pc in chunks:
             pc.invalidate_stats()
 
-        def one_by_one():
+        def payload_by_payload():
             for pc, g in zip(reversed(chunks), reversed(built.grads)):
                 land_chunks([pc], [g])
 
+        def one_by_one():    # what ElixirModule's gradient hook issues: a chunk's own per-tensor gradients, one launch
+            for pc in reversed(chunks):
+                land_tensors([pc], lambda t: grads[t])
+
+        t_pc_payload = behind_blocker(payload_by_payload)
+        for pc in chunks:
+            pc.invalidate_stats()
         t_pc_land = behind_blocker(one_by_one)
         opt.mark_gradients_scaled()
         torch.cuda.synchronize()
@@ -219,18 +230,13 @@ def fused_landing_leg(built, steps):
         assert opt.last_step_info['found_inf'] is False
         if i > 0:
             pc_land_s.append(t_pc_land)
+            pc_payload_s.append(t_pc_payload)
             pc_step_s.append(dt)
     t_pc_step, t_pc_land = float(np.mean(pc_step_s)), float(np.mean(pc_land_s))
 
     # the same landing straight from per-tensor gradients (views of the saved buffers stand in for
     # the .grad tensors), next to what it replaces: a zeroed payload per chunk, one slice copy per
     # tensor, and the copy of the payload into the shard
-    from elixir_amd.chunk import land_tensors
-    grads = {}
-    for pc, g in zip(chunks, built.grads):
-        for t, info in pc.tensors_info.items():
-            grads[t] = g[info.offset:info.end]
-
     def slice_copies():
         for pc in chunks:
             payload = torch.zeros(pc.chunk_size, dtype=pc.chunk_dtype, device=pc.shard_device)
@@ -266,10 +272,11 @@ def fused_landing_leg(built, steps):
         'step_gbps_28B': BYTES_UPDATE * n_valid / t_step / 1e9,
         'step_frac_28B': BYTES_UPDATE * n_valid / t_step / 1e9 / HBM_PEAK_GBPS,
         'per_chunk_landing': {
-            'what': 'every chunk landed by a launch of its own, the last chunk first (what the hooks of backward do); '
-                    'the step that follows is decided on the device all the same',
+            'what': 'every chunk landed by a launch of its own straight from its per-tensor gradients, the last chunk '
+                    'first (what the hooks of backward do); the step that follows is decided on the device all the same',
             'launches': len(chunks),
             'landing_ms_all_chunks': t_pc_land * 1e3,
+            'landing_ms_all_chunks_from_payloads': float(np.mean(pc_payload_s)) * 1e3,
             'ms_per_step': t_pc_step * 1e3,
             'step_frac_28B': BYTES_UPDATE * n_valid / t_pc_step / 1e9 / HBM_PEAK_GBPS,
         },
