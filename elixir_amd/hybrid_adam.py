@@ -510,13 +510,8 @@ class HybridAdam(torch.optim.Optimizer):
         for group, count in zip(groups, steady.layout):
             if len(group['params']) != count:
                 return False
-        for p, p_ptr, g_ptr, g_dtype in steady.watch:
-            g = p.grad
-            if g is None:
-                if g_ptr is not None:
-                    return False
-            elif g_ptr is None or g.data_ptr() != g_ptr or g.dtype != g_dtype or p.data_ptr() != p_ptr:
-                return False
+        if not self._watch_holds(steady.watch):
+            return False
         step = steady.step
         for state in steady.states:
             if state['step'] != step:
@@ -711,23 +706,36 @@ class HybridAdam(torch.optim.Optimizer):
 
     # ---- standalone, on ordinary parameters
 
+    def _watch_holds(self, watch) -> bool:
+        """Whether every buffer a cached walk recorded is still the one in use: parameter, gradient (address and
+        dtype) and, for a parameter that has stepped, its state entry with both moments where they were."""
+        states = self.state
+        for p, p_ptr, g_ptr, g_dtype, state, m_ptr, v_ptr in watch:
+            g = p.grad
+            if g is None:
+                if g_ptr is not None:
+                    return False
+                continue
+            if g_ptr is None or g.data_ptr() != g_ptr or g.dtype != g_dtype or p.data_ptr() != p_ptr:
+                return False
+            if states.get(p) is not state:
+                return False
+            m, v = state.get('exp_avg'), state.get('exp_avg_sq')
+            if m is None or v is None or m.data_ptr() != m_ptr or v.data_ptr() != v_ptr:
+                return False
+        return True
+
     def _standalone_items(self):
         """(items, gradient dtype, device) of the parameters that carry a gradient: per parameter its state
         dict, its group index and (gradient, parameter, exp_avg, exp_avg_sq addresses, element count).  The
-        walk with its checks is repeated only when a parameter, a gradient buffer or the group layout has
-        changed since the last step (every buffer is watched by address and dtype)."""
+        walk with its checks is repeated only when a parameter, a gradient buffer, a state entry or one of its
+        moments, or the group layout has changed since the last step (every buffer is watched by address, the
+        gradient by dtype too)."""
         cache = self._standalone_cache
         if cache is not None:
             watch, layout, result = cache
             if layout == tuple(len(g['params']) for g in self.param_groups):
-                for p, p_ptr, g_ptr, g_dtype in watch:
-                    g = p.grad
-                    if g is None:
-                        if g_ptr is not None:
-                            break
-                    elif g_ptr is None or g.data_ptr() != g_ptr or g.dtype != g_dtype or p.data_ptr() != p_ptr:
-                        break
-                else:
+                if self._watch_holds(watch):
                     return result
         items, watch = [], []
         grad_dtype = None
@@ -735,7 +743,7 @@ class HybridAdam(torch.optim.Optimizer):
         for gi, group in enumerate(self.param_groups):
             for p in group['params']:
                 if p.grad is None or p.numel() == 0:
-                    watch.append((p, p.data_ptr(), None, None))
+                    watch.append((p, p.data_ptr(), None, None, None, 0, 0))
                     continue
                 if p.device.type != 'cuda':
                     raise RuntimeError('HybridAdam runs on the GPU: parameters must live in device memory')
@@ -753,9 +761,9 @@ class HybridAdam(torch.optim.Optimizer):
                     state['step'] = 0
                     state['exp_avg'] = torch.zeros_like(p, memory_format=torch.preserve_format)
                     state['exp_avg_sq'] = torch.zeros_like(p, memory_format=torch.preserve_format)
-                watch.append((p, p.data_ptr(), p.grad.data_ptr(), p.grad.dtype))
-                items.append((state, gi, (p.grad.data_ptr(), p.data.data_ptr(), state['exp_avg'].data_ptr(),
-                                          state['exp_avg_sq'].data_ptr(), p.numel())))
+                m_ptr, v_ptr = state['exp_avg'].data_ptr(), state['exp_avg_sq'].data_ptr()
+                watch.append((p, p.data_ptr(), p.grad.data_ptr(), p.grad.dtype, state, m_ptr, v_ptr))
+                items.append((state, gi, (p.grad.data_ptr(), p.data.data_ptr(), m_ptr, v_ptr, p.numel())))
         result = (items, grad_dtype, device)
         self._standalone_cache = (watch, tuple(len(g['params']) for g in self.param_groups), result)
         return result

@@ -210,8 +210,8 @@ def test_standalone_steps_over_unchanged_buffers_take_the_steady_path(oracle, mo
     are rewritten in place) repeats the launch of the step before with new hyper records only.  Twelve
     steps with a learning rate that changes every step and a divisor that changes too: every step after
     the first goes that way, and master / exp_avg / exp_avg_sq have the oracle's bits after each.  A step
-    count edited behind the optimizer's back, a gradient that moves and a loaded state each send one step
-    through the full preparation again -- with the right result."""
+    count edited behind the optimizer's back, a gradient that moves, a loaded state, a moment that moves and a
+    replaced state entry each send one step through the full preparation again -- with the right result."""
     import elixir_amd.hybrid_adam as H
     sizes = [50_001, 4_097][:n_groups]
     torch.manual_seed(3)
@@ -262,6 +262,18 @@ def test_standalone_steps_over_unchanged_buffers_take_the_steady_path(oracle, mo
     one_step(False)
     # a loaded state
     opt.load_state_dict(opt.state_dict())
+    one_step(False)
+    one_step(n_groups == 1)
+    # a moment that moved (same values in a new tensor): the launch must follow it, as torch's optimizers would
+    old_m = opt.state[params[0]]['exp_avg']
+    opt.state[params[0]]['exp_avg'] = old_m.clone()
+    frozen = old_m.clone()
+    one_step(False)
+    assert torch.equal(old_m, frozen)                  # the buffer left behind is no longer written
+    one_step(n_groups == 1)
+    # a state entry replaced as a whole
+    st = opt.state[params[0]]
+    opt.state[params[0]] = dict(step=st['step'], exp_avg=st['exp_avg'].clone(), exp_avg_sq=st['exp_avg_sq'].clone())
     one_step(False)
     one_step(n_groups == 1)
 
