@@ -106,14 +106,14 @@ int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t 
         const uint64_t t = (r.n_alloc + tile - 1) / tile;
         if (t > max_tiles) max_tiles = t;
     }
-    if (max_tiles > kMaxLandBlocks) return ELX_E_SIZE;
     if (h_slot_offsets) {
         if (n_slots == 0 || n_slots > n_rows) return ELX_E_SIZE;
         if (h_slot_offsets[0] != 0 || h_slot_offsets[n_slots] != n_rows) return ELX_E_RANGE;
         for (uint32_t s = 0; s < n_slots; ++s)
             if (h_slot_offsets[s] > h_slot_offsets[s + 1]) return ELX_E_ORDER;
     }
-    *blocks_per_row = (uint32_t)max_tiles;
+    // a row with more tiles than a launch may have workgroups per row: each workgroup takes several
+    *blocks_per_row = (uint32_t)(max_tiles < kMaxLandBlocks ? max_tiles : kMaxLandBlocks);
     return 0;
 }
 

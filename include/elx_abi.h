@@ -454,7 +454,8 @@ int elx_land_grads_mt(const ElxChunk *d_rows, uint32_t n_rows, const uint32_t *d
  * Host-side validation of HOST copies of a landing table before it is uploaded (the launch itself
  * sees device pointers only): NULL destination, element alignment, n_valid <= n_alloc, slot offsets
  * that start at 0, end at n_rows and never decrease (h_slot_offsets may be NULL: one slot per row).
- * On success *blocks_per_row is the one-tile-per-workgroup grid width, ceil(max n_alloc / tile).
+ * On success *blocks_per_row is the one-tile-per-workgroup grid width, ceil(max n_alloc / tile), or
+ * elx_land_max_blocks() when the longest row has more tiles than that (its workgroups take several).
  */
 int elx_check_land_rows(const ElxChunk *h_rows, uint32_t n_rows, const uint32_t *h_slot_offsets, uint32_t n_slots,
                         int src_dtype, int dst_dtype, uint32_t *blocks_per_row);

@@ -215,6 +215,17 @@ def test_check_land_rows_accepts_and_rejects():
     assert _abi.check_land_rows(rows, None, _abi.ELX_F16, _abi.ELX_F16) == 5
     assert _abi.check_land_rows(rows, np.array([0, 2, 3], dtype=np.uint32), _abi.ELX_F16, _abi.ELX_F16) == 5
     assert _abi.check_land_rows(rows, None, _abi.ELX_F32, _abi.ELX_F16) == 10
+    # a row with more tiles than a launch may have workgroups per row: the width is capped, the workgroups stride
+    long = rows.copy()
+    long['n_alloc'][0] = long['n_valid'][0] = (1 << 32) + 77
+    cap = _abi.host_lib().elx_land_max_blocks()
+    assert cap == 1 << 20 and _abi.check_land_rows(long, None, _abi.ELX_F16, _abi.ELX_F16) == cap
+    long['n_alloc'][0] = long['n_valid'][0] = cap * tile
+    assert _abi.check_land_rows(long, None, _abi.ELX_F16, _abi.ELX_F16) == cap
+    long['n_alloc'][0] = long['n_valid'][0] = cap * tile - 1
+    assert _abi.check_land_rows(long, None, _abi.ELX_F16, _abi.ELX_F16) == cap
+    long['n_alloc'][0] = long['n_valid'][0] = (cap - 1) * tile
+    assert _abi.check_land_rows(long, None, _abi.ELX_F16, _abi.ELX_F16) == cap - 1
 
     def expect(code, r=rows, offsets=None, sd=_abi.ELX_F16, dd=_abi.ELX_F16):
         with pytest.raises(_abi.ElxError) as e:

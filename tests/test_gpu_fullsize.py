@@ -303,3 +303,80 @@ def test_one_buffer_beyond_two_to_the_32_elements():
     for b, e in windows:
         assert torch.equal(low[b:e], p.data[b:e].to(torch.bfloat16)), (b, e)
     assert int(torch.count_nonzero(low[::4099])) == int(torch.count_nonzero(p.data[::4099].to(torch.bfloat16)))
+
+
+def test_one_table_row_beyond_two_to_the_32_elements():
+    """The table forms over ONE row of 2**32 + 2**20 + 77 elements, straight through the C ABI: the landing
+    launch (every element moved by workgroups that take several tiles each, the flags of the valid head
+    taken, a non-finite value behind the 2**32 boundary found, one in the padding ignored), the stats launch
+    over the same row, and the refresh launch (several pieces per workgroup)."""
+    from elixir_amd import _abi
+    from elixir_amd.chunk import DeviceTable
+    dev = torch.device('cuda', 0)
+    stream = torch.cuda.current_stream().cuda_stream
+    n = (1 << 32) + (1 << 20) + 77
+    n_valid = n - 1000
+    step = 1 << 28
+    gen = torch.Generator(device=dev).manual_seed(6)
+    src = torch.empty(n, dtype=torch.float16, device=dev)
+    src.normal_(0, 0.5, generator=gen)
+    dst = torch.empty(n, dtype=torch.float16, device=dev)
+    dst.fill_(7.0)
+    rows = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+    rows[0]['grad'], rows[0]['lowp_out'], rows[0]['n_alloc'], rows[0]['n_valid'] = src.data_ptr(), dst.data_ptr(), n, n_valid
+    table = DeviceTable(rows, dev)
+    bpr = _abi.check_land_rows(rows, None, O.F16, O.F16)
+    assert bpr == _abi.land_max_blocks() < -(-n // _abi.land_tile_elems(O.F16))    # more tiles than workgroups
+    ws = torch.empty(_abi.land_workspace_records(1, bpr, 1) * 16, dtype=torch.uint8, device=dev)
+    out = torch.zeros(16, dtype=torch.uint8, device=dev)
+
+    def land():
+        _abi.land_grads_mt(table.ptr, 1, O.F16, O.F16, 1.0, bpr, ws.data_ptr(), out.data_ptr(), True, stream)
+        return out.cpu().numpy().view(_abi.STATS_DTYPE)[0]
+
+    def same(a, b):
+        return all(torch.equal(a[i:i + step].view(torch.int16), b[i:i + step].view(torch.int16)) for i in range(0, n, step))
+
+    rec = land()
+    assert same(dst, src)
+    ref = sum(float(src[i:min(n_valid, i + step)].double().square().sum()) for i in range(0, n_valid, step))
+    # (against the exact sum both launches sit 5e-8 low, alike: the square of a 16-bit value m * 2**e has
+    # m * m mod 4 in {0, 1}, so the bits an fp32 partial sum rounds away are below one half more often than above)
+    assert rec['overflow'] == 0 and abs(float(rec['sumsq']) - ref) <= 1e-6 * ref
+
+    # the stats launch over the same row: the same flags, the same sum to the last few bits
+    stats_rows = rows.copy()
+    stats_rows[0]['grad'], stats_rows[0]['lowp_out'] = dst.data_ptr(), 0
+    stats_table = DeviceTable(stats_rows, dev)
+    partials = torch.empty(1024 * 16, dtype=torch.uint8, device=dev)
+    out2 = torch.zeros(16, dtype=torch.uint8, device=dev)
+
+    def stats():
+        _abi.grad_stats_mt(stats_table.ptr, 1, O.F16, 1024, partials.data_ptr(), out2.data_ptr(), False, stream)
+        return out2.cpu().numpy().view(_abi.STATS_DTYPE)[0]
+
+    rec2 = stats()
+    assert rec2['overflow'] == 0 and abs(float(rec2["sumsq"]) - float(rec["sumsq"])) <= 1e-9 * ref
+
+    src[n_valid + 5] = float('inf')                       # in the padding: moved, not counted
+    rec = land()
+    assert rec['overflow'] == 0 and same(dst, src) and stats()['overflow'] == 0
+    src[(1 << 32) + 999] = float('nan')                   # behind the boundary, inside the valid head
+    assert land()['overflow'] == 1 and stats()['overflow'] == 1
+    src[(1 << 32) + 999] = 0.0
+    src[n_valid - 1] = float('-inf')                      # the last valid element
+    assert land()['overflow'] == 1 and stats()['overflow'] == 1
+    del src, ws, partials
+
+    # the refresh launch over one row: fp32 master -> bf16, 4.2 M pieces over at most 2**20 workgroups
+    master = torch.empty(n, dtype=torch.float32, device=dev)
+    master.normal_(0, 0.02, generator=gen)
+    low = dst.view(torch.bfloat16)
+    low.fill_(7.0)
+    wb_rows = np.zeros(1, dtype=_abi.CHUNK_DTYPE)
+    wb_rows[0]['lowp_out'], wb_rows[0]['master'], wb_rows[0]['n_alloc'] = low.data_ptr(), master.data_ptr(), n
+    wb_table = DeviceTable(wb_rows, dev)
+    assert -(-n // _abi.refresh_piece_elems()) > 1 << 20
+    _abi.writeback_mt(wb_table.ptr, 1, O.BF16, n, True, stream)
+    for i in range(0, n, step):
+        assert torch.equal(low[i:i + step], master[i:i + step].to(torch.bfloat16)), i
