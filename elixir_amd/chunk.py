@@ -169,7 +169,7 @@ class StatsArena:
     optimizer step can fetch the flags of all chunks with one device-to-host copy.  Slots are handed
     out in consecutive runs (the chunks of one landing sit side by side) and go back to the arena
     when their chunk is given another slot or is garbage-collected."""
-    CAPACITY = 8192
+    CAPACITY = 65535    # the chunks one launch can take: a set never needs more slots than that (1 MiB per device)
     _arenas: Dict[torch.device, 'StatsArena'] = {}
 
     def __init__(self, device: torch.device):

@@ -878,12 +878,14 @@ def test_launch_plan_properties_random():
     check()
 
 
-def test_stats_arena_hands_out_runs_and_takes_them_back():
+def test_stats_arena_hands_out_runs_and_takes_them_back(monkeypatch):
     """Slots of the record arena: consecutive runs in list order, kept when a list lands again, given
     back when a chunk moves to another run or is garbage-collected, and a clear error when no run is
     free.  (The arena's buffer sits on the CPU here; nothing is launched.)"""
     import gc
     from elixir_amd.chunk import StatsArena
+    assert StatsArena.CAPACITY == 65535                      # as many chunks as one launch takes rows
+    monkeypatch.setattr(StatsArena, 'CAPACITY', 4096)        # a small one, so that the churn below outnumbers it
 
     def chunk():
         c = ea.Chunk(None, 64, torch.float16, None, shard_device='cpu', temp_device='cpu')
