@@ -73,6 +73,65 @@ def test_fp32_training_matches_torch_adamw():
             torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'step {step} {name}')
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+def test_frozen_parameters_stay_out_of_the_chunks(dtype):
+    """Parameters that need no gradient (module.py:83-90, optimizer.py:248-249): they are moved to the
+    training dtype and the GPU and otherwise left alone -- no chunk holds them, the optimizer has no
+    range for them, ``state_dict`` hands them out and ``load_state_dict`` takes them back -- while the
+    rest trains as torch's AdamW trains it with the same parameters frozen."""
+    torch.manual_seed(0)
+    ref = Net().to(DEV)
+    for p in (ref.norm1.weight, ref.norm1.bias, ref.fc2.bias):
+        p.requires_grad_(False)
+    model = copy.deepcopy(ref)
+    frozen = {'norm1.weight', 'norm1.bias', 'fc2.bias'}
+    trainable = [(n, p) for n, p in model.named_parameters() if p.requires_grad]
+    assert {n for n, p in model.named_parameters() if not p.requires_grad} == frozen
+    ropt = torch.optim.AdamW([dict(params=[p for p in ref.parameters() if p.requires_grad and p.dim() > 1], weight_decay=0.1),
+                              dict(params=[p for p in ref.parameters() if p.requires_grad and p.dim() == 1], weight_decay=0.0)],
+                             lr=1e-2)
+    module = ea.ElixirModule(model, ea.greedy_search([(n, p.numel()) for n, p in trainable], 4096, dtype), dtype=dtype)
+    # the groups name every parameter, frozen ones too: the wrapper drops those (optimizer.py:248-249)
+    inner = ea.HybridAdam(groups_of(model, 0.1), lr=1e-2, weight_decay=0.1)
+    opt = ea.ElixirOptimizer(module, inner, initial_scale=64.0)
+    assert set(module.no_grad_state_dict) == frozen and not frozen & set(module.grad_state_dict)
+    assert sum(len(g['params']) for g in opt.param_groups) == len(trainable)
+    for name in frozen:
+        t = module.no_grad_state_dict[name]
+        assert t.dtype == dtype and t.is_cuda and not t.requires_grad
+    chunked = {t for c in module.param_chunks for t in c.tensors_info}
+    assert not any(module.no_grad_state_dict[n] in chunked for n in frozen)
+    before = {n: module.no_grad_state_dict[n].clone() for n in frozen}
+    initial = {n: t.detach().float().cpu().clone() for n, t in ref.state_dict().items()}
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    for step in range(3):
+        x = batch(gen)
+        ropt.zero_grad()
+        ref(x).backward()
+        ropt.step()
+        opt.zero_grad()
+        opt.backward(module(x))
+        opt.step()
+        assert opt.last_step_info['found_inf'] is False
+    module.materialize_params()
+    sd = module.state_dict()
+    for name, want in ref.state_dict().items():
+        if name in frozen:
+            assert torch.equal(sd[name], before[name]) and sd[name].dtype == dtype
+            assert torch.equal(sd[name].float().cpu(), want.to(dtype).float().cpu())
+        elif dtype == torch.float32:
+            torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=f'{name}')
+        else:
+            # (fp16 gradients are other gradients: after three steps of Adam only the size of the move is comparable)
+            moved = (sd[name].float() - initial[name]).abs().max().item()
+            assert 0 < moved <= 3 * 1e-2 * 1.2 and torch.isfinite(sd[name]).all(), (name, moved)
+    # loading a state dict writes the frozen ones where they live
+    new = {n: (t.float() + 1.0) for n, t in sd.items()}
+    module.load_state_dict(new)
+    for name in frozen:
+        assert torch.equal(module.no_grad_state_dict[name].float().cpu(), (before[name].float() + 1.0).to(dtype).float().cpu())
+
+
 @pytest.mark.parametrize('make', [lambda ps: torch.optim.SGD(ps, lr=5e-2, momentum=0.9, nesterov=True),
                                   lambda ps: torch.optim.RMSprop(ps, lr=1e-3)], ids=['sgd', 'rmsprop'])
 def test_inner_optimizer_outside_the_fused_list_runs_unfused(make):
