@@ -380,3 +380,51 @@ def test_one_table_row_beyond_two_to_the_32_elements():
     _abi.writeback_mt(wb_table.ptr, 1, O.BF16, n, True, stream)
     for i in range(0, n, step):
         assert torch.equal(low[i:i + step], master[i:i + step].to(torch.bfloat16)), i
+
+
+def test_one_chunk_beyond_two_to_the_32_elements_through_the_optimizer(oracle):
+    """A chunk of 2**32 + 2**25 elements in which one tensor crosses element 2**32, through ElixirOptimizer
+    (clipped AdamW, fp16 x 2**16): stepped once with its own stats pass and once behind a fused landing;
+    windows at the segment boundaries, across elements 2**31 and 2**32 and at the ragged end are replayed by
+    the oracle, the norm is held against torch's, the whole low-precision shard equals the cast of the
+    master shard, and an inf planted behind element 2**32 skips the step."""
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    shapes = [('a.weight', (3000, 4096)), ('big.weight', ((1 << 32) + 4096, )), ('b.bias', (2 << 19, )), ('c.weight', (77, 8))]
+    built = workloads.build('c5', shapes=shapes, chunk_size=(1 << 32) + (1 << 25), seed=9)
+    opt, module, dtype = built.optimizer, built.module, built.spec.dtype
+    assert len(module.param_chunks) == 1 and built.n_valid == sum(int(np.prod(s)) for _, s in shapes) > 1 << 32
+    pc = module.param_chunks[0]
+    oc = pc.paired_chunk
+    m, v = opt._binding.moments(oc)
+    rng = np.random.default_rng(1)
+    piece = 1 << 28
+    for fused in (False, True):
+        built.land_gradients(fused=fused)
+        wins = _slices(pc, opt, rng) + [((1 << 32) - 2048, (1 << 32) + 2048), ((1 << 31) - 100, (1 << 31) + 100)]
+        pre = {b: (to_np(pc.shard[b:e]), to_np(oc.shard[b:e]), to_np(m[b:e]), to_np(v[b:e])) for b, e in wins}
+        norm_sq = sum(float(pc.shard[i:min(pc.n_valid, i + piece)].float().norm(2).item())**2 for i in range(0, pc.n_valid, piece))
+        opt.step()
+        info = opt.last_step_info
+        assert info['found_inf'] is False and math.isclose(info['total_norm'], math.sqrt(norm_sq), rel_tol=1e-6)
+        assert info['combined_scale'] == O.combined_scale(built.spec.loss_scale, info['total_norm'], built.spec.max_norm)
+        for b, e in wins:
+            wp, wm, wv, wl = _oracle_on_slice(pc, opt, b, e, pre[b], info['combined_scale'], dtype)
+            assert np.array_equal(to_np(oc.shard[b:e]).view(np.uint32), wp.view(np.uint32)), (fused, b, e)
+            assert np.array_equal(to_np(m[b:e]).view(np.uint32), wm.view(np.uint32)), (fused, b, e)
+            assert np.array_equal(to_np(v[b:e]).view(np.uint32), wv.view(np.uint32)), (fused, b, e)
+            assert ulp_distance(to_np(pc.shard[b:e]), wl) == 0, (fused, b, e)
+        for i in range(0, pc.shard_size, piece):
+            assert torch.equal(pc.shard[i:i + piece], oc.shard[i:i + piece].to(dtype)), (fused, i)
+    keep = (oc.shard[(1 << 32):(1 << 32) + 65536].clone(), m[(1 << 32):(1 << 32) + 65536].clone())
+    built.land_gradients(fused=True)
+    pc.shard[(1 << 32) + 5000] = float('inf')
+    pc.invalidate_stats()
+    opt.mark_gradients_scaled()
+    scale = opt.loss_scale
+    opt.step()
+    assert opt.last_step_info['found_inf'] is True and opt.loss_scale == scale * 0.5
+    assert torch.equal(keep[0], oc.shard[(1 << 32):(1 << 32) + 65536]) and torch.equal(keep[1], m[(1 << 32):(1 << 32) + 65536])
+    for i in range(0, pc.shard_size, piece):
+        assert torch.equal(pc.shard[i:i + piece], oc.shard[i:i + piece].to(dtype)), i
