@@ -43,11 +43,12 @@ def to_divide(a: int, b: int) -> int:
 
 def greedy_groups(sizes: Sequence[int], chunk_size: int) -> List[List[int]]:
     """The packing rule of mini_waste.py:78-96: walk the tensors in order and open a new chunk
-    whenever the room left in the current one is smaller than the next tensor."""
+    whenever the room left in the current one is smaller than the next tensor.  (A tensor without elements
+    at the head of the list opens the first chunk here; the reference files it under its last one.)"""
     groups: List[List[int]] = []
     last_left = 0
     for i, p_size in enumerate(sizes):
-        if last_left < p_size:
+        if last_left < p_size or not groups:
             last_left = chunk_size
             groups.append([])
         assert last_left >= p_size, f'tensor {i} with {p_size} elements does not fit a chunk of {chunk_size}'

@@ -132,6 +132,50 @@ def test_frozen_parameters_stay_out_of_the_chunks(dtype):
         assert torch.equal(module.no_grad_state_dict[name].float().cpu(), (before[name].float() + 1.0).to(dtype).float().cpu())
 
 
+class NetWithEmptyParameters(nn.Module):
+    """Two parameters without elements, one of them first in the module's own order."""
+
+    def __init__(self, width=24, hidden=32):
+        super().__init__()
+        self.nothing = nn.Parameter(torch.zeros(0))
+        self.inp = nn.Linear(width, hidden)
+        self.norm = nn.LayerNorm(hidden)
+        self.none_either = nn.Parameter(torch.zeros(0, 3))
+        self.head = nn.Linear(hidden, 50, bias=False)
+
+    def forward(self, x):
+        h = self.norm(torch.tanh(self.inp(x.to(self.inp.weight.dtype))))
+        return self.head(h).float().logsumexp(-1).mean() + self.nothing.sum() + self.none_either.sum()
+
+
+def test_parameters_without_elements_are_carried_along():
+    """A parameter of zero elements sits in a chunk with an empty range (chunk.py:223-247), gets no fake
+    parameter (optimizer.py:251-253: ``begin >= end``), lands nothing and comes back from ``state_dict``;
+    the rest trains as under torch's AdamW."""
+    torch.manual_seed(0)
+    ref = NetWithEmptyParameters().to(DEV)
+    model = copy.deepcopy(ref)
+    named = [(n, p.numel()) for n, p in model.named_parameters()]
+    assert named[0] == ('nothing', 0) and ('none_either', 0) in named
+    ropt = torch.optim.AdamW(groups_of(ref, 0.1), lr=1e-2, weight_decay=0.1)
+    module, opt = wrap(model, torch.float32)
+    assert sum(len(g['params']) for g in opt.param_groups) == len(named) - 2
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    for step in range(3):
+        x = batch(gen)
+        ropt.zero_grad()
+        ref(x).backward()
+        ropt.step()
+        opt.zero_grad()
+        opt.backward(module(x))
+        opt.step()
+    module.materialize_params()
+    sd = module.state_dict()
+    for name, want in ref.state_dict().items():
+        assert sd[name].shape == want.shape
+        torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=name)
+
+
 @pytest.mark.parametrize('make', [lambda ps: torch.optim.SGD(ps, lr=5e-2, momentum=0.9, nesterov=True),
                                   lambda ps: torch.optim.RMSprop(ps, lr=1e-3)], ids=['sgd', 'rmsprop'])
 def test_inner_optimizer_outside_the_fused_list_runs_unfused(make):

@@ -396,6 +396,17 @@ def test_launch_plan_chooses_the_cache_policy_of_the_update_launch_by_size():
     assert info.with_cache_policy(2).flags == state_flags and info.with_cache_policy(2)[:3] == tuple(info)
 
 
+def test_greedy_packing_carries_tensors_without_elements():
+    """mini_waste.py:78-96 with sizes of zero in the list: such a tensor never opens a chunk of its own
+    behind the first and never overflows one; at the head of the list it opens the first chunk."""
+    from elixir_amd.module import greedy_groups
+    assert greedy_groups([0, 5, 0, 60, 10, 0], 64) == [[0, 1, 2], [3], [4, 5]]
+    assert greedy_groups([64, 0, 0, 1], 64) == [[0, 1, 2], [3]]
+    assert greedy_groups([0], 64) == [[0]] and greedy_groups([], 64) == []
+    with pytest.raises(AssertionError, match='does not fit'):
+        greedy_groups([65], 64)
+
+
 def test_launch_plan_keeps_rows_bounded_for_the_large_workloads():
     from elixir_amd.launch_plan import FlatBuffer, build_plan
     from elixir_amd.module import greedy_groups
