@@ -192,8 +192,11 @@ class ElixirModule(nn.Module):
         # copies, as the blocks of the replicated cache are in the reference) have not seen yet
         self._params_stale = False
         if not self.synthetic:
+            hooked = set()
             for param in self.grad_state_dict.values():
-                param.register_post_accumulate_grad_hook(self._gradient_handler)
+                if param not in hooked:    # a tied weight is listed under each of its names: one hook all the same
+                    hooked.add(param)
+                    param.register_post_accumulate_grad_hook(self._gradient_handler)
 
     def __init_chunk_group(self, sr: SearchResult, module):
         device = gpu_device() if torch.cuda.is_available() else torch.device('cpu')

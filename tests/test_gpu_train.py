@@ -132,6 +132,58 @@ def test_frozen_parameters_stay_out_of_the_chunks(dtype):
         assert torch.equal(module.no_grad_state_dict[name].float().cpu(), (before[name].float() + 1.0).to(dtype).float().cpu())
 
 
+class TiedNet(nn.Module):
+    """The output projection shares its weight with the embedding, as GPT-2's does."""
+
+    def __init__(self, vocab=50, hidden=32):
+        super().__init__()
+        self.emb = nn.Embedding(vocab, hidden)
+        self.fc = nn.Linear(hidden, hidden)
+        self.head = nn.Linear(hidden, vocab, bias=False)
+        self.head.weight = self.emb.weight
+
+    def forward(self, idx):
+        return self.head(torch.tanh(self.fc(self.emb(idx)))).float().logsumexp(-1).mean()
+
+
+@pytest.mark.parametrize('chunk_size', [1600, 4096])
+def test_a_tied_weight_lands_once_and_trains_like_torch(chunk_size):
+    """One parameter under two names (``emb.weight`` / ``head.weight``): it sits in one chunk once -- alone in
+    it with the smaller chunk size, as the reference's searches place a parameter that is used twice
+    (search/simple.py:33) --, its gradient (the sum over both uses) lands once from the hook of backward, and
+    ``state_dict`` hands the trained values out under both names."""
+    torch.manual_seed(0)
+    ref = TiedNet().to(DEV)
+    model = copy.deepcopy(ref)
+    assert model.head.weight is model.emb.weight
+    named = [(n, p.numel()) for n, p in model.named_parameters()]
+    assert [n for n, _ in named] == ['emb.weight', 'fc.weight', 'fc.bias']
+    ropt = torch.optim.AdamW(ref.parameters(), lr=1e-2, weight_decay=0.1)
+    module = ea.ElixirModule(model, ea.greedy_search(named, chunk_size, torch.float32), dtype=torch.float32)
+    opt = ea.ElixirOptimizer(module, ea.HybridAdam(model.parameters(), lr=1e-2, weight_decay=0.1))
+    assert [c.num_tensors for c in module.param_chunks] == ([1, 2] if chunk_size == 1600 else [3])
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    for step in range(3):
+        idx = torch.randint(0, 50, (8, 16), device=DEV, generator=gen)
+        ropt.zero_grad()
+        ref(idx).backward()
+        ropt.step()
+        opt.zero_grad()
+        opt.backward(module(idx))
+        opt.step()
+        assert opt.last_step_info['found_inf'] is False
+    module.materialize_params()
+    assert model.head.weight is model.emb.weight
+    sd = module.state_dict()
+    assert torch.equal(sd['head.weight'], sd['emb.weight'])
+    for name, want in ref.state_dict().items():
+        torch.testing.assert_close(sd[name], want.cpu(), rtol=2e-6, atol=2e-5, msg=name)
+    module.load_state_dict({n: t + 1.0 for n, t in sd.items()})
+    again = module.state_dict()
+    for name in sd:
+        assert torch.equal(again[name], sd[name] + 1.0), name
+
+
 class NetWithEmptyParameters(nn.Module):
     """Two parameters without elements, one of them first in the module's own order."""
 
