@@ -184,6 +184,62 @@ def test_a_tied_weight_lands_once_and_trains_like_torch(chunk_size):
         assert torch.equal(again[name], sd[name] + 1.0), name
 
 
+class NetWithBuffers(nn.Module):
+    """Batch normalisation brings buffers along: two floating-point ones and an integer count per layer (the
+    reference's own optimizer test trains a ResNet, test/wrapper/test_optimizer.py:55)."""
+
+    def __init__(self, width=24, hidden=32):
+        super().__init__()
+        self.inp = nn.Linear(width, hidden, bias=False)
+        self.bn1 = nn.BatchNorm1d(hidden)
+        self.fc = nn.Linear(hidden, hidden, bias=False)
+        self.bn2 = nn.BatchNorm1d(hidden)
+        self.head = nn.Linear(hidden, 10)
+
+    def forward(self, x):
+        h = torch.relu(self.bn1(self.inp(x.to(self.inp.weight.dtype))))
+        h = torch.relu(self.bn2(self.fc(h)))
+        return self.head(h).float().logsumexp(-1).mean()
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+def test_buffers_move_with_the_module_and_stay_out_of_the_chunks(dtype):
+    """module.py:91-95: floating-point buffers go to the training dtype and the GPU, integer ones keep their
+    type; no chunk holds them, ``state_dict`` hands them out as the wrapped module keeps them.  In fp32 the
+    whole state after three steps, running statistics included, is the one plain PyTorch training reaches."""
+    torch.manual_seed(0)
+    ref = NetWithBuffers().to(DEV)
+    model = copy.deepcopy(ref)
+    named = [(n, p.numel()) for n, p in model.named_parameters()]
+    buffers = {n for n, _ in model.named_buffers()}
+    assert len(buffers) == 6
+    ropt = torch.optim.AdamW(groups_of(ref, 0.1), lr=1e-2, weight_decay=0.1)
+    module, opt = wrap(model, dtype, chunk_size=1024, initial_scale=64.0)
+    for name, buf in model.named_buffers():
+        assert buf.is_cuda and buf.dtype == (torch.int64 if name.endswith('num_batches_tracked') else dtype), name
+    assert sum(c.num_tensors for c in module.param_chunks) == len(named)
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    for step in range(3):
+        x = torch.randn(64, 24, device=DEV, generator=gen)
+        ropt.zero_grad()
+        ref(x).backward()
+        ropt.step()
+        opt.zero_grad()
+        opt.backward(module(x))
+        opt.step()
+        assert opt.last_step_info['found_inf'] is False
+    module.materialize_params()
+    sd = module.state_dict()
+    assert set(sd) == set(ref.state_dict())
+    for name, want in ref.state_dict().items():
+        if name.endswith('num_batches_tracked'):
+            assert sd[name].dtype == torch.int64 and int(sd[name]) == 3
+        elif dtype == torch.float32:
+            torch.testing.assert_close(sd[name].cpu(), want.cpu(), rtol=2e-6, atol=2e-5, msg=name)
+        else:
+            assert sd[name].dtype == (dtype if name in buffers else torch.float32) and torch.isfinite(sd[name].float()).all()
+
+
 class NetWithEmptyParameters(nn.Module):
     """Two parameters without elements, one of them first in the module's own order."""
 
