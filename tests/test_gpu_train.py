@@ -184,6 +184,39 @@ def test_a_tied_weight_lands_once_and_trains_like_torch(chunk_size):
         assert torch.equal(again[name], sd[name] + 1.0), name
 
 
+def test_two_wrapped_models_in_one_process_do_not_disturb_each_other():
+    """Two modules with an optimizer each (fp16 with a dynamic loss scale, bf16 with a constant one, other
+    chunk sizes, both clipped) share one GPU: its record arena, the library's tables and streams.  Stepped in
+    turns they end with the bits they end with when one trains after the other."""
+
+    def run(in_turns):
+        torch.manual_seed(0)
+        a, b = Net().to(DEV), Net(hidden=48).to(DEV)
+        ma, oa = wrap(a, torch.float16, chunk_size=4096, initial_scale=64.0, max_norm=1.0)
+        mb, ob = wrap(b, torch.bfloat16, chunk_size=16384, max_norm=0.5)
+        ga, gb = torch.Generator(device=DEV).manual_seed(1), torch.Generator(device=DEV).manual_seed(2)
+
+        def step(m, o, g):
+            o.zero_grad()
+            o.backward(m(batch(g)))
+            o.step()
+
+        if in_turns:
+            for _ in range(4):
+                step(ma, oa, ga)
+                step(mb, ob, gb)
+        else:
+            for _ in range(4):
+                step(ma, oa, ga)
+            for _ in range(4):
+                step(mb, ob, gb)
+        return [c.paired_chunk.shard.clone() for m in (ma, mb) for c in m.param_chunks] + \
+               [t.clone() for o in (oa, ob) for c in o._binding.chunks for t in o._binding.moments(c)]
+
+    for u, v in zip(run(True), run(False)):
+        assert torch.equal(u, v)
+
+
 class NetWithBuffers(nn.Module):
     """Batch normalisation brings buffers along: two floating-point ones and an integer count per layer (the
     reference's own optimizer test trains a ResNet, test/wrapper/test_optimizer.py:55)."""
